@@ -1,0 +1,169 @@
+/*
+ * wol_c_api.h -- C ABI of the MI355X (gfx950) weight-only quantized linear
+ * library (libwol_gfx950.so).
+ *
+ * These entry points are what Paddle's three PHI GPU kernels for this path
+ * call once their bodies are replaced:
+ *
+ *   wol_quantize    <- phi::WeightQuantizeKernel<T, GPUContext>
+ *                      paddle/phi/kernels/weight_quantize_kernel.h:21-28,
+ *                      paddle/phi/kernels/gpu/weight_quantize_kernel.cu:25-115
+ *                      (arithmetic: the CPU kernel's,
+ *                      paddle/phi/kernels/impl/weight_quantize_kernel_impl.h:45-183)
+ *   wol_dequantize  <- phi::WeightDequantizeKernel<T, GPUContext>
+ *                      paddle/phi/kernels/weight_dequantize_kernel.h:21-28,
+ *                      paddle/phi/kernels/gpu/weight_dequantize_kernel.cu:440-475
+ *   wol_linear      <- phi::WeightOnlyLinearKernel<T, GPUContext>
+ *                      paddle/phi/kernels/weight_only_linear_kernel.h:21-30,
+ *                      paddle/phi/kernels/gpu/weight_only_linear_kernel.cu:26-201
+ *
+ * Conventions
+ *   - Plain pointers and sizes only.  Every pointer is DEVICE memory owned by
+ *     the caller; the library never allocates, frees or synchronises.  All
+ *     work is enqueued on `stream` (a hipStream_t passed as void*; NULL is the
+ *     null stream), the way the reference enqueues on dev_ctx.stream().
+ *   - K = in_features, N = out_features, M = tokens (x.numel() / K).
+ *   - dtype is the activation / scale / bias / output type T.
+ *   - Every function returns a wol_status; 0 is success.  Nothing throws.
+ *     Argument errors mirror the reference's InferMeta checks
+ *     (paddle/phi/infermeta/unary.cc:5946-6011, binary.cc:4499-4570,
+ *     multiary.cc:5495-5575); the PHI glue turns a non-zero status into
+ *     PADDLE_THROW(InvalidArgument / External).
+ *   - Thread-safe and re-entrant: no mutable global state.
+ */
+#ifndef WOL_C_API_H_
+#define WOL_C_API_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* T: the two types the reference registers (gpu/weight_quantize_kernel.cu:118-123). */
+#define WOL_DTYPE_F16 0
+#define WOL_DTYPE_BF16 1
+
+/* float -> T flavour used for the SCALE (the codes are computed against the
+ * rounded scale, impl/weight_quantize_kernel_impl.h:55,92-94).
+ * RNE   : bf16 of CPU/CUDA builds (paddle/phi/common/bfloat16.h:61-88), fp16 of
+ *         F16C and device builds (paddle/phi/common/float16.h:107-119).
+ * TRUNC : bf16 of HIP builds (bfloat16.h:103-110), fp16 of a host build
+ *         without F16C (float16.h:121-139). */
+#define WOL_ROUND_RNE 0
+#define WOL_ROUND_TRUNC 1
+
+/* Weight tensor layouts.  All hold the same K*N*bits/8 bytes.
+ * CANONICAL  : the reference's codes before any layout step: [K,N] int8, or
+ *              [K,N/2] bytes with column 2j in the low nibble (two's
+ *              complement nibbles) -- the x_int buffer of
+ *              paddle/phi/kernels/cpu/weight_quantize_kernel.cc:95-107.
+ * PADDLE_HIP : what a PADDLE_WITH_HIP build returns (:113-125): CANONICAL
+ *              transposed bytewise to [N,K] / [N/2,K], int4 nibbles stored +8.
+ * GFX950     : this library's streaming layout (see wol_layout_version). */
+#define WOL_LAYOUT_CANONICAL 0
+#define WOL_LAYOUT_PADDLE_HIP 1
+#define WOL_LAYOUT_GFX950 2
+
+typedef enum wol_status {
+  WOL_OK = 0,
+  WOL_ERR_NULL_POINTER = 1,   /* a required pointer is NULL                     */
+  WOL_ERR_BAD_DTYPE = 2,      /* dtype not F16/BF16                             */
+  WOL_ERR_BAD_BITS = 3,       /* bits not 8/4 (weight_dtype not int8/int4)      */
+  WOL_ERR_BAD_GROUP_SIZE = 4, /* group_size not -1/64/128                       */
+  WOL_ERR_BAD_SHAPE = 5,      /* K % 64, N % 16, M < 0 ... (InferMeta contract) */
+  WOL_ERR_BAD_LAYOUT = 6,     /* unknown layout id                              */
+  WOL_ERR_BAD_ROUND_MODE = 7,
+  WOL_ERR_WORKSPACE = 8,      /* workspace NULL or smaller than the query says  */
+  WOL_ERR_ALIGNMENT = 9,      /* a pointer is not 16-byte aligned               */
+  WOL_ERR_HIP = 10,           /* a HIP launch failed; see hipGetLastError       */
+  WOL_ERR_NO_DEVICE = 11      /* no gfx950 device / code object not loadable    */
+} wol_status;
+
+/* Human-readable text for a status (static storage). */
+const char* wol_status_str(int status);
+
+/* Version tag of the GFX950 layout.  A checkpoint that stores packed weights
+ * should store this beside them; a different value means "repack". */
+int wol_layout_version(void);
+
+/* Bytes of device scratch wol_quantize needs (per-channel abs-max uses an
+ * fp32 [N] buffer; group-wise needs none).  Returns 0 for invalid arguments. */
+size_t wol_quantize_workspace(int64_t K, int64_t N, int bits, int group_size);
+
+/*
+ * weight_quantize.  w: [K,N] T row-major.  Computes, bit-exactly as the
+ * reference's CPU kernel does,
+ *     scale[gk,n] = cast_T( max_k |w[k,n]| / bound ),  bound = 127 | 7
+ *     code[k,n]   = clip( round_half_away( float(w) / float(scale) ) )
+ * and writes the codes in `layout` (GFX950 for wol_linear) into codes_out
+ * (K*N*bits/8 bytes; reported to Paddle as [N,K] int8 or [N/2,K] int8,
+ * paddle/phi/infermeta/unary.cc:5994-6005) and scale_out ([N] or
+ * [ceil(K/g),N] T, :5985-5992).
+ * Requires K % 64 == 0, N % 16 == 0, group_size in {-1,64,128}.
+ */
+int wol_quantize(const void* w, int dtype, int64_t K, int64_t N, int bits,
+                 int group_size, int round_mode, int layout, void* codes_out,
+                 void* scale_out, void* workspace, size_t workspace_bytes,
+                 void* stream);
+
+/*
+ * weight_dequantize.  out_KN[k,n] = cast_T( float(code[k,n]) * float(scale) ),
+ * written directly as [K,N] row-major T (the reference writes [N,K] and then
+ * transposes, gpu/weight_dequantize_kernel.cu:464-470).  `layout` names the
+ * layout of `codes`.  The final cast is round-to-nearest-even.
+ */
+int wol_dequantize(const void* codes, int layout, const void* scale, int dtype,
+                   int64_t K, int64_t N, int bits, int group_size,
+                   void* out_KN, void* stream);
+
+/* Bytes of device scratch wol_linear needs for this problem (may be 0). */
+size_t wol_linear_workspace(int64_t M, int64_t K, int64_t N, int bits,
+                            int group_size);
+
+/*
+ * weight_only_linear.  out[M,N] = x[M,K] . dequant(W)[K,N] (+ bias[N]),
+ * fp32 accumulation, one round-to-nearest-even cast to T at the end.
+ * codes must be in GFX950 layout.  bias may be NULL.
+ * scale: [N] T (group_size -1) or [ceil(K/g),N] T, as wol_quantize wrote it.
+ * M <= 64 takes the streaming (HBM-bound) kernel, larger M the MFMA GEMM; the
+ * reference's split is M <= 3 (gpu/weight_only_linear_kernel.cu:60-61).
+ */
+int wol_linear(const void* x, const void* codes, const void* bias,
+               const void* scale, int dtype, int64_t M, int64_t K, int64_t N,
+               int bits, int group_size, void* out, void* workspace,
+               size_t workspace_bytes, void* stream);
+
+/* Same as wol_linear but writes the fp32 accumulators (plus bias) instead of
+ * casting to T: out_f32 is [M,N] float.  Used to check the arithmetic without
+ * the final rounding. */
+int wol_linear_f32(const void* x, const void* codes, const void* bias,
+                   const void* scale, int dtype, int64_t M, int64_t K,
+                   int64_t N, int bits, int group_size, float* out_f32,
+                   void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Re-lays a code tensor between layouts (any pair of the three).  It is a
+ * pure, invertible permutation (plus the documented nibble/byte bias of the
+ * target layout), which is what makes the packed weights checkpointable and
+ * comparable with the reference's codes.
+ */
+int wol_repack(const void* codes_in, int layout_in, void* codes_out,
+               int layout_out, int64_t K, int64_t N, int bits, void* stream);
+
+/*
+ * Host-side index helper (no device work): byte offset of element (k, n) in a
+ * code tensor of the given layout, and through *nibble_shift which nibble of
+ * that byte holds it (0 or 4; always 0 for int8).  Returns -1 for arguments
+ * outside the contract.  For tools that read or write packed checkpoints; it
+ * has no counterpart in the reference, whose layouts are implicit in its
+ * kernels (paddle/phi/kernels/impl/weight_quantize_kernel_impl.h:185-441).
+ */
+int64_t wol_code_offset(int layout, int64_t K, int64_t N, int bits, int64_t k,
+                        int64_t n, int* nibble_shift);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* WOL_C_API_H_ */

@@ -1,0 +1,357 @@
+/*
+ * wo_oracle.c -- CPU restatement of Paddle's weight-only quantisation path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  Nothing that ships (the HIP library, the host
+ * layer, the Python mirror of paddle.nn.quant) may link, load or call this
+ * file.  It exists so that the GPU kernels can be compared with an
+ * independent, single-threaded statement of the reference arithmetic, and so
+ * that the benchmark can time a CPU baseline beside the GPU numbers.
+ *
+ * Each function cites the reference source it follows (paths relative to the
+ * Paddle tree).  How each function is pinned:
+ *   casts         : checked against the reference's own float16.h / bfloat16.h
+ *                   compiled as oracle/_ref (exhaustive over the fp16 range,
+ *                   dense sample for bf16) and against committed vectors made
+ *                   from that build.
+ *   scales, codes : closed form max|w|/bound -> cast -> round-half-away ->
+ *                   clip; pinned by an independent numpy brute force, by
+ *                   invariants (|q| <= bound, non-degenerate groups reach
+ *                   |q| == bound, |w - q*s| <= s/2 unless clipped) and by the
+ *                   known answers recorded from a run of the reference header
+ *                   (all-zero column: scale bits 0x0000, int8 code 127, int4
+ *                   nibble 0x9).
+ *   dequant/linear: products of <=8-bit codes with <=11-bit scales are exact
+ *                   in fp32, so dequant has one correct answer; the linear is
+ *                   checked against a float64 matmul of the same operands.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define WO_F16 0
+#define WO_BF16 1
+
+/* cast flavours (which build of the reference the scale cast imitates) */
+#define WO_CAST_RNE 0   /* bf16: CPU/CUDA build; fp16: F16C or device build */
+#define WO_CAST_TRUNC 1 /* bf16: HIP build (>>16); fp16: stock host build    */
+
+static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+/* ---- bfloat16 ---------------------------------------------------------- */
+
+/* paddle/phi/common/bfloat16.h:61-88 (cpu_float_to_bfloat16): zero keeps only
+ * the sign, inf passes through, NaN becomes 0x7FFF, everything else (normal
+ * and subnormal) is round-to-nearest-even on the raw bits. */
+uint16_t wo_f32_to_bf16_rne(float f) {
+  uint32_t u = f2u(f);
+  uint32_t mag = u & 0x7FFFFFFFu;
+  if (mag == 0) return (uint16_t)((u >> 16) & 0x8000u);
+  if (mag == 0x7F800000u) return (uint16_t)(u >> 16);
+  if (mag > 0x7F800000u) return 0x7FFFu;
+  uint32_t lsb = (u >> 16) & 1u;
+  return (uint16_t)((u + 0x7FFFu + lsb) >> 16);
+}
+
+/* paddle/phi/common/bfloat16.h:103-110 (PADDLE_WITH_HIP): drop the low half. */
+uint16_t wo_f32_to_bf16_trunc(float f) { return (uint16_t)(f2u(f) >> 16); }
+
+/* paddle/phi/common/bfloat16.h:190-213: the bf16 bits are the high half. */
+float wo_bf16_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
+
+/* ---- float16 ----------------------------------------------------------- */
+
+/* paddle/phi/common/float16.h:118-119 (_cvtss_sh(val, 0)) and the device
+ * __float2half: IEEE round-to-nearest-even with gradual underflow. */
+uint16_t wo_f32_to_f16_rne(float f) {
+  uint32_t u = f2u(f);
+  uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+  uint32_t mag = u & 0x7FFFFFFFu;
+  if (mag > 0x7F800000u) /* NaN: quiet it, keep the top payload bits */
+    return (uint16_t)(sign | 0x7E00u | ((mag >> 13) & 0x03FFu));
+  if (mag >= 0x47800000u) return (uint16_t)(sign | 0x7C00u); /* >= 65536, inf */
+  int32_t e = (int32_t)(mag >> 23) - 127;
+  if (e >= -14) { /* normal half, may round up into the next binade or to inf */
+    uint32_t m = mag & 0x007FFFFFu;
+    uint32_t h = ((uint32_t)(e + 15) << 10) | (m >> 13);
+    uint32_t rem = m & 0x1FFFu;
+    if (rem > 0x1000u || (rem == 0x1000u && (h & 1u))) h++;
+    return (uint16_t)(sign | h);
+  }
+  if (e < -25) return sign; /* below half of the smallest subnormal */
+  /* subnormal half: value = m24 * 2^(e-23), target unit 2^-24 */
+  uint32_t m24 = (mag & 0x007FFFFFu) | 0x00800000u;
+  int shift = -e - 1; /* 14..24 */
+  uint32_t h = m24 >> shift;
+  uint32_t rem = m24 & ((1u << shift) - 1u);
+  uint32_t half = 1u << (shift - 1);
+  if (rem > half || (rem == half && (h & 1u))) h++;
+  return (uint16_t)(sign | h);
+}
+
+/* paddle/phi/common/float16.h:121-139, the software routine a host build
+ * without F16C falls into.  What it computes, case by case on |val|:
+ *   below 2^-14   : floor(|val| * 2^24) (subnormal, magnitude truncated)
+ *   up to 65504   : exponent rebias, mantissa truncated to 10 bits
+ *   above 65504   : infinity (even where nearest-even would give 65504)
+ *   NaN           : payload >> 13, but payloads that would shift to zero
+ *                   become the smallest half NaN (0x7C01)
+ */
+uint16_t wo_f32_to_f16_trunc(float f) {
+  uint32_t u = f2u(f);
+  uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+  uint32_t mag = u & 0x7FFFFFFFu;
+  if (mag > 0x7F800000u) {
+    if (mag < 0x7F802000u) return (uint16_t)(sign | 0x7C01u);
+    return (uint16_t)(sign | 0x7C00u | ((mag >> 13) & 0x03FFu));
+  }
+  if (mag > 0x477FE000u) return (uint16_t)(sign | 0x7C00u);
+  if (mag < 0x38800000u) {
+    /* |val| * 2^37 truncated to an integer, then the common >> 13 */
+    float scaled = u2f(mag) * u2f(0x52000000u);
+    uint32_t q = (uint32_t)(int32_t)scaled;
+    return (uint16_t)(sign | (q >> 13));
+  }
+  return (uint16_t)(sign | ((mag >> 13) - 0x1C000u));
+}
+
+/* paddle/phi/common/float16.h:315-345 (operator float): exact widening. */
+float wo_f16_to_f32(uint16_t h) {
+  uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+  uint32_t e = (h >> 10) & 0x1Fu;
+  uint32_t m = h & 0x03FFu;
+  if (e == 0) {
+    if (m == 0) return u2f(sign);
+    float v = (float)m * u2f(0x33800000u); /* m * 2^-24, exact */
+    return u2f(f2u(v) | sign);
+  }
+  if (e == 31) return u2f(sign | 0x7F800000u | (m << 13));
+  return u2f(sign | ((e + 112u) << 23) | (m << 13));
+}
+
+float wo_to_f32(uint16_t h, int dtype) {
+  return dtype == WO_BF16 ? wo_bf16_to_f32(h) : wo_f16_to_f32(h);
+}
+
+uint16_t wo_from_f32(float f, int dtype, int cast_mode) {
+  if (dtype == WO_BF16)
+    return cast_mode == WO_CAST_TRUNC ? wo_f32_to_bf16_trunc(f)
+                                      : wo_f32_to_bf16_rne(f);
+  return cast_mode == WO_CAST_TRUNC ? wo_f32_to_f16_trunc(f)
+                                    : wo_f32_to_f16_rne(f);
+}
+
+void wo_cast_array_from_f32(const float* in, int64_t n, int dtype,
+                            int cast_mode, uint16_t* out) {
+  for (int64_t i = 0; i < n; ++i) out[i] = wo_from_f32(in[i], dtype, cast_mode);
+}
+
+void wo_cast_array_to_f32(const uint16_t* in, int64_t n, int dtype, float* out) {
+  for (int64_t i = 0; i < n; ++i) out[i] = wo_to_f32(in[i], dtype);
+}
+
+/* |x| as the reference's xabs<T> takes it (impl/weight_quantize_kernel_impl.h:
+ * 40-43): negate when x < 0, so -0 and NaN pass through unchanged. */
+static inline float abs_like_ref(float v) { return v < 0.0f ? -v : v; }
+
+/* ---- scales ------------------------------------------------------------ */
+
+/* paddle/phi/kernels/impl/weight_quantize_kernel_impl.h:45-57
+ * (per_channel_scale).  w is [K,N] row-major in T; the running maximum starts
+ * from the signed first element of the column. */
+void wo_per_channel_scale(const uint16_t* w, int64_t K, int64_t N, int dtype,
+                          float bound, int cast_mode, uint16_t* scale) {
+  for (int64_t n = 0; n < N; ++n) {
+    float mx = wo_to_f32(w[n], dtype);
+    for (int64_t k = 0; k < K; ++k) {
+      float a = abs_like_ref(wo_to_f32(w[k * N + n], dtype));
+      mx = a > mx ? a : mx;
+    }
+    scale[n] = wo_from_f32(mx / bound, dtype, cast_mode);
+  }
+}
+
+/* paddle/phi/kernels/impl/weight_quantize_kernel_impl.h:59-78
+ * (group_wise_scale).  scale is [ceil(K/g), N]; the maximum starts at 0 and
+ * the last group may be short. */
+void wo_group_wise_scale(const uint16_t* w, int64_t K, int64_t N, int dtype,
+                         float bound, int64_t g, int cast_mode,
+                         uint16_t* scale) {
+  for (int64_t n = 0; n < N; ++n) {
+    for (int64_t k0 = 0; k0 < K; k0 += g) {
+      float mx = 0.0f;
+      for (int64_t k = k0; k < k0 + g && k < K; ++k) {
+        float a = abs_like_ref(wo_to_f32(w[k * N + n], dtype));
+        mx = a > mx ? a : mx;
+      }
+      scale[(k0 / g) * N + n] = wo_from_f32(mx / bound, dtype, cast_mode);
+    }
+  }
+}
+
+/* ---- codes ------------------------------------------------------------- */
+
+/* The int8 branch of per_channel_quant / group_wise_quant
+ * (impl/weight_quantize_kernel_impl.h:91-96, :143-149): C round() (halves
+ * away from zero), then std::min(127.f, r) and std::max(-127.f, .) spelled
+ * out so that a NaN quotient (0/0 in an all-zero column) lands on 127. */
+static inline int8_t quant_code_int8(float w, float s) {
+  float r = roundf(w / s);
+  float lo = (r < 127.0f) ? r : 127.0f;      /* std::min(127.f, r)  */
+  float cl = (-127.0f < lo) ? lo : -127.0f;  /* std::max(-127.f, lo) */
+  return (int8_t)cl;
+}
+
+/* The int4 branch (impl/weight_quantize_kernel_impl.h:104-114, :155-166):
+ * the rounded quotient is converted to int BEFORE clipping.  The conversion
+ * of NaN, infinities and out-of-range values is undefined in C++; the
+ * reference runs on x86, where it yields INT_MIN, so they clip to -7. */
+static inline int quant_code_int4(float w, float s) {
+  float r = roundf(w / s);
+  int v;
+  if (r >= -2147483648.0f && r < 2147483648.0f) v = (int)r;
+  else v = INT32_MIN;
+  int lo = v < 7 ? v : 7;
+  return lo > -7 ? lo : -7;
+}
+
+/* per_channel_quant<T,bits> and group_wise_quant<T,bits>
+ * (impl/weight_quantize_kernel_impl.h:80-183), group_size -1 meaning one
+ * scale per column.  Output is the canonical code tensor: [K,N] int8, or
+ * [K,N/2] bytes with column 2j in the low nibble and 2j+1 in the high one.
+ * nibble_bias is 0 for the CPU/CUDA flavour and 8 for the HIP flavour
+ * (:109-111). */
+void wo_quant_codes(const uint16_t* w, const uint16_t* scale, int64_t K,
+                    int64_t N, int dtype, int bits, int64_t group_size,
+                    int nibble_bias, int8_t* codes) {
+  for (int64_t k = 0; k < K; ++k) {
+    const uint16_t* wrow = w + k * N;
+    const uint16_t* srow =
+        group_size > 0 ? scale + (k / group_size) * N : scale;
+    if (bits == 8) {
+      int8_t* out = codes + k * N;
+      for (int64_t n = 0; n < N; ++n)
+        out[n] = quant_code_int8(wo_to_f32(wrow[n], dtype),
+                                 wo_to_f32(srow[n], dtype));
+    } else {
+      int8_t* out = codes + k * (N / 2);
+      for (int64_t j = 0; j < N / 2; ++j) {
+        int q0 = quant_code_int4(wo_to_f32(wrow[2 * j], dtype),
+                                 wo_to_f32(srow[2 * j], dtype)) + nibble_bias;
+        int q1 = quant_code_int4(wo_to_f32(wrow[2 * j + 1], dtype),
+                                 wo_to_f32(srow[2 * j + 1], dtype)) + nibble_bias;
+        out[j] = (int8_t)((q0 & 0x0F) | ((q1 & 0x0F) << 4));
+      }
+    }
+  }
+}
+
+/* Scale + codes in one call: the arithmetic half of quant_compute
+ * (paddle/phi/kernels/cpu/weight_quantize_kernel.cc:95-107), bound 127 or 7.
+ * Returns 0, or -1 on an argument the reference's InferMeta would reject
+ * (paddle/phi/infermeta/unary.cc:5961-5983). */
+int wo_weight_quantize(const uint16_t* w, int64_t K, int64_t N, int dtype,
+                       int bits, int64_t group_size, int cast_mode,
+                       int nibble_bias, int8_t* codes, uint16_t* scale) {
+  if (K % 64 != 0 || N % 16 != 0) return -1;
+  if (!(group_size == -1 || group_size == 64 || group_size == 128)) return -1;
+  if (bits != 8 && bits != 4) return -1;
+  float bound = bits == 8 ? 127.0f : 7.0f;
+  if (group_size == -1)
+    wo_per_channel_scale(w, K, N, dtype, bound, cast_mode, scale);
+  else
+    wo_group_wise_scale(w, K, N, dtype, bound, group_size, cast_mode, scale);
+  wo_quant_codes(w, scale, K, N, dtype, bits, group_size, nibble_bias, codes);
+  return 0;
+}
+
+/* The HIP-flavour layout step of quant_compute
+ * (cpu/weight_quantize_kernel.cc:113-125): a byte transpose of the canonical
+ * tensor, [K,N] -> [N,K] for int8 and [K,N/2] -> [N/2,K] for int4. */
+void wo_transpose_bytes(const int8_t* in, int64_t rows, int64_t cols,
+                        int8_t* out) {
+  for (int64_t r = 0; r < rows; ++r)
+    for (int64_t c = 0; c < cols; ++c) out[c * rows + r] = in[r * cols + c];
+}
+
+/* Signed code of element (k,n) of a canonical tensor. */
+static inline int code_at(const int8_t* codes, int64_t k, int64_t n, int64_t N,
+                          int bits, int nibble_bias) {
+  if (bits == 8) return codes[k * N + n];
+  uint8_t b = (uint8_t)codes[k * (N / 2) + n / 2];
+  int nib = (n & 1) ? (b >> 4) : (b & 0x0F);
+  if (nibble_bias) return nib - nibble_bias; /* HIP flavour: nibble - 8 */
+  return nib >= 8 ? nib - 16 : nib;          /* two's complement nibble  */
+}
+
+/* ---- dequantise -------------------------------------------------------- */
+
+/* out32[k,n] = float(code) * float(scale), the formula of
+ * paddle/phi/kernels/gpu/weight_dequantize_kernel.cu:44-65 and :116-173, with
+ * the scale indexed [k/g, n] as weight_quantize writes it.  The reference then
+ * rounds to T; outT (optional) holds that, with the chosen cast flavour. */
+void wo_dequantize(const int8_t* codes, const uint16_t* scale, int64_t K,
+                   int64_t N, int dtype, int bits, int64_t group_size,
+                   int nibble_bias, int cast_mode, float* out32,
+                   uint16_t* outT) {
+  for (int64_t k = 0; k < K; ++k) {
+    const uint16_t* srow =
+        group_size > 0 ? scale + (k / group_size) * N : scale;
+    for (int64_t n = 0; n < N; ++n) {
+      float v = (float)code_at(codes, k, n, N, bits, nibble_bias) *
+                wo_to_f32(srow[n], dtype);
+      if (out32) out32[k * N + n] = v;
+      if (outT) outT[k * N + n] = wo_from_f32(v, dtype, cast_mode);
+    }
+  }
+}
+
+/* ---- linear ------------------------------------------------------------ */
+
+/* out[m,n] = sum_k x[m,k] * dequant(W)[k,n] + bias[n], the contract of
+ * WeightOnlyLinearKernel (paddle/phi/kernels/gpu/weight_only_linear_kernel.cu:
+ * 48-58; m = x.numel()/k, bias optional, output dtype = x dtype).  The
+ * dequantised weight stays in fp32 and is never rounded to T.  acc64 != 0
+ * accumulates in double (error-study variant), else in fp32 in k order.
+ * out32 receives the unrounded result, outT (optional) its RNE cast to T. */
+void wo_linear(const uint16_t* x, const int8_t* codes, const uint16_t* bias,
+               const uint16_t* scale, int64_t M, int64_t K, int64_t N,
+               int dtype, int bits, int64_t group_size, int nibble_bias,
+               int acc64, float* out32, uint16_t* outT) {
+  float* wrow = (float*)malloc((size_t)N * sizeof(float));
+  float* acc_f = (float*)malloc((size_t)N * sizeof(float));
+  double* acc_d = (double*)malloc((size_t)N * sizeof(double));
+  for (int64_t m = 0; m < M; ++m) {
+    for (int64_t n = 0; n < N; ++n) { acc_f[n] = 0.0f; acc_d[n] = 0.0; }
+    for (int64_t k = 0; k < K; ++k) {
+      const uint16_t* srow =
+          group_size > 0 ? scale + (k / group_size) * N : scale;
+      for (int64_t n = 0; n < N; ++n)
+        wrow[n] = (float)code_at(codes, k, n, N, bits, nibble_bias) *
+                  wo_to_f32(srow[n], dtype);
+      float xv = wo_to_f32(x[m * K + k], dtype);
+      if (acc64) {
+        for (int64_t n = 0; n < N; ++n) acc_d[n] += (double)xv * (double)wrow[n];
+      } else {
+        for (int64_t n = 0; n < N; ++n) acc_f[n] += xv * wrow[n];
+      }
+    }
+    for (int64_t n = 0; n < N; ++n) {
+      float b = bias ? wo_to_f32(bias[n], dtype) : 0.0f;
+      float v = acc64 ? (float)(acc_d[n] + (double)b) : acc_f[n] + b;
+      out32[m * N + n] = v;
+      if (outT) outT[m * N + n] = wo_from_f32(v, dtype, WO_CAST_RNE);
+    }
+  }
+  free(wrow); free(acc_f); free(acc_d);
+}
+
+/* Dequantise once into fp32 [K,N] (the middle stage of the CPU baseline:
+ * quantize, dequantize, fp32 matmul). */
+void wo_dequantize_f32(const int8_t* codes, const uint16_t* scale, int64_t K,
+                       int64_t N, int dtype, int bits, int64_t group_size,
+                       int nibble_bias, float* out32) {
+  wo_dequantize(codes, scale, K, N, dtype, bits, group_size, nibble_bias,
+                WO_CAST_RNE, out32, NULL);
+}

@@ -1,0 +1,144 @@
+"""ctypes front end of the CPU oracle (oracle/wo_oracle.c).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and
+by the cpu_baseline leg of bench.py, always as the checker or the timed CPU
+baseline, never by the shipped package.
+
+Arrays are numpy: weights / activations / scales travel as uint16 bit patterns
+of float16 or bfloat16, codes as int8.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libwo_oracle.so")
+
+F16, BF16 = 0, 1
+CAST_RNE, CAST_TRUNC = 0, 1
+
+_u16p = np.ctypeslib.ndpointer(np.uint16, flags="C_CONTIGUOUS")
+_i8p = np.ctypeslib.ndpointer(np.int8, flags="C_CONTIGUOUS")
+_f32p = np.ctypeslib.ndpointer(np.float32, flags="C_CONTIGUOUS")
+_i64 = ctypes.c_int64
+_int = ctypes.c_int
+
+
+def build(force=False):
+    """Compile the oracle (and oracle/_ref when the reference tree exists)."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.check_call(["make", "-C", _HERE, "-B"] if force else ["make", "-C", _HERE])
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        L = ctypes.CDLL(_LIB_PATH)
+        L.wo_from_f32.argtypes = [ctypes.c_float, _int, _int]
+        L.wo_from_f32.restype = ctypes.c_uint16
+        L.wo_to_f32.argtypes = [ctypes.c_uint16, _int]
+        L.wo_to_f32.restype = ctypes.c_float
+        L.wo_cast_array_from_f32.argtypes = [_f32p, _i64, _int, _int, _u16p]
+        L.wo_cast_array_to_f32.argtypes = [_u16p, _i64, _int, _f32p]
+        L.wo_per_channel_scale.argtypes = [_u16p, _i64, _i64, _int, ctypes.c_float, _int, _u16p]
+        L.wo_group_wise_scale.argtypes = [_u16p, _i64, _i64, _int, ctypes.c_float, _i64, _int, _u16p]
+        L.wo_quant_codes.argtypes = [_u16p, _u16p, _i64, _i64, _int, _int, _i64, _int, _i8p]
+        L.wo_weight_quantize.argtypes = [_u16p, _i64, _i64, _int, _int, _i64, _int, _int, _i8p, _u16p]
+        L.wo_weight_quantize.restype = _int
+        L.wo_transpose_bytes.argtypes = [_i8p, _i64, _i64, _i8p]
+        L.wo_dequantize.argtypes = [_i8p, _u16p, _i64, _i64, _int, _int, _i64, _int, _int,
+                                    ctypes.c_void_p, ctypes.c_void_p]
+        L.wo_linear.argtypes = [_u16p, _i8p, ctypes.c_void_p, _u16p, _i64, _i64, _i64, _int, _int,
+                                _i64, _int, _int, _f32p, ctypes.c_void_p]
+        _lib = L
+    return _lib
+
+
+def from_f32(a, dtype, cast_mode=CAST_RNE):
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    out = np.empty(a.shape, np.uint16)
+    lib().wo_cast_array_from_f32(a.reshape(-1), a.size, dtype, cast_mode, out.reshape(-1))
+    return out
+
+
+def to_f32(a, dtype):
+    a = np.ascontiguousarray(a, dtype=np.uint16)
+    out = np.empty(a.shape, np.float32)
+    lib().wo_cast_array_to_f32(a.reshape(-1), a.size, dtype, out.reshape(-1))
+    return out
+
+
+def weight_quantize(w_bits, dtype, bits, group_size=-1, cast_mode=CAST_RNE, nibble_bias=0):
+    """w_bits: [K,N] uint16.  Returns (codes, scale): canonical codes [K,N] int8
+    or [K,N/2] packed nibbles, scale [N] or [ceil(K/g),N] uint16."""
+    w_bits = np.ascontiguousarray(w_bits, dtype=np.uint16)
+    K, N = w_bits.shape
+    codes = np.empty((K, N if bits == 8 else N // 2), np.int8)
+    if group_size == -1:
+        scale = np.empty((N,), np.uint16)
+    else:
+        scale = np.empty(((K + group_size - 1) // group_size, N), np.uint16)
+    rc = lib().wo_weight_quantize(w_bits, K, N, dtype, bits, group_size, cast_mode, nibble_bias,
+                                  codes, scale)
+    if rc != 0:
+        raise ValueError("oracle: shape/group_size outside the weight_quantize contract")
+    return codes, scale
+
+
+def transpose_bytes(a):
+    a = np.ascontiguousarray(a, dtype=np.int8)
+    out = np.empty((a.shape[1], a.shape[0]), np.int8)
+    lib().wo_transpose_bytes(a, a.shape[0], a.shape[1], out)
+    return out
+
+
+def dequantize(codes, scale, dtype, bits, group_size=-1, nibble_bias=0, cast_mode=CAST_RNE):
+    """Returns (fp32 [K,N], T-bits [K,N])."""
+    codes = np.ascontiguousarray(codes, dtype=np.int8)
+    scale = np.ascontiguousarray(scale, dtype=np.uint16)
+    K = codes.shape[0]
+    N = codes.shape[1] if bits == 8 else codes.shape[1] * 2
+    out32 = np.empty((K, N), np.float32)
+    outT = np.empty((K, N), np.uint16)
+    lib().wo_dequantize(codes, scale, K, N, dtype, bits, group_size, nibble_bias, cast_mode,
+                        out32.ctypes.data, outT.ctypes.data)
+    return out32, outT
+
+
+def linear(x_bits, codes, scale, bias_bits, dtype, bits, group_size=-1, nibble_bias=0, acc64=False):
+    """x_bits [M,K] uint16.  Returns (out32 [M,N] fp32, outT [M,N] uint16)."""
+    x_bits = np.ascontiguousarray(x_bits, dtype=np.uint16)
+    codes = np.ascontiguousarray(codes, dtype=np.int8)
+    scale = np.ascontiguousarray(scale, dtype=np.uint16)
+    M, K = x_bits.shape
+    N = codes.shape[1] if bits == 8 else codes.shape[1] * 2
+    assert codes.shape[0] == K
+    out32 = np.empty((M, N), np.float32)
+    outT = np.empty((M, N), np.uint16)
+    bias_ptr = None
+    if bias_bits is not None:
+        bias_bits = np.ascontiguousarray(bias_bits, dtype=np.uint16)
+        bias_ptr = bias_bits.ctypes.data
+    lib().wo_linear(x_bits, codes, bias_ptr, scale, M, K, N, dtype, bits, group_size, nibble_bias,
+                    1 if acc64 else 0, out32, outT.ctypes.data)
+    return out32, outT
+
+
+def ref_casts(flavour):
+    """Load oracle/_ref/libref_casts_<flavour>.so (plain | f16c | hipflavour), or None."""
+    path = os.path.join(_HERE, "_ref", "libref_casts_%s.so" % flavour)
+    if not os.path.exists(path):
+        return None
+    L = ctypes.CDLL(path)
+    L.ref_f32_to_bf16_array.argtypes = [_f32p, _i64, _u16p]
+    if flavour != "hipflavour":
+        L.ref_f32_to_f16_array.argtypes = [_f32p, _i64, _u16p]
+        L.ref_f16_to_f32_array.argtypes = [_u16p, _i64, _f32p]
+    return L

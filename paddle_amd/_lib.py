@@ -1,0 +1,79 @@
+"""ctypes binding of libwol_gfx950.so (the C ABI of include/wol_c_api.h).
+
+The library is the only compute path: if it is missing, import fails loudly
+instead of falling back to anything else.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libwol_gfx950.so")
+
+DTYPE_F16, DTYPE_BF16 = 0, 1
+ROUND_RNE, ROUND_TRUNC = 0, 1
+LAYOUT_CANONICAL, LAYOUT_PADDLE_HIP, LAYOUT_GFX950 = 0, 1, 2
+
+# every symbol include/wol_c_api.h declares
+SYMBOLS = (
+    "wol_status_str",
+    "wol_layout_version",
+    "wol_quantize_workspace",
+    "wol_quantize",
+    "wol_dequantize",
+    "wol_linear_workspace",
+    "wol_linear",
+    "wol_linear_f32",
+    "wol_repack",
+    "wol_code_offset",
+)
+
+
+class WolError(RuntimeError):
+    """A non-zero wol_status that is not an argument error."""
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            "libwol_gfx950.so is not built (%s); run paddle_amd/csrc/build.sh or "
+            "__graft_entry__.build()" % LIB_PATH
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    vp, i64, ci, sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t
+    lib.wol_status_str.argtypes = [ci]
+    lib.wol_status_str.restype = ctypes.c_char_p
+    lib.wol_layout_version.argtypes = []
+    lib.wol_layout_version.restype = ci
+    lib.wol_quantize_workspace.argtypes = [i64, i64, ci, ci]
+    lib.wol_quantize_workspace.restype = sz
+    lib.wol_quantize.argtypes = [vp, ci, i64, i64, ci, ci, ci, ci, vp, vp, vp, sz, vp]
+    lib.wol_quantize.restype = ci
+    lib.wol_dequantize.argtypes = [vp, ci, vp, ci, i64, i64, ci, ci, vp, vp]
+    lib.wol_dequantize.restype = ci
+    lib.wol_linear_workspace.argtypes = [i64, i64, i64, ci, ci]
+    lib.wol_linear_workspace.restype = sz
+    lib.wol_linear.argtypes = [vp, vp, vp, vp, ci, i64, i64, i64, ci, ci, vp, vp, sz, vp]
+    lib.wol_linear.restype = ci
+    lib.wol_linear_f32.argtypes = [vp, vp, vp, vp, ci, i64, i64, i64, ci, ci, vp, vp, sz, vp]
+    lib.wol_linear_f32.restype = ci
+    lib.wol_repack.argtypes = [vp, ci, vp, ci, i64, i64, ci, vp]
+    lib.wol_repack.restype = ci
+    lib.wol_code_offset.argtypes = [ci, i64, i64, ci, i64, i64, ctypes.POINTER(ci)]
+    lib.wol_code_offset.restype = i64
+    return lib
+
+
+lib = _load()
+
+# statuses that are argument errors (the reference raises InvalidArgument,
+# which Paddle surfaces as ValueError)
+_ARG_ERRORS = {1, 2, 3, 4, 5, 6, 7, 8, 9}
+
+
+def check(status):
+    if status == 0:
+        return
+    msg = lib.wol_status_str(status).decode()
+    if status in _ARG_ERRORS:
+        raise ValueError("(InvalidArgument) %s [wol_status %d]" % (msg, status))
+    raise WolError("%s [wol_status %d]" % (msg, status))

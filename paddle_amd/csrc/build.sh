@@ -1,0 +1,21 @@
+#!/bin/bash
+# Builds paddle_amd/lib/libwol_gfx950.so from the HIP sources beside this file.
+set -euo pipefail
+HERE="$(cd "$(dirname "${BASH_SOURCE[0]}")" && pwd)"
+ROOT="$(cd "$HERE/../.." && pwd)"
+OUT="$HERE/../lib"
+OBJ="$HERE/build"
+mkdir -p "$OUT" "$OBJ"
+HIPCC="${HIPCC:-/opt/rocm/bin/hipcc}"
+FLAGS=(--offload-arch=gfx950 -O3 -std=c++17 -fPIC -I"$ROOT/include" -I"$HERE"
+       -Xclang -target-feature -Xclang -packed-fp32-ops
+       -Wno-unused-command-line-argument -Wno-unknown-attributes)
+pids=()
+for f in wol_quantize wol_linear_stream wol_linear_gemm wol_c_api; do
+  "$HIPCC" "${FLAGS[@]}" -c "$HERE/$f.hip" -o "$OBJ/$f.o" &
+  pids+=($!)
+done
+for p in "${pids[@]}"; do wait "$p"; done
+"$HIPCC" --offload-arch=gfx950 -shared -fPIC -o "$OUT/libwol_gfx950.so" \
+  "$OBJ/wol_quantize.o" "$OBJ/wol_linear_stream.o" "$OBJ/wol_linear_gemm.o" "$OBJ/wol_c_api.o"
+echo "built $OUT/libwol_gfx950.so"

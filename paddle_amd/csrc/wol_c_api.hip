@@ -1,0 +1,145 @@
+// extern "C" entry points of libwol_gfx950.so: argument validation (the
+// shape/dtype contract of the reference's InferMeta functions), kernel
+// selection, nothing else.  See include/wol_c_api.h for the contract.
+#include "wol_common.h"
+
+namespace {
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// paddle/phi/infermeta/unary.cc:5961-5983 (weight_quantize) and
+// multiary.cc:5503-5560 (weight_only_linear): K % 64, N % 16, group size.
+int check_problem(int dtype, int64_t K, int64_t N, int bits, int group_size) {
+  if (dtype != WOL_DTYPE_F16 && dtype != WOL_DTYPE_BF16) return WOL_ERR_BAD_DTYPE;
+  if (bits != 8 && bits != 4) return WOL_ERR_BAD_BITS;
+  if (!(group_size == -1 || group_size == 64 || group_size == 128)) return WOL_ERR_BAD_GROUP_SIZE;
+  if (K <= 0 || N <= 0 || K % 64 != 0 || N % 16 != 0) return WOL_ERR_BAD_SHAPE;
+  // byte offsets inside a tensor are kept in int64; row indices in int32
+  if (K > (int64_t{1} << 30) || N > (int64_t{1} << 30)) return WOL_ERR_BAD_SHAPE;
+  return WOL_OK;
+}
+
+bool layout_ok(int layout) {
+  return layout == WOL_LAYOUT_CANONICAL || layout == WOL_LAYOUT_PADDLE_HIP ||
+         layout == WOL_LAYOUT_GFX950;
+}
+
+// The streaming kernel covers M <= 64 (four 16-row MFMA tiles).
+constexpr int64_t kStreamMaxM = 64;
+
+int linear_impl(const void* x, const void* codes, const void* bias, const void* scale, int dtype,
+                int64_t M, int64_t K, int64_t N, int bits, int group_size, void* out, bool out_f32,
+                void* stream) {
+  const int rc = check_problem(dtype, K, N, bits, group_size);
+  if (rc != WOL_OK) return rc;
+  if (M < 0 || M > (int64_t{1} << 30)) return WOL_ERR_BAD_SHAPE;
+  if (M == 0) return WOL_OK;  // empty batch: nothing to write
+  if (x == nullptr || codes == nullptr || scale == nullptr || out == nullptr)
+    return WOL_ERR_NULL_POINTER;
+  if (!aligned16(x) || !aligned16(codes)) return WOL_ERR_ALIGNMENT;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (M <= kStreamMaxM)
+    return wol::launch_linear_stream(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out,
+                                     out_f32, s);
+  return wol::launch_linear_gemm(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out,
+                                 out_f32, s);
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* wol_status_str(int status) {
+  switch (status) {
+    case WOL_OK: return "ok";
+    case WOL_ERR_NULL_POINTER: return "a required pointer is NULL";
+    case WOL_ERR_BAD_DTYPE: return "dtype must be float16 (0) or bfloat16 (1)";
+    case WOL_ERR_BAD_BITS: return "weight_dtype must be int8 or int4";
+    case WOL_ERR_BAD_GROUP_SIZE: return "group_size must be -1, 64 or 128";
+    case WOL_ERR_BAD_SHAPE:
+      return "shape outside the contract (K divisible by 64, N divisible by 16, sizes positive)";
+    case WOL_ERR_BAD_LAYOUT: return "unknown weight layout";
+    case WOL_ERR_BAD_ROUND_MODE: return "round_mode must be RNE (0) or TRUNC (1)";
+    case WOL_ERR_WORKSPACE: return "workspace missing or too small";
+    case WOL_ERR_ALIGNMENT: return "pointer not 16-byte aligned";
+    case WOL_ERR_HIP: return "HIP launch failed";
+    case WOL_ERR_NO_DEVICE: return "no gfx950 device";
+    default: return "unknown status";
+  }
+}
+
+int wol_layout_version(void) { return wol::kLayoutVersion; }
+
+size_t wol_quantize_workspace(int64_t K, int64_t N, int bits, int group_size) {
+  if (check_problem(WOL_DTYPE_F16, K, N, bits, group_size) != WOL_OK) return 0;
+  return group_size == -1 ? static_cast<size_t>(N) * sizeof(uint32_t) : 0;
+}
+
+int wol_quantize(const void* w, int dtype, int64_t K, int64_t N, int bits, int group_size,
+                 int round_mode, int layout, void* codes_out, void* scale_out, void* workspace,
+                 size_t workspace_bytes, void* stream) {
+  const int rc = check_problem(dtype, K, N, bits, group_size);
+  if (rc != WOL_OK) return rc;
+  if (round_mode != WOL_ROUND_RNE && round_mode != WOL_ROUND_TRUNC) return WOL_ERR_BAD_ROUND_MODE;
+  if (!layout_ok(layout)) return WOL_ERR_BAD_LAYOUT;
+  if (w == nullptr || codes_out == nullptr || scale_out == nullptr) return WOL_ERR_NULL_POINTER;
+  if (!aligned16(w) || !aligned16(codes_out)) return WOL_ERR_ALIGNMENT;
+  const size_t need = wol_quantize_workspace(K, N, bits, group_size);
+  if (need > 0 && (workspace == nullptr || workspace_bytes < need)) return WOL_ERR_WORKSPACE;
+  return wol::launch_quantize(w, dtype, K, N, bits, group_size, round_mode, layout, codes_out,
+                              scale_out, workspace, static_cast<hipStream_t>(stream));
+}
+
+int wol_dequantize(const void* codes, int layout, const void* scale, int dtype, int64_t K,
+                   int64_t N, int bits, int group_size, void* out_KN, void* stream) {
+  const int rc = check_problem(dtype, K, N, bits, group_size);
+  if (rc != WOL_OK) return rc;
+  if (!layout_ok(layout)) return WOL_ERR_BAD_LAYOUT;
+  if (codes == nullptr || scale == nullptr || out_KN == nullptr) return WOL_ERR_NULL_POINTER;
+  if (!aligned16(scale) || !aligned16(out_KN)) return WOL_ERR_ALIGNMENT;
+  return wol::launch_dequantize(codes, layout, scale, dtype, K, N, bits, group_size, out_KN,
+                                static_cast<hipStream_t>(stream));
+}
+
+size_t wol_linear_workspace(int64_t M, int64_t K, int64_t N, int bits, int group_size) {
+  (void)M; (void)K; (void)N; (void)bits; (void)group_size;
+  return 0;  // both kernels keep their partial sums on chip
+}
+
+int wol_linear(const void* x, const void* codes, const void* bias, const void* scale, int dtype,
+               int64_t M, int64_t K, int64_t N, int bits, int group_size, void* out,
+               void* workspace, size_t workspace_bytes, void* stream) {
+  (void)workspace; (void)workspace_bytes;
+  return linear_impl(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out, false, stream);
+}
+
+int wol_linear_f32(const void* x, const void* codes, const void* bias, const void* scale,
+                   int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
+                   float* out_f32, void* workspace, size_t workspace_bytes, void* stream) {
+  (void)workspace; (void)workspace_bytes;
+  return linear_impl(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out_f32, true,
+                     stream);
+}
+
+int wol_repack(const void* codes_in, int layout_in, void* codes_out, int layout_out, int64_t K,
+               int64_t N, int bits, void* stream) {
+  const int rc = check_problem(WOL_DTYPE_F16, K, N, bits, -1);
+  if (rc != WOL_OK) return rc;
+  if (!layout_ok(layout_in) || !layout_ok(layout_out)) return WOL_ERR_BAD_LAYOUT;
+  if (codes_in == nullptr || codes_out == nullptr) return WOL_ERR_NULL_POINTER;
+  if (codes_in == codes_out) return WOL_ERR_BAD_LAYOUT;  // not in place
+  return wol::launch_repack(codes_in, layout_in, codes_out, layout_out, K, N, bits,
+                            static_cast<hipStream_t>(stream));
+}
+
+int64_t wol_code_offset(int layout, int64_t K, int64_t N, int bits, int64_t k, int64_t n,
+                        int* nibble_shift) {
+  if (check_problem(WOL_DTYPE_F16, K, N, bits, -1) != WOL_OK || !layout_ok(layout)) return -1;
+  if (k < 0 || k >= K || n < 0 || n >= N) return -1;
+  int shift = 0;
+  const int64_t off = wol::code_offset(layout, K, N, bits, k, n, &shift);
+  if (nibble_shift != nullptr) *nibble_shift = shift;
+  return off;
+}
+
+}  // extern "C"

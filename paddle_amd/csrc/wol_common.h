@@ -1,0 +1,189 @@
+// Shared definitions of the gfx950 weight-only library: scalar type casts,
+// the three code layouts and the index arithmetic of the GFX950 layout.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "wol_c_api.h"
+
+namespace wol {
+
+// ---------------------------------------------------------------------------
+// GFX950 layout, version 1
+//
+// The weight is cut into strips of 16 output columns; strip tn holds columns
+// [16*tn, 16*tn+16) for every k and is contiguous: 16*K*bits/8 bytes, so a
+// slice of the tensor along N at a multiple of 16 is still a valid tensor.
+// Inside a strip the bytes are ordered exactly as one wavefront consumes them
+// as the B operand of v_mfma_f32_16x16x32_{bf16,f16}: lane = 16*kb + j reads
+// column j and the eight k values 8*kb .. 8*kb+7 of a 32-deep k step, and one
+// 16-byte load per lane covers KT = 64 (int8) or 128 (int4) consecutive k:
+//
+//   int8: tile = 64 k  -> 1 KiB.  lane's 16 B = [k step 0: 8 B][k step 1: 8 B],
+//         byte i of a k step = code(k0 + 32*step + 8*kb + i, n) + 128.
+//   int4: tile = 128 k -> 1 KiB.  lane's 16 B = 4 dwords, one per k step;
+//         nibble position p of a dword holds i = 2*p (p < 4) or 2*(p-4)+1, so
+//         that (dword >> 4*p) & 0x000F000F is the pair (i, i+1) = (2p, 2p+1)
+//         in the low/high halves; nibble = code + 8.
+//         A K that is 64 mod 128 ends with a half tile of 512 B (8 B per lane,
+//         two k steps).
+// Biased (unsigned) storage lets a code turn into a bf16/fp16 bit pattern with
+// one AND-OR; the bias is removed exactly by the consumer.
+// ---------------------------------------------------------------------------
+constexpr int kLayoutVersion = 1;
+constexpr int kStripCols = 16;
+
+__host__ __device__ inline int64_t strip_bytes(int64_t K, int bits) {
+  return kStripCols * K * bits / 8;
+}
+
+// Byte offset and nibble shift (0 or 4; always 0 for int8) of element (k, n).
+__host__ __device__ inline int64_t gfx950_offset(int64_t K, int bits, int64_t k,
+                                                int64_t n, int* nib_shift) {
+  const int64_t tn = n / kStripCols;
+  const int j = static_cast<int>(n % kStripCols);
+  const int kb = static_cast<int>((k % 32) / 8);
+  const int i = static_cast<int>(k % 8);
+  const int lane = kb * 16 + j;
+  if (bits == 8) {
+    const int64_t kt = k / 64;
+    const int step = static_cast<int>((k % 64) / 32);
+    *nib_shift = 0;
+    return tn * strip_bytes(K, 8) + kt * 1024 + lane * 16 + step * 8 + i;
+  }
+  const int pos = (i >> 1) + 4 * (i & 1);
+  const int64_t full = K / 128;  // number of full tiles
+  const int64_t kt = k / 128;
+  *nib_shift = (pos & 1) * 4;
+  if (kt < full) {
+    const int step = static_cast<int>((k % 128) / 32);
+    return tn * strip_bytes(K, 4) + kt * 1024 + lane * 16 + step * 4 + pos / 2;
+  }
+  const int step = static_cast<int>((k % 64) / 32);  // half tile at the end
+  return tn * strip_bytes(K, 4) + full * 1024 + lane * 8 + step * 4 + pos / 2;
+}
+
+// Byte offset / nibble shift of element (k, n) in any layout.
+__host__ __device__ inline int64_t code_offset(int layout, int64_t K, int64_t N,
+                                              int bits, int64_t k, int64_t n,
+                                              int* nib_shift) {
+  if (layout == WOL_LAYOUT_GFX950) return gfx950_offset(K, bits, k, n, nib_shift);
+  if (bits == 8) {
+    *nib_shift = 0;
+    return layout == WOL_LAYOUT_CANONICAL ? k * N + n : n * K + k;
+  }
+  *nib_shift = static_cast<int>(n & 1) * 4;
+  return layout == WOL_LAYOUT_CANONICAL ? k * (N / 2) + n / 2
+                                        : (n / 2) * K + k;
+}
+
+// Stored byte / nibble of a signed code q in a layout, and back.
+__host__ __device__ inline int encode_code(int layout, int bits, int q) {
+  if (bits == 8) return layout == WOL_LAYOUT_GFX950 ? ((q + 128) & 0xFF) : (q & 0xFF);
+  return layout == WOL_LAYOUT_CANONICAL ? (q & 0xF) : ((q + 8) & 0xF);
+}
+
+__host__ __device__ inline int decode_code(int layout, int bits, int v) {
+  if (bits == 8) return layout == WOL_LAYOUT_GFX950 ? (v & 0xFF) - 128
+                                                    : static_cast<int8_t>(v & 0xFF);
+  v &= 0xF;
+  if (layout == WOL_LAYOUT_CANONICAL) return v >= 8 ? v - 16 : v;
+  return v - 8;
+}
+
+// ---------------------------------------------------------------------------
+// T <-> float.  Inputs are bit patterns (uint16_t); widening is exact.
+// ---------------------------------------------------------------------------
+__device__ inline float bf16_to_f32(uint16_t h) {
+  return __uint_as_float(static_cast<uint32_t>(h) << 16);
+}
+
+__device__ inline float f16_to_f32(uint16_t h) {
+  return static_cast<float>(__builtin_bit_cast(_Float16, h));
+}
+
+template <int DT>
+__device__ inline float to_f32(uint16_t h) {
+  return DT == WOL_DTYPE_BF16 ? bf16_to_f32(h) : f16_to_f32(h);
+}
+
+// Round-to-nearest-even float -> bf16, with the special cases of
+// paddle/phi/common/bfloat16.h:61-88: zero keeps only its sign, infinity
+// passes, NaN becomes 0x7FFF.
+__device__ inline uint16_t f32_to_bf16_rne(float f) {
+  const uint32_t u = __float_as_uint(f);
+  const uint32_t mag = u & 0x7FFFFFFFu;
+  if (mag > 0x7F800000u) return 0x7FFFu;
+  if (mag == 0x7F800000u || mag == 0) return static_cast<uint16_t>(u >> 16);
+  return static_cast<uint16_t>((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+
+// Round-to-nearest-even float -> fp16 (v_cvt_f16_f32 under the default
+// rounding mode, denormals on).  NaN is canonicalised like _cvtss_sh does:
+// quiet bit set, top payload bits kept.
+__device__ inline uint16_t f32_to_f16_rne(float f) {
+  const uint32_t u = __float_as_uint(f);
+  const uint32_t mag = u & 0x7FFFFFFFu;
+  if (mag > 0x7F800000u)
+    return static_cast<uint16_t>(((u >> 16) & 0x8000u) | 0x7E00u | ((mag >> 13) & 0x3FFu));
+  return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
+}
+
+// The truncating flavours (WOL_ROUND_TRUNC): bf16 drops the low half
+// (paddle/phi/common/bfloat16.h:103-110); fp16 follows the software routine of
+// a host build without F16C (paddle/phi/common/float16.h:121-139): magnitudes
+// truncate, anything above 65504 is infinity, subnormals are floor(|f|*2^24).
+__device__ inline uint16_t f32_to_bf16_trunc(float f) {
+  return static_cast<uint16_t>(__float_as_uint(f) >> 16);
+}
+
+__device__ inline uint16_t f32_to_f16_trunc(float f) {
+  const uint32_t u = __float_as_uint(f);
+  const uint16_t sign = static_cast<uint16_t>((u >> 16) & 0x8000u);
+  const uint32_t mag = u & 0x7FFFFFFFu;
+  if (mag > 0x7F800000u) {
+    if (mag < 0x7F802000u) return sign | 0x7C01u;
+    return sign | 0x7C00u | static_cast<uint16_t>((mag >> 13) & 0x3FFu);
+  }
+  if (mag > 0x477FE000u) return sign | 0x7C00u;
+  if (mag < 0x38800000u) {
+    // |f| < 2^-14: the product is exact (power-of-two factor) and < 2^23.
+    const float scaled = __uint_as_float(mag) * __uint_as_float(0x52000000u);
+    return sign | static_cast<uint16_t>(static_cast<uint32_t>(scaled) >> 13);
+  }
+  return sign | static_cast<uint16_t>((mag >> 13) - 0x1C000u);
+}
+
+template <int DT>
+__device__ inline uint16_t from_f32(float f, int round_mode) {
+  if (DT == WOL_DTYPE_BF16)
+    return round_mode == WOL_ROUND_TRUNC ? f32_to_bf16_trunc(f) : f32_to_bf16_rne(f);
+  return round_mode == WOL_ROUND_TRUNC ? f32_to_f16_trunc(f) : f32_to_f16_rne(f);
+}
+
+template <int DT>
+__device__ inline uint16_t from_f32_rne(float f) {
+  return DT == WOL_DTYPE_BF16 ? f32_to_bf16_rne(f) : f32_to_f16_rne(f);
+}
+
+// Launchers implemented in the .hip files; each returns a wol_status.
+int launch_quantize(const void* w, int dtype, int64_t K, int64_t N, int bits, int group_size,
+                    int round_mode, int layout, void* codes, void* scale, void* workspace,
+                    hipStream_t stream);
+int launch_dequantize(const void* codes, int layout, const void* scale, int dtype, int64_t K,
+                      int64_t N, int bits, int group_size, void* out, hipStream_t stream);
+int launch_repack(const void* in, int layout_in, void* out, int layout_out, int64_t K, int64_t N,
+                  int bits, hipStream_t stream);
+int launch_linear_stream(const void* x, const void* codes, const void* bias, const void* scale,
+                         int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
+                         void* out, bool out_f32, hipStream_t stream);
+int launch_linear_gemm(const void* x, const void* codes, const void* bias, const void* scale,
+                       int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
+                       void* out, bool out_f32, hipStream_t stream);
+
+inline int check_launch() {
+  return hipGetLastError() == hipSuccess ? WOL_OK : WOL_ERR_HIP;
+}
+
+}  // namespace wol

@@ -1,0 +1,9 @@
+"""Mirror of paddle.nn.quant's weight-only entry points
+(python/paddle/nn/quant/__init__.py:28-42 in the reference)."""
+from .quantized_linear import (  # noqa: F401
+    weight_dequantize,
+    weight_only_linear,
+    weight_quantize,
+)
+
+__all__ = ["weight_only_linear", "weight_quantize", "weight_dequantize"]
