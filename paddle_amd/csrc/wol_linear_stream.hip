@@ -7,13 +7,24 @@
 // coalesced, one tile of 64 or 128 k), turns the biased codes into bf16/fp16
 // bit patterns with AND-OR / byte-permute tricks (the code plus a constant
 // offset, exact), and issues v_mfma_f32_16x16x32 with the activations as the
-// A operand (rows >= M are zero) -- the MFMA does the multiply and the
-// reduction over k across lanes.  The constant offset is removed by a second
-// MFMA of the same A against a constant B, which is exact in fp32 up to the
-// accumulator's rounding; accumulators restart every 64 k so the cancelling
-// terms stay small.  Scales multiply the fp32 partial sums (once per group),
-// never the weights, so nothing is rounded to T before the final cast.
-// Partial sums of the WK wavefronts meet in LDS in a fixed order.
+// A operand -- the MFMA does the multiply and the reduction over k across
+// lanes.  The constant offset is removed by a second MFMA of the same A
+// against a constant B, exact in fp32 up to the accumulator's rounding; the
+// accumulator restarts every k step so the cancelling terms stay small.
+// Scales multiply the fp32 partial sums, never the weights, so nothing is
+// rounded to T before the final cast.
+//
+// Small M does not fill the 16 rows of the A operand, and rows of the result
+// are independent of each other, so the spare rows carry other k steps: with
+// MP = M rounded up to a power of two, one 16-byte-per-lane load of x (1 KiB,
+// coalesced) fills row group `slot` with the activations of k step `slot`,
+// S = 16/MP steps at once.  The MFMA of step s against that operand produces
+// the wanted dot products in row group s and unrelated finite sums elsewhere;
+// a per-lane select keeps only row group s.  For M = 1 this is one x load per
+// 512 k instead of sixteen.  Rows beyond M may hold anything (they are never
+// stored), so no operand is ever zero-filled.
+// Partial sums of row groups and of the WK wavefronts meet in LDS in a fixed
+// order.
 #include "wol_common.h"
 
 namespace wol {
@@ -43,16 +54,25 @@ __device__ inline f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
 template <int DT, int BITS>
 struct Dequant;
 
+// (v & mask) | magic.  magic arrives in a VGPR whose value the compiler cannot
+// see, which lets it pick the three-operand v_and_or_b32 (mask on the scalar
+// bus) instead of two instructions with literals.  Written as plain C so the
+// compiler's MFMA hazard tracking sees every register it touches.
+__device__ inline uint32_t and_or(uint32_t v, uint32_t mask, uint32_t magic) {
+  return (v & mask) | magic;
+}
+
 template <>
 struct Dequant<WOL_DTYPE_BF16, 4> {
   static constexpr uint32_t kCancel = 0xC308C308u;  // -136, -136
-  __device__ static inline u32x4 run(const uint32_t* w) {
+  static constexpr uint32_t kMagic = 0x43004300u;
+  __device__ static inline u32x4 run(const uint32_t* w, uint32_t magic) {
     const uint32_t v = w[0];
     u32x4 o;
-    o.x = (v & 0x000F000Fu) | 0x43004300u;
-    o.y = ((v >> 4) & 0x000F000Fu) | 0x43004300u;
-    o.z = ((v >> 8) & 0x000F000Fu) | 0x43004300u;
-    o.w = ((v >> 12) & 0x000F000Fu) | 0x43004300u;
+    o.x = and_or(v, 0x000F000Fu, magic);
+    o.y = and_or(v >> 4, 0x000F000Fu, magic);
+    o.z = and_or(v >> 8, 0x000F000Fu, magic);
+    o.w = and_or(v >> 12, 0x000F000Fu, magic);
     return o;
   }
 };
@@ -60,13 +80,14 @@ struct Dequant<WOL_DTYPE_BF16, 4> {
 template <>
 struct Dequant<WOL_DTYPE_F16, 4> {
   static constexpr uint32_t kCancel = 0xD480D480u;  // -72, -72
-  __device__ static inline u32x4 run(const uint32_t* w) {
+  static constexpr uint32_t kMagic = 0x54005400u;
+  __device__ static inline u32x4 run(const uint32_t* w, uint32_t magic) {
     const uint32_t v = w[0];
     u32x4 o;
-    o.x = ((v << 4) & 0x00F000F0u) | 0x54005400u;
-    o.y = (v & 0x00F000F0u) | 0x54005400u;
-    o.z = ((v >> 4) & 0x00F000F0u) | 0x54005400u;
-    o.w = ((v >> 8) & 0x00F000F0u) | 0x54005400u;
+    o.x = and_or(v << 4, 0x00F000F0u, magic);
+    o.y = and_or(v, 0x00F000F0u, magic);
+    o.z = and_or(v >> 4, 0x00F000F0u, magic);
+    o.w = and_or(v >> 8, 0x00F000F0u, magic);
     return o;
   }
 };
@@ -74,12 +95,13 @@ struct Dequant<WOL_DTYPE_F16, 4> {
 template <>
 struct Dequant<WOL_DTYPE_BF16, 8> {
   static constexpr uint32_t kCancel = 0xC300C300u;  // -128, -128
+  static constexpr uint32_t kMagic = 0u;
   __device__ static inline uint32_t pair(uint32_t lo_byte_val, uint32_t hi_byte_val) {
     // high halves of two fp32 values side by side (both are exact in bf16)
     return __builtin_amdgcn_perm(__float_as_uint(static_cast<float>(hi_byte_val)),
                                  __float_as_uint(static_cast<float>(lo_byte_val)), 0x07060302u);
   }
-  __device__ static inline u32x4 run(const uint32_t* w) {
+  __device__ static inline u32x4 run(const uint32_t* w, uint32_t) {
     u32x4 o;
     o.x = pair(w[0] & 0xFFu, (w[0] >> 8) & 0xFFu);
     o.y = pair((w[0] >> 16) & 0xFFu, w[0] >> 24);
@@ -92,230 +114,374 @@ struct Dequant<WOL_DTYPE_BF16, 8> {
 template <>
 struct Dequant<WOL_DTYPE_F16, 8> {
   static constexpr uint32_t kCancel = 0xE480E480u;  // -1152, -1152
-  __device__ static inline u32x4 run(const uint32_t* w) {
+  static constexpr uint32_t kMagic = 0x64646464u;
+  __device__ static inline u32x4 run(const uint32_t* w, uint32_t magic) {
     u32x4 o;
-    o.x = __builtin_amdgcn_perm(w[0], 0x64646464u, 0x00050004u);
-    o.y = __builtin_amdgcn_perm(w[0], 0x64646464u, 0x00070006u);
-    o.z = __builtin_amdgcn_perm(w[1], 0x64646464u, 0x00050004u);
-    o.w = __builtin_amdgcn_perm(w[1], 0x64646464u, 0x00070006u);
+    o.x = __builtin_amdgcn_perm(w[0], magic, 0x00050004u);
+    o.y = __builtin_amdgcn_perm(w[0], magic, 0x00070006u);
+    o.z = __builtin_amdgcn_perm(w[1], magic, 0x00050004u);
+    o.w = __builtin_amdgcn_perm(w[1], magic, 0x00070006u);
     return o;
   }
 };
 
-template <int DT, int BITS, int MT, int WK>
+// Sum of v over the four lane groups (lanes l, l^16, l^32, l^48), in every lane.
+__device__ inline float sum_lane_groups(float v, bool x16, bool x32) {
+  if (x32) {
+    const auto p = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(p[0]) + __uint_as_float(p[1]);
+  }
+  if (x16) {
+    const auto q = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(q[0]) + __uint_as_float(q[1]);
+  }
+  return v;
+}
+
+// NU > 0: every wavefront owns exactly NU units and issues all their loads at
+// once (the whole problem is in flight from the first cycle; used when K is
+// small enough).  NU == 0: a wavefront walks its share of the units with the
+// loads of the next unit in flight while it consumes the current one.
+template <int DT, int BITS, int MP, int MT, int WK, int NU, bool GROUPED>
 struct StreamKernel {
-  static constexpr int kTileK = BITS == 8 ? 64 : 128;
-  static constexpr int kSubs = kTileK / 64;         // 64-k sub-blocks per tile
-  static constexpr int kDwPerStep = BITS == 8 ? 2 : 1;
-  static constexpr int kUnroll = MT == 1 ? 4 : (MT == 2 ? 2 : 1);
+  static_assert(MT == 1 || MP == 16, "several M tiles only with full 16-row operands");
+  static constexpr int kS = 16 / MP;                  // k steps sharing one A operand
+  static constexpr int kSPT = BITS == 8 ? 2 : 4;      // k steps per 16-byte weight tile
+  static constexpr int kDw = BITS == 8 ? 2 : 1;       // dwords per k step
+  static constexpr int kU = kS > kSPT ? kS : kSPT;    // k steps per unit of work
+  static constexpr int kNT = kU / kSPT;               // weight tiles per unit
+  static constexpr int kNA = kU / kS;                 // A operands per unit
+  static constexpr int kRowsPerGroup = MP < 4 ? 4 / MP : 1;  // row groups inside one lane group
+  static constexpr int kClasses = kS / kRowsPerGroup;        // lane groups that receive results
+  static constexpr int kLive = MP == 1 ? 1 : (MP == 2 ? 2 : 4);  // accumulators left after folding
 
   const uint16_t* x;
   const uint16_t* scale;
-  int M;
-  int64_t K, N;
-  int group_size;
-  int out_f32;
-  int lane, j, kb;
-  int64_t n;
-  f32x4 tot[MT];
+  int M, K, N;
+  int gshift;  // log2(group_size) when GROUPED
+  int lane, j, kb, n;
+  uint32_t magic;
+  // totc[mt][c] gathers the steps whose results belong to lane group c (for
+  // MP = 8: lane groups 2c, 2c+1); lanes outside that group accumulate sums
+  // that are discarded when the classes are merged at the end.
+  f32x4 totc[MT][kClasses];
 
-  __device__ inline u32x4 load_a(int mt, int64_t k) const {
-    const int m = mt * 16 + j;
-    u32x4 a = {0u, 0u, 0u, 0u};
-    if (m < M) a = *reinterpret_cast<const u32x4*>(x + static_cast<int64_t>(m) * K + k + 8 * kb);
-    return a;
+  // Everything one unit of work (kU k steps of this strip) reads from memory.
+  struct Unit {
+    u32x4 wv[kNT];
+    u32x4 av[kNA][MT];
+    uint16_t sraw[kU / 2];
+  };
+
+  // A operand whose row group `slot` holds k step (step0 + slot); with
+  // spread == false every row group holds step0.
+  __device__ inline u32x4 load_a(int mt, int step0, bool spread) const {
+    int m = mt * 16 + (j % MP);
+    if (MP > 1 || MT > 1) m = m < M ? m : M - 1;  // rows past M are never stored
+    int step = step0 + (spread ? j / MP : 0);
+    if (NU == 0) {  // a partial unit at the end of K must not read past the row
+      const int last = K / 32 - 1;
+      step = step < last ? step : last;
+    }
+    return *reinterpret_cast<const u32x4*>(x + static_cast<int64_t>(m) * K + step * 32 + 8 * kb);
   }
 
-  __device__ inline float load_scale(int64_t k) const {
-    return to_f32<DT>(scale[(k / group_size) * N + n]);
+  __device__ inline uint16_t load_scale_raw(int step) const {
+    const uint16_t* row = scale + static_cast<int64_t>((step * 32) >> gshift) * N;  // uniform
+    return row[n];
   }
 
-  // One 64-k sub-block: two k steps whose codes are in w[0 .. 2*kDwPerStep).
-  __device__ inline void sub_block(const uint32_t* w, const u32x4 (&a)[2][MT], float s) {
+  __device__ inline void load_unit(Unit& d, const u32x4* tp, int u) const {
+    const int step0 = u * kU;
+#pragma unroll
+    for (int i = 0; i < kNT; ++i) d.wv[i] = __builtin_nontemporal_load(tp + (step0 / kSPT + i) * 64);
+#pragma unroll
+    for (int a = 0; a < kNA; ++a)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) d.av[a][mt] = load_a(mt, step0 + a * kS, true);
+    if (GROUPED) {
+#pragma unroll
+      for (int p = 0; p < kU / 2; ++p) d.sraw[p] = load_scale_raw(step0 + 2 * p);
+    }
+  }
+
+  // mfma(A, constant B): the term that removes the dequantiser's offset.  It
+  // depends on A only, so it is computed once per A operand and used as the
+  // accumulator input of every step that shares the operand.
+  __device__ inline f32x4 cancel_term(u32x4 a) const {
     const u32x4 cancel = {Dequant<DT, BITS>::kCancel, Dequant<DT, BITS>::kCancel,
                           Dequant<DT, BITS>::kCancel, Dequant<DT, BITS>::kCancel};
-    const u32x4 b0 = Dequant<DT, BITS>::run(w);
-    const u32x4 b1 = Dequant<DT, BITS>::run(w + kDwPerStep);
+    return mfma16<DT>(a, cancel, f32x4{0.f, 0.f, 0.f, 0.f});
+  }
+
+  // One k step: dequantise, one MFMA per M tile, add the rows of row group
+  // `slot` to that group's class.
+  __device__ inline void step_mfma(const uint32_t* w, const u32x4 (&a)[MT], const f32x4 (&cc)[MT],
+                                   int slot, float sc) {
+    const u32x4 b = Dequant<DT, BITS>::run(w, magic);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-      acc = mfma16<DT>(a[0][mt], b0, acc);
-      acc = mfma16<DT>(a[0][mt], cancel, acc);
-      acc = mfma16<DT>(a[1][mt], b1, acc);
-      acc = mfma16<DT>(a[1][mt], cancel, acc);
-      tot[mt] += acc * s;
+      const f32x4 acc = mfma16<DT>(a[mt], b, cc[mt]);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const bool rsel = MP >= 4 ? true : (r / MP == slot % kRowsPerGroup);
+        if (rsel) {
+          const float t = totc[mt][slot / kRowsPerGroup][r];
+          totc[mt][slot / kRowsPerGroup][r] = GROUPED ? fmaf(acc[r], sc, t) : t + acc[r];
+        }
+      }
     }
   }
 
-  __device__ inline void run(const uint8_t* codes, const uint16_t* bias, void* out, float* red) {
+  __device__ inline void compute_unit(const Unit& d) {
+    f32x4 cc[kNA][MT];
+#pragma unroll
+    for (int a = 0; a < kNA; ++a)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) cc[a][mt] = cancel_term(d.av[a][mt]);
+#pragma unroll
+    for (int s = 0; s < kU; ++s) {
+      const u32x4 t = d.wv[s / kSPT];
+      const uint32_t w[4] = {t.x, t.y, t.z, t.w};
+      const float sc = GROUPED ? to_f32<DT>(d.sraw[s / 2]) : 1.0f;
+      step_mfma(w + (s % kSPT) * kDw, d.av[s / kS], cc[s / kS], s % kS, sc);
+    }
+  }
+
+  __device__ inline void run(const uint8_t* codes, const uint16_t* bias, void* out, int out_f32,
+                             float* red) {
     lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     j = lane & 15;
     kb = lane >> 4;
-    const int64_t tn = blockIdx.x;
+    const int tn = blockIdx.x;
     n = tn * kStripCols + j;
-    const uint8_t* strip = codes + tn * strip_bytes(K, BITS);
-    const int ntile = static_cast<int>(K / kTileK);
-    const int t0 = static_cast<int>(static_cast<int64_t>(ntile) * wave / WK);
-    const int t1 = static_cast<int>(static_cast<int64_t>(ntile) * (wave + 1) / WK);
-    const bool grouped = group_size > 0;
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) tot[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    const u32x4* tp = reinterpret_cast<const u32x4*>(strip) + lane;
-    int t = t0;
-    for (; t + kUnroll <= t1; t += kUnroll) {
-      u32x4 wv[kUnroll];
-      u32x4 av[kUnroll][kSubs][2][MT];
-      float sv[kUnroll][kSubs];
-#pragma unroll
-      for (int u = 0; u < kUnroll; ++u) wv[u] = tp[static_cast<int64_t>(t + u) * 64];
-#pragma unroll
-      for (int u = 0; u < kUnroll; ++u) {
-#pragma unroll
-        for (int sb = 0; sb < kSubs; ++sb) {
-          const int64_t k = static_cast<int64_t>(t + u) * kTileK + sb * 64;
-          sv[u][sb] = grouped ? load_scale(k) : 1.0f;
-#pragma unroll
-          for (int st = 0; st < 2; ++st)
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) av[u][sb][st][mt] = load_a(mt, k + 32 * st);
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < kUnroll; ++u) {
-        const uint32_t w[4] = {wv[u].x, wv[u].y, wv[u].z, wv[u].w};
-#pragma unroll
-        for (int sb = 0; sb < kSubs; ++sb) sub_block(w + 2 * kDwPerStep * sb, av[u][sb], sv[u][sb]);
-      }
-    }
-    for (; t < t1; ++t) {
-      const u32x4 wv = tp[static_cast<int64_t>(t) * 64];
-      const uint32_t w[4] = {wv.x, wv.y, wv.z, wv.w};
-#pragma unroll
-      for (int sb = 0; sb < kSubs; ++sb) {
-        const int64_t k = static_cast<int64_t>(t) * kTileK + sb * 64;
-        u32x4 a[2][MT];
-#pragma unroll
-        for (int st = 0; st < 2; ++st)
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt) a[st][mt] = load_a(mt, k + 32 * st);
-        sub_block(w + 2 * kDwPerStep * sb, a, grouped ? load_scale(k) : 1.0f);
-      }
-    }
-    if (BITS == 4 && (K % 128) != 0 && wave == WK - 1) {
-      // half tile at the end of the strip: 8 bytes per lane, 64 k
-      const int64_t k = static_cast<int64_t>(ntile) * 128;
-      const u32x2 wv = *reinterpret_cast<const u32x2*>(strip + static_cast<int64_t>(ntile) * 1024 + lane * 8);
-      const uint32_t w[2] = {wv.x, wv.y};
-      u32x4 a[2][MT];
-#pragma unroll
-      for (int st = 0; st < 2; ++st)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) a[st][mt] = load_a(mt, k + 32 * st);
-      sub_block(w, a, grouped ? load_scale(k) : 1.0f);
-    }
-
-    // Meet in LDS: red[wave][mt][r][lane], summed in wave order.
+    const uint8_t* strip = codes + static_cast<int64_t>(tn) * strip_bytes(K, BITS);
+    magic = Dequant<DT, BITS>::kMagic;
+    asm volatile("" : "+v"(magic));  // keep the constant in a VGPR
+    const int nsteps = K / 32;
+    const int nunits = nsteps / kU;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) red[((wave * MT + mt) * 4 + r) * 64 + lane] = tot[mt][r];
+      for (int c = 0; c < kClasses; ++c) totc[mt][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const u32x4* tp = reinterpret_cast<const u32x4*>(strip) + lane;
+    if (NU > 0) {
+      Unit d[NU > 0 ? NU : 1];
+#pragma unroll
+      for (int i = 0; i < NU; ++i) load_unit(d[i], tp, wave * NU + i);
+#pragma unroll
+      for (int i = 0; i < NU; ++i) compute_unit(d[i]);
+    } else {
+      const int u0 = nunits * wave / WK, u1 = nunits * (wave + 1) / WK;
+      if (u0 < u1) {
+        Unit d0, d1;
+        int u = u0;
+        load_unit(d0, tp, u);
+        while (true) {
+          if (u + 1 < u1) load_unit(d1, tp, u + 1);
+          compute_unit(d0);
+          if (++u >= u1) break;
+          if (u + 1 < u1) load_unit(d0, tp, u + 1);
+          compute_unit(d1);
+          if (++u >= u1) break;
+        }
+      }
+      if (wave == WK - 1) {
+        // k steps past the last whole unit, two at a time (64 k): 8 bytes of
+        // codes per lane (int4, including the half tile that ends a K that is
+        // 64 mod 128) or one whole tile (int8).  Every row group carries the
+        // same step, row group 0 is kept.
+        for (int step = nunits * kU; step < nsteps; step += 2) {
+          uint32_t w[4];
+          if (BITS == 8) {
+            const u32x4 t = tp[(step / 2) * 64];
+            w[0] = t.x; w[1] = t.y; w[2] = t.z; w[3] = t.w;
+          } else {
+            const int tile = step / 4, nfull = K / 128;
+            const uint8_t* p = tile < nfull ? strip + tile * 1024 + lane * 16 + (step % 4) * 4
+                                            : strip + nfull * 1024 + lane * 8;
+            const u32x2 t = *reinterpret_cast<const u32x2*>(p);
+            w[0] = t.x; w[1] = t.y; w[2] = 0; w[3] = 0;
+          }
+          const float sc = GROUPED ? to_f32<DT>(load_scale_raw(step)) : 1.0f;
+#pragma unroll
+          for (int st = 0; st < 2; ++st) {
+            u32x4 a[MT];
+            f32x4 cc[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+              a[mt] = load_a(mt, step + st, false);
+              cc[mt] = cancel_term(a[mt]);
+            }
+            step_mfma(w + st * kDw, a, cc, 0, sc);
+          }
+        }
+      }
+    }
+
+    // Merge the classes: every lane keeps the class of its own lane group.
+    f32x4 tot[MT];
+    {
+      const int mine = MP == 8 ? (kb >> 1) : kb;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        tot[mt] = totc[mt][0];
+#pragma unroll
+        for (int c = 1; c < kClasses; ++c)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) tot[mt][r] = mine == c ? totc[mt][c][r] : tot[mt][r];
+      }
+    }
+    // Fold the kS row groups that carried the same output row: registers
+    // first (MP < 4 keeps several row groups in one lane), then across the
+    // lane groups.  Afterwards rows 0 .. MP-1 hold the wavefront's sums.
+    if (MP == 1) {
+      tot[0][0] = (tot[0][0] + tot[0][1]) + (tot[0][2] + tot[0][3]);
+    } else if (MP == 2) {
+      tot[0][0] += tot[0][2];
+      tot[0][1] += tot[0][3];
+    }
+    if (MP <= 8) {
+#pragma unroll
+      for (int r = 0; r < kLive; ++r) tot[0][r] = sum_lane_groups(tot[0][r], MP <= 4, true);
+    }
+    // Meet in LDS: red[wave][mt][r][lane], summed over wavefronts in order.
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int r = 0; r < kLive; ++r) red[((wave * MT + mt) * 4 + r) * 64 + lane] = tot[mt][r];
     __syncthreads();
-    for (int idx = threadIdx.x; idx < MT * 256; idx += WK * 64) {
-      const int mt = idx / 256, r = (idx % 256) / 64, l = idx % 64;
+    const int rows = M < 16 * MT ? M : 16 * MT;
+    for (int idx = threadIdx.x; idx < rows * 16; idx += WK * 64) {
+      const int m = idx / 16, nl = idx % 16;
+      const int mt = m / 16, row = m % 16;
       float s = 0.0f;
 #pragma unroll
-      for (int w = 0; w < WK; ++w) s += red[((w * MT + mt) * 4 + r) * 64 + l];
-      const int m = mt * 16 + (l / 16) * 4 + r;
-      const int64_t nn = tn * kStripCols + (l % 16);
-      if (m < M) {
-        if (!grouped) s *= to_f32<DT>(scale[nn]);
-        if (bias != nullptr) s += to_f32<DT>(bias[nn]);
-        if (out_f32)
-          static_cast<float*>(out)[static_cast<int64_t>(m) * N + nn] = s;
-        else
-          static_cast<uint16_t*>(out)[static_cast<int64_t>(m) * N + nn] = from_f32_rne<DT>(s);
-      }
+      for (int w = 0; w < WK; ++w)
+        s += red[((w * MT + mt) * 4 + (row % 4)) * 64 + (row / 4) * 16 + nl];
+      const int nn = tn * kStripCols + nl;
+      if (!GROUPED) s *= to_f32<DT>(scale[nn]);
+      if (bias != nullptr) s += to_f32<DT>(bias[nn]);
+      if (out_f32)
+        static_cast<float*>(out)[static_cast<int64_t>(m) * N + nn] = s;
+      else
+        static_cast<uint16_t*>(out)[static_cast<int64_t>(m) * N + nn] = from_f32_rne<DT>(s);
     }
   }
 };
 
-template <int DT, int BITS, int MT, int WK>
+template <int DT, int BITS, int MP, int MT, int WK, int NU, bool GROUPED>
 __global__ __launch_bounds__(WK * 64) void stream_kernel(
     const uint16_t* __restrict__ x, const uint8_t* __restrict__ codes,
     const uint16_t* __restrict__ bias, const uint16_t* __restrict__ scale, void* __restrict__ out,
-    int M, int64_t K, int64_t N, int group_size, int out_f32) {
+    int M, int K, int N, int gshift, int out_f32) {
   extern __shared__ float red[];
-  StreamKernel<DT, BITS, MT, WK> k;
+  StreamKernel<DT, BITS, MP, MT, WK, NU, GROUPED> k;
   k.x = x;
   k.scale = scale;
   k.M = M;
   k.K = K;
   k.N = N;
-  k.group_size = group_size;
-  k.out_f32 = out_f32;
-  k.run(codes, bias, out, red);
+  k.gshift = gshift;
+  k.run(codes, bias, out, out_f32, red);
 }
 
 struct Args {
   const void* x; const void* codes; const void* bias; const void* scale; void* out;
-  int M; int64_t K, N; int group_size; int out_f32; hipStream_t stream;
+  int M, K, N, gshift, out_f32; hipStream_t stream;
 };
 
-template <int DT, int BITS, int MT, int WK>
+template <int DT, int BITS, int MP, int MT, int WK, int NU>
 void launch_one(const Args& a) {
   const size_t lds = static_cast<size_t>(WK) * MT * 256 * sizeof(float);
-  stream_kernel<DT, BITS, MT, WK>
-      <<<dim3(static_cast<unsigned>(a.N / kStripCols)), dim3(WK * 64), lds, a.stream>>>(
-          static_cast<const uint16_t*>(a.x), static_cast<const uint8_t*>(a.codes),
-          static_cast<const uint16_t*>(a.bias), static_cast<const uint16_t*>(a.scale), a.out, a.M,
-          a.K, a.N, a.group_size, a.out_f32);
+  const dim3 grid(static_cast<unsigned>(a.N / kStripCols)), block(WK * 64);
+  const uint16_t* x = static_cast<const uint16_t*>(a.x);
+  const uint8_t* codes = static_cast<const uint8_t*>(a.codes);
+  const uint16_t* bias = static_cast<const uint16_t*>(a.bias);
+  const uint16_t* scale = static_cast<const uint16_t*>(a.scale);
+  if (a.gshift >= 0)
+    stream_kernel<DT, BITS, MP, MT, WK, NU, true><<<grid, block, lds, a.stream>>>(
+        x, codes, bias, scale, a.out, a.M, a.K, a.N, a.gshift, a.out_f32);
+  else
+    stream_kernel<DT, BITS, MP, MT, WK, NU, false><<<grid, block, lds, a.stream>>>(
+        x, codes, bias, scale, a.out, a.M, a.K, a.N, a.gshift, a.out_f32);
 }
 
-template <int DT, int BITS, int MT>
-void launch_wk(const Args& a, int wk) {
-  if (wk >= 16 && MT <= 2) launch_one<DT, BITS, MT, (MT <= 2 ? 16 : 8)>(a);
-  else if (wk >= 8) launch_one<DT, BITS, MT, 8>(a);
-  else if (wk >= 4) launch_one<DT, BITS, MT, 4>(a);
-  else if (wk >= 2) launch_one<DT, BITS, MT, 2>(a);
-  else launch_one<DT, BITS, MT, 1>(a);
+// wk in {1,2,4,8,16}; nu == 1 selects the all-loads-at-once variant (exactly
+// one unit per wavefront), anything else the walking variant.
+template <int DT, int BITS, int MP, int MT>
+void launch_wk(const Args& a, int wk, int nu) {
+  constexpr int kMaxWk = MT <= 2 ? 16 : 8;  // LDS for the cross-wavefront sums
+  if (nu == 1) {
+    if (wk >= 16 && kMaxWk == 16) launch_one<DT, BITS, MP, MT, kMaxWk, 1>(a);
+    else if (wk >= 8) launch_one<DT, BITS, MP, MT, 8, 1>(a);
+    else if (wk >= 4) launch_one<DT, BITS, MP, MT, 4, 1>(a);
+    else if (wk >= 2) launch_one<DT, BITS, MP, MT, 2, 1>(a);
+    else launch_one<DT, BITS, MP, MT, 1, 1>(a);
+  } else {
+    if (wk >= 16 && kMaxWk == 16) launch_one<DT, BITS, MP, MT, kMaxWk, 0>(a);
+    else if (wk >= 8) launch_one<DT, BITS, MP, MT, 8, 0>(a);
+    else if (wk >= 4) launch_one<DT, BITS, MP, MT, 4, 0>(a);
+    else if (wk >= 2) launch_one<DT, BITS, MP, MT, 2, 0>(a);
+    else launch_one<DT, BITS, MP, MT, 1, 0>(a);
+  }
 }
 
 template <int DT, int BITS>
-void launch_mt(const Args& a, int wk) {
-  const int mt = (a.M + 15) / 16;
-  if (mt <= 1) launch_wk<DT, BITS, 1>(a, wk);
-  else if (mt == 2) launch_wk<DT, BITS, 2>(a, wk);
-  else if (mt == 3) launch_wk<DT, BITS, 3>(a, wk);
-  else launch_wk<DT, BITS, 4>(a, wk);
-}
-
-template <int DT>
-void launch_bits(const Args& a, int bits, int wk) {
-  if (bits == 8) launch_mt<DT, 8>(a, wk);
-  else launch_mt<DT, 4>(a, wk);
+void launch_m(const Args& a, int wk, int nu) {
+  if (a.M <= 1) launch_wk<DT, BITS, 1, 1>(a, wk, nu);
+  else if (a.M <= 2) launch_wk<DT, BITS, 2, 1>(a, wk, nu);
+  else if (a.M <= 4) launch_wk<DT, BITS, 4, 1>(a, wk, nu);
+  else if (a.M <= 8) launch_wk<DT, BITS, 8, 1>(a, wk, nu);
+  else if (a.M <= 16) launch_wk<DT, BITS, 16, 1>(a, wk, nu);
+  else if (a.M <= 32) launch_wk<DT, BITS, 16, 2>(a, wk, nu);
+  else if (a.M <= 48) launch_wk<DT, BITS, 16, 3>(a, wk, nu);
+  else launch_wk<DT, BITS, 16, 4>(a, wk, nu);
 }
 
 }  // namespace
 
-// Wavefronts per workgroup: enough to put ~5 wavefronts on each of the 1024
-// SIMDs, but no more than there are tiles along K.
-static int pick_wk(int64_t K, int64_t N, int bits) {
+// Work split.  A unit is kU k steps of one strip.  When the problem is small
+// enough that one unit per wavefront keeps every wavefront resident at once
+// (at most ~6 per SIMD on 1024 SIMDs) and the unit count per strip is a power
+// of two up to 16, each wavefront takes exactly one unit and loads it at once.
+// Otherwise wavefronts walk several units with two in flight, and WK aims at
+// about four wavefronts per SIMD.
+static void pick_split(int64_t M, int64_t K, int64_t N, int bits, int* wk, int* nu) {
   const int64_t strips = N / kStripCols;
-  const int64_t ntile = K / (bits == 8 ? 64 : 128);
-  int wk = 1;
-  while (wk < 16 && strips * wk * 2 <= 6144 && wk * 2 <= ntile) wk *= 2;
-  return wk;
+  int mp = 1;
+  while (mp < 16 && mp < M) mp *= 2;
+  const int s = 16 / mp, spt = bits == 8 ? 2 : 4;
+  const int ku = s > spt ? s : spt;
+  const int64_t nsteps = K / 32, nunits = nsteps / ku;
+  const int maxwk = M <= 32 ? 16 : 8;
+  if (nunits * ku == nsteps && nunits <= maxwk && (nunits & (nunits - 1)) == 0 &&
+      strips * nunits <= 6144) {
+    *wk = static_cast<int>(nunits);
+    *nu = 1;
+    return;
+  }
+  int w = 1;
+  while (w < maxwk && strips * w * 2 <= 4096 && w * 4 <= nunits) w *= 2;
+  *wk = w;
+  *nu = 0;
 }
 
 int launch_linear_stream(const void* x, const void* codes, const void* bias, const void* scale,
                          int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
                          void* out, bool out_f32, hipStream_t stream) {
-  const Args a{x, codes, bias, scale, out, static_cast<int>(M), K, N, group_size, out_f32 ? 1 : 0, stream};
-  const int wk = pick_wk(K, N, bits);
-  if (dtype == WOL_DTYPE_BF16) launch_bits<WOL_DTYPE_BF16>(a, bits, wk);
-  else launch_bits<WOL_DTYPE_F16>(a, bits, wk);
+  const int gshift = group_size == 64 ? 6 : (group_size == 128 ? 7 : -1);
+  const Args a{x, codes, bias, scale, out, static_cast<int>(M), static_cast<int>(K),
+               static_cast<int>(N), gshift, out_f32 ? 1 : 0, stream};
+  int wk = 1, nu = 0;
+  pick_split(M, K, N, bits, &wk, &nu);
+  if (dtype == WOL_DTYPE_BF16) {
+    if (bits == 8) launch_m<WOL_DTYPE_BF16, 8>(a, wk, nu); else launch_m<WOL_DTYPE_BF16, 4>(a, wk, nu);
+  } else {
+    if (bits == 8) launch_m<WOL_DTYPE_F16, 8>(a, wk, nu); else launch_m<WOL_DTYPE_F16, 4>(a, wk, nu);
+  }
   return check_launch();
 }
 

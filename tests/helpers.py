@@ -9,9 +9,21 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-from oracle import wo_oracle as O  # noqa: E402  (the checker; tests only)
 
-F16, BF16 = O.F16, O.BF16
+
+class _LazyOracle:
+    """The CPU oracle (the checker), imported on first use so that code which
+    only wants the data generators does not load it."""
+
+    def __getattr__(self, name):
+        from oracle import wo_oracle
+
+        return getattr(wo_oracle, name)
+
+
+O = _LazyOracle()
+
+F16, BF16 = 0, 1
 DT_NAMES = {F16: "float16", BF16: "bfloat16"}
 
 
