@@ -130,6 +130,9 @@ def main():
     ap.add_argument("--prefill-steps", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--eager", action="store_true", help="time eager launches instead of a graph")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three 256 MiB device copies (a known-size kernel to scale "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings with)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (the path has no collectives); "
@@ -147,6 +150,14 @@ def main():
         sys.exit(3)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.copy_calibration:
+        src = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---------------- decode (the headline metric) ----------------
     c = DECODE

@@ -1,0 +1,60 @@
+"""Thin wrappers that call the C ABI (through paddle_amd._lib) on torch device
+memory, for the GPU parity tests."""
+import numpy as np
+import torch
+
+import helpers as H
+from paddle_amd import _lib
+
+DEV = "cuda:0"
+
+
+def quantize(w_bits, dt, bits, g, layout=_lib.LAYOUT_GFX950, round_mode=_lib.ROUND_RNE):
+    """Returns (codes as flat uint8 numpy, scale bits numpy) from wol_quantize."""
+    w = H.bits_to_torch(w_bits, dt, DEV)
+    K, N = w.shape
+    codes = torch.full((K * N * bits // 8,), 0x55, dtype=torch.uint8, device=DEV)
+    sshape = (N,) if g == -1 else ((K + g - 1) // g, N)
+    scale = torch.zeros(sshape, dtype=w.dtype, device=DEV)
+    wsb = _lib.lib.wol_quantize_workspace(K, N, bits, g)
+    ws = torch.full((max(wsb, 16),), 0xAB, dtype=torch.uint8, device=DEV)  # dirty on purpose
+    _lib.check(_lib.lib.wol_quantize(w.data_ptr(), dt, K, N, bits, g, round_mode, layout, codes.data_ptr(),
+                                     scale.data_ptr(), ws.data_ptr(), wsb, None))
+    torch.cuda.synchronize()
+    return codes.cpu().numpy(), H.torch_to_bits(scale)
+
+
+def dequantize(codes_u8, layout, scale_bits, dt, K, N, bits, g):
+    c = torch.from_numpy(np.ascontiguousarray(codes_u8)).to(DEV)
+    s = H.bits_to_torch(scale_bits, dt, DEV)
+    out = torch.zeros((K, N), dtype=s.dtype, device=DEV)
+    _lib.check(_lib.lib.wol_dequantize(c.data_ptr(), layout, s.data_ptr(), dt, K, N, bits, g, out.data_ptr(), None))
+    torch.cuda.synchronize()
+    return H.torch_to_bits(out)
+
+
+def repack(codes_u8, layout_in, layout_out, K, N, bits):
+    c = torch.from_numpy(np.ascontiguousarray(codes_u8)).to(DEV)
+    o = torch.full_like(c, 0x33)
+    _lib.check(_lib.lib.wol_repack(c.data_ptr(), layout_in, o.data_ptr(), layout_out, K, N, bits, None))
+    torch.cuda.synchronize()
+    return o.cpu().numpy()
+
+
+def linear(x_bits, codes_u8, bias_bits, scale_bits, dt, N, bits, g, f32=False):
+    """codes_u8 in gfx950 layout.  Returns fp32 numpy [M,N] (f32=True) or T bits."""
+    x = H.bits_to_torch(x_bits, dt, DEV)
+    M, K = x.shape
+    c = torch.from_numpy(np.ascontiguousarray(codes_u8)).to(DEV)
+    s = H.bits_to_torch(scale_bits, dt, DEV)
+    b = None if bias_bits is None else H.bits_to_torch(bias_bits, dt, DEV)
+    if f32:
+        out = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
+        fn = _lib.lib.wol_linear_f32
+    else:
+        out = torch.full((M, N), float("nan"), dtype=x.dtype, device=DEV)
+        fn = _lib.lib.wol_linear
+    _lib.check(fn(x.data_ptr(), c.data_ptr(), None if b is None else b.data_ptr(), s.data_ptr(), dt, M, K, N, bits, g,
+                  out.data_ptr(), None, 0, None))
+    torch.cuda.synchronize()
+    return out.cpu().numpy() if f32 else H.torch_to_bits(out)

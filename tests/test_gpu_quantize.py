@@ -1,0 +1,122 @@
+"""GPU parity of weight_quantize / weight_dequantize / repack against the CPU
+oracle, through the C ABI.  Codes and scales must be bit-exact."""
+import numpy as np
+import pytest
+
+import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(64, 16), (64, 256), (128, 288), (192, 48), (320, 1040), (512, 1024)]
+
+
+@pytest.fixture(scope="module")
+def G(device):
+    import gpu_calls
+
+    return gpu_calls
+
+
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("g", [-1, 64, 128])
+def test_quantize_bit_exact_all_layouts(G, oracle, dt, bits, g):
+    for K, N in SHAPES:
+        for adv in (False, True):
+            print("case", dt, bits, g, K, N, adv, flush=True)
+            wb = H.adversarial_weight(K, N, dt) if adv else H.make_weight(K, N, dt, seed=K + N)
+            oc, osc = oracle.weight_quantize(wb, dt, bits, g)
+            q = H.q_from_canonical(oc, bits)
+            gc, gs = G.quantize(wb, dt, bits, g, layout=0)
+            assert np.array_equal(gs, osc)
+            assert np.array_equal(gc.view(np.int8).reshape(oc.shape), oc)
+            gp, gs2 = G.quantize(wb, dt, bits, g, layout=2)
+            assert np.array_equal(gs2, osc)
+            assert np.array_equal(gp, H.gfx950_from_q(q, bits))
+            gh, _ = G.quantize(wb, dt, bits, g, layout=1)
+            assert np.array_equal(gh, H.paddle_hip_from_q(q, bits).view(np.uint8).reshape(-1))
+
+
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+@pytest.mark.parametrize("bits", [8, 4])
+def test_quantize_truncating_scale_flavour(G, oracle, dt, bits):
+    K, N = 256, 128
+    for g in (-1, 128):
+        for wb in (H.make_weight(K, N, dt, seed=3), H.adversarial_weight(K, N, dt)):
+            oc, osc = oracle.weight_quantize(wb, dt, bits, g, cast_mode=oracle.CAST_TRUNC)
+            gc, gs = G.quantize(wb, dt, bits, g, layout=0, round_mode=1)
+            assert np.array_equal(gs, osc)
+            assert np.array_equal(gc.view(np.int8).reshape(oc.shape), oc)
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+def test_quantize_nan_and_inf_inputs(G, oracle, bits):
+    # NaN never wins a maximum (unless it is the first element of a per-channel
+    # column); infinities give an infinite scale and zero / NaN quotients.
+    dt = H.BF16
+    K, N = 128, 32
+    wb = H.make_weight(K, N, dt, seed=17)
+    wb[5, 2] = 0x7FC0   # NaN inside a column
+    wb[0, 3] = 0x7FC0   # NaN as first element
+    wb[70, 4] = 0x7F80  # +inf
+    wb[9, 5] = 0xFF80   # -inf
+    for g in (-1, 64):
+        oc, osc = oracle.weight_quantize(wb, dt, bits, g)
+        gc, gs = G.quantize(wb, dt, bits, g, layout=0)
+        assert np.array_equal(gs, osc)
+        assert np.array_equal(gc.view(np.int8).reshape(oc.shape), oc)
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+def test_repack_round_trips(G, bits):
+    rng = np.random.default_rng(bits)
+    bound = 127 if bits == 8 else 7
+    for K, N in [(64, 16), (192, 48), (320, 1040)]:
+        q = rng.integers(-bound, bound + 1, (K, N)).astype(np.int32)
+        forms = {0: H.canonical_from_q(q, bits).view(np.uint8).reshape(-1),
+                 1: H.paddle_hip_from_q(q, bits).view(np.uint8).reshape(-1),
+                 2: H.gfx950_from_q(q, bits)}
+        for a in (0, 1, 2):
+            for b in (0, 1, 2):
+                got = G.repack(forms[a], a, b, K, N, bits)
+                assert np.array_equal(got, forms[b]), (K, N, a, b)
+
+
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("g", [-1, 64, 128])
+def test_dequantize_bit_exact(G, oracle, dt, bits, g):
+    for K, N in SHAPES:
+        wb = H.make_weight(K, N, dt, seed=K + 3 * N)
+        oc, osc = oracle.weight_quantize(wb, dt, bits, g)
+        _, oT = oracle.dequantize(oc, osc, dt, bits, g)
+        q = H.q_from_canonical(oc, bits)
+        for layout, codes in ((0, oc.view(np.uint8).reshape(-1)), (1, H.paddle_hip_from_q(q, bits).view(np.uint8).reshape(-1)),
+                              (2, H.gfx950_from_q(q, bits))):
+            got = G.dequantize(codes, layout, osc, dt, K, N, bits, g)
+            assert np.array_equal(got, oT), (K, N, layout)
+
+
+def test_quantize_dequantize_round_trip_full_size(G):
+    # the reference's own round-trip check (test_weight_only_linear.py:675-706)
+    # at its size, 4096 x 12288: |dequant(quant(w)) - w| <= scale / 2 everywhere
+    import torch
+
+    from paddle_amd.nn import quant as Q
+
+    for dt, tdt in ((H.F16, torch.float16), (H.BF16, torch.bfloat16)):
+        gen = torch.Generator(device="cuda").manual_seed(5)
+        w = (torch.randn(4096, 12288, device="cuda", generator=gen) * 0.02).to(tdt)
+        for algo, bound, g in (("weight_only_int8", 127, -1), ("weight_only_int4", 7, 128)):
+            codes, scale = Q.weight_quantize(w, algo=algo, group_size=g)
+            back = Q.weight_dequantize(codes, scale, algo=algo, out_dtype=DT_NAME[dt], group_size=g)
+            s_full = scale.float() if g == -1 else scale.float().repeat_interleave(g, dim=0)
+            err = (back.float() - w.float()).abs()
+            # half a quantisation step plus the rounding of the product to T
+            rel = 2.0**-8 if dt == H.BF16 else 2.0**-11
+            assert bool((err <= s_full * 0.5 * (1 + 2**-7) + back.float().abs() * rel).all())
+            amax = w.float().abs().amax(dim=0) if g == -1 else w.float().abs().view(-1, g, 12288).amax(dim=1)
+            assert torch.allclose(scale.float() * bound, amax, rtol=rel * 1.01, atol=0)
+
+
+DT_NAME = {H.F16: "float16", H.BF16: "bfloat16"}

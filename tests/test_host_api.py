@@ -1,0 +1,176 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports what
+include/wol_c_api.h declares, argument errors come back as statuses before any
+device work, the layout index helper is a bijection that agrees with the
+numpy statement of the layout, and the Python mirror reproduces the
+reference's shape contract and error behaviour."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+import helpers as H
+
+ROOT = H.ROOT
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from paddle_amd import _lib
+
+    return _lib
+
+
+def test_library_exports_every_declared_symbol(lib):
+    hdr = open(os.path.join(ROOT, "include", "wol_c_api.h")).read()
+    declared = set(re.findall(r"\b(wol_[a-z0-9_]+)\s*\(", hdr))
+    declared -= {"wol_status"}
+    assert declared == set(lib.SYMBOLS), declared ^ set(lib.SYMBOLS)
+    raw = ctypes.CDLL(lib.LIB_PATH)
+    for name in declared:
+        assert hasattr(raw, name), name
+
+
+def test_status_strings_and_version(lib):
+    L = lib.lib
+    assert L.wol_layout_version() == 1
+    assert L.wol_status_str(0) == b"ok"
+    seen = {L.wol_status_str(i) for i in range(0, 12)}
+    assert len(seen) == 12
+    assert L.wol_status_str(99) == b"unknown status"
+
+
+def test_workspace_queries(lib):
+    L = lib.lib
+    assert L.wol_quantize_workspace(4096, 11008, 4, -1) == 4 * 11008
+    assert L.wol_quantize_workspace(4096, 11008, 4, 128) == 0
+    assert L.wol_quantize_workspace(4095, 11008, 4, 128) == 0  # invalid shape
+    assert L.wol_linear_workspace(1, 4096, 11008, 4, 128) == 0
+
+
+def test_argument_errors_return_before_device_work(lib):
+    L = lib.lib
+    p = ctypes.c_void_p(0x1000)  # never dereferenced: every call fails validation first
+    q = lambda **kw: L.wol_quantize(kw.get("w", p), kw.get("dt", 0), kw.get("K", 64), kw.get("N", 16), kw.get("bits", 8),
+                                    kw.get("g", 64), kw.get("rm", 0), kw.get("layout", 2), p, p, None, 0, None)
+    assert q(dt=2) == 2
+    assert q(bits=5) == 3
+    assert q(g=32) == 4
+    assert q(K=32) == 5 and q(N=8) == 5 and q(K=0) == 5
+    assert q(layout=7) == 6
+    assert q(rm=3) == 7
+    assert q(w=None) == 1
+    assert q(w=ctypes.c_void_p(0x1008)) == 9
+    assert q(g=-1) == 8  # per-channel needs the abs-max workspace
+    lin = lambda **kw: L.wol_linear(kw.get("x", p), p, None, p, kw.get("dt", 1), kw.get("M", 1), kw.get("K", 64),
+                                    kw.get("N", 16), kw.get("bits", 4), kw.get("g", -1), p, None, 0, None)
+    assert lin(dt=5) == 2 and lin(bits=2) == 3 and lin(g=100) == 4 and lin(K=100) == 5 and lin(M=-1) == 5
+    assert lin(x=None) == 1
+    assert lin(M=0) == 0  # empty batch is a no-op
+    assert L.wol_dequantize(p, 9, p, 0, 64, 16, 8, -1, p, None) == 6
+    assert L.wol_repack(p, 0, p, 2, 64, 16, 8, None) == 6  # in-place is refused
+    assert L.wol_repack(p, 0, ctypes.c_void_p(0x2000), 2, 64, 24, 8, None) == 5
+    with pytest.raises(ValueError, match="InvalidArgument"):
+        lib.check(5)
+    with pytest.raises(lib.WolError):
+        lib.check(10)
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("K", [64, 128, 192, 320])
+def test_code_offset_is_a_bijection_matching_the_layout(lib, bits, K):
+    L = lib.lib
+    N = 48
+    rng = np.random.default_rng(K + bits)
+    bound = 127 if bits == 8 else 7
+    q = rng.integers(-bound, bound + 1, (K, N)).astype(np.int32)
+    want = {0: H.canonical_from_q(q, bits).view(np.uint8).reshape(-1),
+            1: H.paddle_hip_from_q(q, bits).view(np.uint8).reshape(-1),
+            2: H.gfx950_from_q(q, bits)}
+    for layout in (0, 1, 2):
+        buf = np.zeros(K * N * bits // 8, np.uint8)
+        hits = np.zeros(K * N * bits // 8 * (2 if bits == 4 else 1), np.int32)
+        sh = ctypes.c_int(0)
+        for k in range(K):
+            for n in range(N):
+                off = L.wol_code_offset(layout, K, N, bits, k, n, ctypes.byref(sh))
+                assert 0 <= off < buf.size
+                if bits == 8:
+                    v = (q[k, n] + 128) & 0xFF if layout == 2 else q[k, n] & 0xFF
+                    buf[off] = v
+                    hits[off] += 1
+                else:
+                    v = (q[k, n] & 0xF) if layout == 0 else (q[k, n] + 8) & 0xF
+                    buf[off] |= v << sh.value
+                    hits[2 * off + sh.value // 4] += 1
+        assert (hits == 1).all()  # every slot written exactly once: a permutation
+        assert np.array_equal(buf, want[layout]), layout
+    assert L.wol_code_offset(2, K, N, bits, K, 0, None) == -1
+    assert L.wol_code_offset(2, K, N, bits, 0, -1, None) == -1
+
+
+def test_strip_slices_are_self_contained(lib):
+    # a slice of the gfx950 tensor along N at a multiple of 16 is the gfx950
+    # tensor of the sliced weight (what column-parallel sharding relies on)
+    rng = np.random.default_rng(1)
+    for bits in (8, 4):
+        bound = 127 if bits == 8 else 7
+        q = rng.integers(-bound, bound + 1, (192, 64)).astype(np.int32)
+        full = H.gfx950_from_q(q, bits)
+        per_strip = 16 * 192 * bits // 8
+        assert np.array_equal(full[per_strip:3 * per_strip], H.gfx950_from_q(q[:, 16:48], bits))
+
+
+# ------------------------------------------------------------ Python mirror
+def test_infer_meta_contracts():
+    from paddle_amd.nn.quant import quantized_linear as QL
+
+    assert QL.weight_quantize_infer_meta((4096, 11008), "weight_only_int8", -1) == ([11008, 4096], [11008])
+    assert QL.weight_quantize_infer_meta((4096, 11008), "weight_only_int4", 128) == ([5504, 4096], [32, 11008])
+    assert QL.weight_quantize_infer_meta((192, 32), "weight_only_int8", 128) == ([32, 192], [2, 32])
+    assert QL.weight_quantize_infer_meta((64, 16), "llm.int8", -1) == ([16, 64], [16])
+    for bad in (((64,), "weight_only_int8", -1), ((63, 16), "weight_only_int8", -1), ((64, 8), "weight_only_int8", -1),
+                ((64, 16), "weight_only_int8", 32), ((64, 16), "int8", -1)):
+        with pytest.raises(ValueError, match="InvalidArgument"):
+            QL.weight_quantize_infer_meta(*bad)
+    assert QL.weight_dequantize_infer_meta((256, 64), (256,), "weight_only_int8", -1) == [64, 256]
+    assert QL.weight_dequantize_infer_meta((128, 64), (1, 256), "weight_only_int4", 64) == [64, 256]
+    for bad in (((256, 64), (255,), "weight_only_int8", -1), ((256, 64), (256,), "llm.int8", -1),
+                ((256, 64), (1, 256), "weight_only_int8", -1), ((256, 64), (2, 256), "weight_only_int8", 64),
+                ((256, 64), (1, 128), "weight_only_int8", 64)):
+        with pytest.raises(ValueError, match="InvalidArgument"):
+            QL.weight_dequantize_infer_meta(*bad)
+    assert QL.weight_only_linear_infer_meta((2, 3, 64), (256, 64), (256,), (256,), "int8", -1) == ([2, 3, 256], 256)
+    assert QL.weight_only_linear_infer_meta((1, 128), (144, 128), None, (1, 288), "int4", 128) == ([1, 288], 288)
+    for bad in (((1, 64), (256, 64), None, (256,), "int2", -1), ((1, 64), (256, 64), None, (256,), "int8", 32),
+                ((1, 64), (24, 64), None, (48,), "int4", -1), ((1, 65), (256, 64), None, (256,), "int8", -1),
+                ((1, 64), (256, 64), (1, 256), (256,), "int8", -1), ((1, 64), (256, 64), None, (1, 256), "int8", -1),
+                ((1, 64), (256, 64), None, (256,), "int8", 64), ((1, 128), (256, 128), None, (1, 256), "int8", 64)):
+        with pytest.raises(ValueError, match="InvalidArgument"):
+            QL.weight_only_linear_infer_meta(*bad)
+
+
+def test_python_api_argument_checks():
+    import torch
+
+    from paddle_amd.nn import quant as Q
+
+    x = torch.zeros(64, 16, dtype=torch.float16)
+    with pytest.raises(AssertionError, match="group_size"):
+        Q.weight_quantize(x, group_size=32)
+    with pytest.raises(AssertionError, match="group_size"):
+        Q.weight_dequantize(torch.zeros(16, 64, dtype=torch.int8), torch.zeros(16), group_size=7)
+    with pytest.raises(AssertionError, match="group size"):
+        Q.weight_only_linear(x, torch.zeros(16, 16, dtype=torch.int8), weight_scale=torch.zeros(16), group_size=1)
+    with pytest.raises(ValueError, match="divisible by 64"):
+        Q.weight_quantize(torch.zeros(32, 16, dtype=torch.float16))
+    with pytest.raises(ValueError, match="float16 or bfloat16"):
+        Q.weight_quantize(torch.zeros(64, 16, dtype=torch.float32))
+    with pytest.raises(TypeError):
+        Q.weight_dequantize(torch.zeros(16, 64, dtype=torch.int8), torch.zeros(16), out_dtype="float32")
+    with pytest.raises(RuntimeError, match="GPU"):
+        Q.weight_quantize(x)  # CPU tensors: there is no CPU kernel to fall back to
+    assert Q.weight_quantize.__defaults__ == ("weight_only_int8", None, -1)
+    assert Q.weight_dequantize.__defaults__ == ("weight_only_int8", "float16", -1)
+    assert Q.weight_only_linear.__defaults__ == (None, None, "int8", None, -1)
