@@ -1,13 +1,18 @@
 // weight_only_linear for large M (prefill): an MFMA GEMM.
 //
-// A workgroup of four wavefronts (2 x 2) computes a BM x BN tile of the
-// output.  The activations of a k tile are staged in LDS (padded rows, read
-// back as 16x16x32 A fragments); the packed weights need no staging because
-// the GFX950 layout already stores them in B-fragment order: every lane loads
-// its 16 bytes for a strip straight from global memory and dequantises them in
-// registers to exact signed bf16/fp16 integers.  Scales are applied to fp32
-// accumulators -- in the epilogue (per-channel) or once per 64-k sub-block
-// (group-wise) -- so the product code*scale is never rounded to T.
+// A workgroup of WM x WN wavefronts computes a BM x BN tile of the output,
+// each wavefront a (16*TM) x (16*TN) sub-tile with v_mfma_f32_16x16x32.  The
+// activations of a k tile are staged in LDS (double buffered, padded rows,
+// read back as A fragments).  The packed weights need no staging: the GFX950
+// layout already stores them in B-fragment order, so every lane loads its 16
+// bytes per strip straight from global memory (prefetched one k tile ahead)
+// and dequantises them in registers to exact signed bf16/fp16 integers; the
+// cost of that is amortised over the TM row tiles of the wavefront.  Scales
+// are applied to fp32 accumulators -- in the epilogue (per-channel) or once
+// per 64-k sub-block (group-wise) -- so code*scale is never rounded to T.
+// The epilogue passes each 16-row slab through LDS so that rows leave as
+// 16-byte stores.  Workgroups are numbered so that each XCD (one L2 each)
+// works on a compact block of neighbouring tiles.
 #include "wol_common.h"
 
 namespace wol {
@@ -46,16 +51,17 @@ struct DequantExact;
 
 template <>
 struct DequantExact<WOL_DTYPE_BF16, 8> {
+  __device__ static inline float sbyte(uint32_t v, int i) {
+    return static_cast<float>(static_cast<int>(static_cast<int8_t>((v >> (8 * i)) & 0xFFu)));
+  }
   __device__ static inline u32x4 run(const uint32_t* w) {
+    // stored byte = code + 128; flipping the top bit gives the two's complement code
+    const uint32_t a = w[0] ^ 0x80808080u, b = w[1] ^ 0x80808080u;
     u32x4 o;
-    o.x = pack_bf16_hi(static_cast<float>(w[0] & 0xFFu) - 128.0f,
-                       static_cast<float>((w[0] >> 8) & 0xFFu) - 128.0f);
-    o.y = pack_bf16_hi(static_cast<float>((w[0] >> 16) & 0xFFu) - 128.0f,
-                       static_cast<float>(w[0] >> 24) - 128.0f);
-    o.z = pack_bf16_hi(static_cast<float>(w[1] & 0xFFu) - 128.0f,
-                       static_cast<float>((w[1] >> 8) & 0xFFu) - 128.0f);
-    o.w = pack_bf16_hi(static_cast<float>((w[1] >> 16) & 0xFFu) - 128.0f,
-                       static_cast<float>(w[1] >> 24) - 128.0f);
+    o.x = pack_bf16_hi(sbyte(a, 0), sbyte(a, 1));
+    o.y = pack_bf16_hi(sbyte(a, 2), sbyte(a, 3));
+    o.z = pack_bf16_hi(sbyte(b, 0), sbyte(b, 1));
+    o.w = pack_bf16_hi(sbyte(b, 2), sbyte(b, 3));
     return o;
   }
 };
@@ -104,143 +110,423 @@ struct DequantExact<WOL_DTYPE_BF16, 4> {
   }
 };
 
-constexpr int kThreads = 256;
+// Workgroup -> output tile.  Hardware deals consecutive workgroup ids to the
+// 8 XCDs in turn; give XCD x the ids that form a compact block of tiles so
+// that its L2 sees every A row block and B column block of that block once.
+__device__ inline void tile_of_block(int nbx, int nby, int* bx, int* by) {
+  const int id = blockIdx.x, total = nbx * nby;
+  constexpr int kXcd = 8;
+  int t = id;
+  if (total % kXcd == 0) {
+    const int per = total / kXcd;
+    t = (id % kXcd) * per + id / kXcd;
+  }
+  // walk the tiles in column-major panels of 8 row blocks so neighbours share B
+  *by = t % nby;
+  *bx = t / nby;
+}
 
-template <int DT, int BITS, bool GROUPED, int WMT, int WNT>
-__global__ __launch_bounds__(kThreads) void gemm_kernel(
+template <int DT, int BITS, bool GROUPED, int WM, int WN, int TM, int TN>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(
     const uint16_t* __restrict__ x, const uint8_t* __restrict__ codes,
     const uint16_t* __restrict__ bias, const uint16_t* __restrict__ scale, void* __restrict__ out,
-    int64_t M, int64_t K, int64_t N, int group_size, int out_f32) {
-  constexpr int BM = 32 * WMT, BN = 32 * WNT;
-  constexpr int TK = BITS == 8 ? 64 : 128;    // k per 16-byte lane load
-  constexpr int kDwPerStep = BITS == 8 ? 2 : 1;
-  constexpr int kRow = TK + 8;                // padded LDS row, in elements
-  __shared__ __attribute__((aligned(16))) uint16_t As[BM * kRow];
+    int M, int K, int N, int gshift, int out_f32, int nbx, int nby) {
+  constexpr int NT = 64 * WM * WN;
+  constexpr int BM = WM * TM * 16, BN = WN * TN * 16;
+  constexpr int TK = BITS == 8 ? 64 : 128;     // k per 16-byte lane load
+  constexpr int kDw = BITS == 8 ? 2 : 1;       // dwords per k step
+  constexpr int kRow = TK + 8;                 // padded LDS row, in elements
+  constexpr int kChunks = BM * (TK / 8) / NT;  // 16-byte pieces of the A tile per thread
+  static_assert(BM * (TK / 8) % NT == 0, "A tile must split evenly over the threads");
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];  // 2 x BM x kRow
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WN, wn = wave % WN;
   const int j = lane & 15, kb = lane >> 4;
-  const int64_t m0 = static_cast<int64_t>(blockIdx.y) * BM;
-  const int64_t strip0 = static_cast<int64_t>(blockIdx.x) * (BN / 16) + wn * WNT;
-  const int64_t nstrips = N / kStripCols;
+  int bx, by;
+  tile_of_block(nbx, nby, &bx, &by);
+  const int m0 = by * BM;
+  const int strip0 = bx * (BN / 16) + wn * TN;
+  const int nstrips = N / kStripCols;
 
-  f32x4 tot[WMT][WNT];
+  // this thread's pieces of the A tile: row r, 8 elements at column 8*cc
+  const uint16_t* aptr[kChunks];
+  int aoff[kChunks];
 #pragma unroll
-  for (int a = 0; a < WMT; ++a)
+  for (int c = 0; c < kChunks; ++c) {
+    const int id = tid + c * NT, r = id / (TK / 8), cc = id % (TK / 8);
+    int m = m0 + r;
+    m = m < M ? m : M - 1;  // rows past M are computed on valid data and never stored
+    aptr[c] = x + static_cast<int64_t>(m) * K + cc * 8;
+    aoff[c] = r * kRow + cc * 8;
+  }
+  // this lane's 16 bytes of every strip of the wavefront
+  const uint8_t* bptr[TN];
 #pragma unroll
-    for (int b = 0; b < WNT; ++b) tot[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < TN; ++s) {
+    const int st = strip0 + s < nstrips ? strip0 + s : nstrips - 1;  // past N: valid data, never stored
+    bptr[s] = codes + static_cast<int64_t>(st) * strip_bytes(K, BITS) + lane * 16;
+  }
 
-  const int64_t nfull = K / TK;
-  const int64_t niter = nfull + ((K % TK) ? 1 : 0);
-  for (int64_t it = 0; it < niter; ++it) {
-    const int64_t k0 = it * TK;
-    const int kw = static_cast<int>(K - k0 < TK ? K - k0 : TK);  // 128 or 64 (int4 tail)
-    __syncthreads();
-    // stage the activations of this k tile: BM rows of kw elements
-    for (int c = threadIdx.x; c < BM * (TK / 8); c += kThreads) {
-      const int r = c / (TK / 8), cc = c % (TK / 8);
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if (m0 + r < M && cc * 8 < kw)
-        v = *reinterpret_cast<const u32x4*>(x + (m0 + r) * K + k0 + cc * 8);
-      *reinterpret_cast<u32x4*>(&As[r * kRow + cc * 8]) = v;
+  f32x4 tot[TM][TN];
+#pragma unroll
+  for (int a = 0; a < TM; ++a)
+#pragma unroll
+    for (int b = 0; b < TN; ++b) tot[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const int nfull = K / TK;
+  const int niter = nfull + ((K % TK) ? 1 : 0);
+  u32x4 areg[kChunks];
+  u32x4 wcur[TN], wnext[TN];
+
+  auto load_a = [&](int it) {
+#pragma unroll
+    for (int c = 0; c < kChunks; ++c) {
+      // the int4 half tile at the end of K has only TK/2 columns
+      const bool ok = it < nfull || (aoff[c] % kRow) < TK / 2;
+      areg[c] = ok ? *reinterpret_cast<const u32x4*>(aptr[c] + it * TK) : u32x4{0u, 0u, 0u, 0u};
     }
-    // this lane's weights: one 16-byte load per strip (8 bytes in the int4 half tile)
-    uint32_t wv[WNT][4];
+  };
+  auto store_a = [&](int buf) {
 #pragma unroll
-    for (int s = 0; s < WNT; ++s) {
-      wv[s][0] = wv[s][1] = wv[s][2] = wv[s][3] = BITS == 8 ? 0x80808080u : 0x88888888u;
-      if (strip0 + s < nstrips) {
-        const uint8_t* sp = codes + (strip0 + s) * strip_bytes(K, BITS);
-        if (kw == TK) {
-          const u32x4 q = *reinterpret_cast<const u32x4*>(sp + it * 1024 + lane * 16);
-          wv[s][0] = q.x; wv[s][1] = q.y; wv[s][2] = q.z; wv[s][3] = q.w;
-        } else {
-          const u32x2 q = *reinterpret_cast<const u32x2*>(sp + nfull * 1024 + lane * 8);
-          wv[s][0] = q.x; wv[s][1] = q.y;
-        }
+    for (int c = 0; c < kChunks; ++c)
+      *reinterpret_cast<u32x4*>(&lds[buf * BM * kRow + aoff[c]]) = areg[c];
+  };
+  auto load_b = [&](u32x4 (&w)[TN], int it) {
+#pragma unroll
+    for (int s = 0; s < TN; ++s) {
+      if (it < nfull) {
+        w[s] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(bptr[s] + it * 1024));
+      } else {  // 8 bytes per lane in the half tile
+        const u32x2 q = *reinterpret_cast<const u32x2*>(bptr[s] - lane * 8 + nfull * 1024);
+        w[s] = u32x4{q.x, q.y, 0u, 0u};
       }
     }
-    __syncthreads();
-    const int nsub = kw / 64;
+  };
+
+  load_a(0);
+  load_b(wcur, 0);
+  store_a(0);
+  __syncthreads();
+
+  for (int it = 0; it < niter; ++it) {
+    const bool more = it + 1 < niter;
+    if (more) {
+      load_a(it + 1);
+      load_b(wnext, it + 1);
+    }
+    const uint16_t* As = lds + (it & 1) * BM * kRow;
+    const int nsub = (it < nfull ? TK : TK / 2) / 64;
 #pragma unroll
     for (int sb = 0; sb < TK / 64; ++sb) {
       if (sb >= nsub) break;
-      f32x4 part[WMT][WNT];
+      f32x4 part[GROUPED ? TM : 1][GROUPED ? TN : 1];
       if (GROUPED) {
 #pragma unroll
-        for (int a = 0; a < WMT; ++a)
+        for (int a = 0; a < TM; ++a)
 #pragma unroll
-          for (int b = 0; b < WNT; ++b) part[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+          for (int b = 0; b < TN; ++b) part[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
       }
 #pragma unroll
       for (int st = 0; st < 2; ++st) {
         const int step = sb * 2 + st;
-        u32x4 bfrag[WNT];
+        u32x4 bfrag[TN];
 #pragma unroll
-        for (int s = 0; s < WNT; ++s) bfrag[s] = DequantExact<DT, BITS>::run(&wv[s][step * kDwPerStep]);
+        for (int s = 0; s < TN; ++s) {
+          const uint32_t w[4] = {wcur[s].x, wcur[s].y, wcur[s].z, wcur[s].w};
+          bfrag[s] = DequantExact<DT, BITS>::run(&w[step * kDw]);
+        }
 #pragma unroll
-        for (int a = 0; a < WMT; ++a) {
-          const int row = (wm * WMT + a) * 16 + j;
+        for (int a = 0; a < TM; ++a) {
+          const int row = (wm * TM + a) * 16 + j;
           const u32x4 af = *reinterpret_cast<const u32x4*>(&As[row * kRow + step * 32 + kb * 8]);
 #pragma unroll
-          for (int s = 0; s < WNT; ++s) {
+          for (int s = 0; s < TN; ++s) {
             if (GROUPED) part[a][s] = mfma16<DT>(af, bfrag[s], part[a][s]);
             else tot[a][s] = mfma16<DT>(af, bfrag[s], tot[a][s]);
           }
         }
       }
       if (GROUPED) {
-        const int64_t g = (k0 + sb * 64) / group_size;
+        const int g = (it * TK + sb * 64) >> gshift;
 #pragma unroll
-        for (int s = 0; s < WNT; ++s) {
-          float sc = 0.0f;
-          if (strip0 + s < nstrips) sc = to_f32<DT>(scale[g * N + (strip0 + s) * 16 + j]);
+        for (int s = 0; s < TN; ++s) {
+          const int st = strip0 + s < nstrips ? strip0 + s : nstrips - 1;
+          const float sc = to_f32<DT>(scale[static_cast<int64_t>(g) * N + st * 16 + j]);
 #pragma unroll
-          for (int a = 0; a < WMT; ++a) tot[a][s] += part[a][s] * sc;
+          for (int a = 0; a < TM; ++a) tot[a][s] += part[a][s] * sc;
         }
       }
     }
+    if (more) store_a((it + 1) & 1);
+    __syncthreads();
+    if (more) {
+#pragma unroll
+      for (int s = 0; s < TN; ++s) wcur[s] = wnext[s];
+    }
   }
 
+  // ---- epilogue: scale, bias, cast; 16-row slabs leave through LDS ----
+  float sc[TN], bv[TN];
 #pragma unroll
-  for (int s = 0; s < WNT; ++s) {
-    if (strip0 + s >= nstrips) continue;
-    const int64_t n = (strip0 + s) * 16 + j;
-    const float sc = GROUPED ? 1.0f : to_f32<DT>(scale[n]);
-    const float bv = bias != nullptr ? to_f32<DT>(bias[n]) : 0.0f;
+  for (int s = 0; s < TN; ++s) {
+    const int st = strip0 + s < nstrips ? strip0 + s : nstrips - 1;
+    const int n = st * 16 + j;
+    sc[s] = GROUPED ? 1.0f : to_f32<DT>(scale[n]);
+    bv[s] = bias != nullptr ? to_f32<DT>(bias[n]) : 0.0f;
+  }
+  if (out_f32) {
 #pragma unroll
-    for (int a = 0; a < WMT; ++a) {
+    for (int s = 0; s < TN; ++s) {
+      if (strip0 + s >= nstrips) continue;
+      const int n = (strip0 + s) * 16 + j;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int64_t m = m0 + (wm * WMT + a) * 16 + kb * 4 + r;
-        if (m >= M) continue;
-        const float v = tot[a][s][r] * sc + bv;
-        if (out_f32) static_cast<float*>(out)[m * N + n] = v;
-        else static_cast<uint16_t*>(out)[m * N + n] = from_f32_rne<DT>(v);
+      for (int a = 0; a < TM; ++a)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int m = m0 + (wm * TM + a) * 16 + kb * 4 + r;
+          if (m < M) static_cast<float*>(out)[static_cast<int64_t>(m) * N + n] = tot[a][s][r] * sc[s] + bv[s];
+        }
+    }
+    return;
+  }
+  constexpr int kSlabRow = TN * 16 + 8;              // padded, in elements
+  uint16_t* slab = lds + wave * 16 * kSlabRow;       // private to the wavefront (A buffers are free now)
+  static_assert(WM * WN * 16 * kSlabRow <= 2 * BM * kRow, "slabs must fit in the A buffers");
+  constexpr int kPieces = 16 * (TN * 16 / 8);        // 16-byte pieces of a slab
+#pragma unroll
+  for (int a = 0; a < TM; ++a) {
+#pragma unroll
+    for (int s = 0; s < TN; ++s)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        slab[(kb * 4 + r) * kSlabRow + s * 16 + j] = from_f32_rne<DT>(tot[a][s][r] * sc[s] + bv[s]);
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int p = lane; p < kPieces; p += 64) {
+      const int r = p / (TN * 2), c = p % (TN * 2);   // row of the slab, 8-column piece
+      const int m = m0 + (wm * TM + a) * 16 + r;
+      const int n = strip0 * 16 + c * 8;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(&slab[r * kSlabRow + c * 8]);
+      if (m < M && n < N)
+        *reinterpret_cast<u32x4*>(static_cast<uint16_t*>(out) + static_cast<int64_t>(m) * N + n) = v;
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+// s_waitcnt that only bounds the number of outstanding vector-memory loads.
+template <int N_>
+__device__ inline void wait_vmcnt() {
+  // gfx9 encoding: vmcnt = [15:14][3:0], expcnt = [6:4], lgkmcnt = [11:8]
+  __builtin_amdgcn_s_waitcnt((N_ & 0xF) | ((N_ >> 4) << 14) | (0x7 << 4) | (0xF << 8));
+}
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// Fast path: per-channel scales, K a multiple of the tile depth.  Both operands
+// travel global -> LDS with direct-to-LDS loads (no registers, no LDS store
+// instructions), three k tiles deep: while tile `it` is consumed the loads of
+// tiles it+1 and it+2 are in flight.  A lands in LDS as unpadded rows whose
+// 16-byte pieces are XOR-swizzled by row so the A-fragment reads of a lane
+// group fall into distinct banks; the raw packed B tiles land exactly as they
+// lie in memory and every lane reads back its own 16 bytes.
+template <int DT, int BITS, int WM, int WN, int TM, int TN>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
+    const uint16_t* __restrict__ x, const uint8_t* __restrict__ codes,
+    const uint16_t* __restrict__ bias, const uint16_t* __restrict__ scale, uint16_t* __restrict__ out,
+    int M, int K, int N, int nbx, int nby) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
+  constexpr int NW = WM * WN;
+  constexpr int BM = WM * TM * 16, BN = WN * TN * 16;
+  constexpr int TK = BITS == 8 ? 64 : 128;
+  constexpr int kDw = BITS == 8 ? 2 : 1;
+  constexpr int C = TK / 8;                      // 16-byte pieces per A row
+  constexpr int kABytes = BM * TK * 2;           // one A tile
+  constexpr int kBBytes = (BN / 16) * 1024;      // one raw B tile (all strips of the workgroup)
+  constexpr int kStage = kABytes + kBBytes;
+  constexpr int kStages = 3;
+  constexpr int kALoads = kABytes / 1024 / NW;   // wave-level loads (1 KiB each) per wavefront
+  constexpr int kBLoads = (BN / 16 + NW - 1) / NW;
+  static_assert(kABytes / 1024 % NW == 0, "A tile must split evenly over the wavefronts");
+  constexpr int kPerStage = kALoads + kBLoads;   // loads every lane issues per stage
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  const int j = lane & 15, kb = lane >> 4;
+  int bx, by;
+  tile_of_block(nbx, nby, &bx, &by);
+  const int m0 = by * BM;
+  const int strip_blk = bx * (BN / 16);
+  const int nstrips = N / kStripCols;
+
+  // global source of this lane for each of its A loads: LDS piece p holds row
+  // p / C, piece (p % C) ^ f(row) of the tile
+  const uint16_t* asrc[kALoads];
+#pragma unroll
+  for (int c = 0; c < kALoads; ++c) {
+    const int p = (c * NW + wave) * 64 + lane;
+    const int row = p / C, slot = p % C;
+    const int cc = slot ^ ((row / (16 / C)) % C);
+    int m = m0 + row;
+    m = m < M ? m : M - 1;
+    asrc[c] = x + static_cast<int64_t>(m) * K + cc * 8;
+  }
+  const uint8_t* bsrc[kBLoads];
+#pragma unroll
+  for (int c = 0; c < kBLoads; ++c) {
+    int st = strip_blk + c * NW + wave;
+    st = st < nstrips ? st : nstrips - 1;
+    bsrc[c] = codes + static_cast<int64_t>(st) * strip_bytes(K, BITS) + lane * 16;
+  }
+  const int niter = K / TK;
+
+  auto issue = [&](int it) {
+    const int t = it < niter ? it : niter - 1;  // past the end: reload the last tile into a spare stage
+    unsigned char* stage = smem + (it % kStages) * kStage;
+#pragma unroll
+    for (int c = 0; c < kALoads; ++c)
+      __builtin_amdgcn_global_load_lds(asrc[c] + t * TK, (lds_ptr_t)(stage + (c * NW + wave) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int c = 0; c < kBLoads; ++c)
+      if (c * NW + wave < BN / 16)
+        __builtin_amdgcn_global_load_lds(bsrc[c] + t * 1024,
+                                         (lds_ptr_t)(stage + kABytes + (c * NW + wave) * 1024), 16, 0, 0);
+  };
+
+  f32x4 tot[TM][TN];
+#pragma unroll
+  for (int a = 0; a < TM; ++a)
+#pragma unroll
+    for (int b = 0; b < TN; ++b) tot[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  issue(0);
+  issue(1);
+  for (int it = 0; it < niter; ++it) {
+    wait_vmcnt<kPerStage>();           // everything but the newest stage has landed
+    __builtin_amdgcn_s_barrier();    // ... for every wavefront; and stage it-1 is free
+    issue(it + 2);
+    const unsigned char* stage = smem + (it % kStages) * kStage;
+    const unsigned char* Bs = stage + kABytes + (wn * TN) * 1024 + lane * 16;
+#pragma unroll
+    for (int step = 0; step < TK / 32; ++step) {
+      u32x4 bfrag[TN];
+#pragma unroll
+      for (int s = 0; s < TN; ++s) {
+        uint32_t w[2];
+        if (BITS == 8) {
+          const u32x2 q = *reinterpret_cast<const u32x2*>(Bs + s * 1024 + step * 8);
+          w[0] = q.x; w[1] = q.y;
+        } else {
+          w[0] = *reinterpret_cast<const uint32_t*>(Bs + s * 1024 + step * 4);
+          w[1] = 0;
+        }
+        bfrag[s] = DequantExact<DT, BITS>::run(w);
+      }
+#pragma unroll
+      for (int a = 0; a < TM; ++a) {
+        const int row = (wm * TM + a) * 16 + j;
+        const int kc = step * 4 + kb;
+        const int slot = kc ^ ((row / (16 / C)) % C);
+        const u32x4 af = *reinterpret_cast<const u32x4*>(stage + row * (TK * 2) + slot * 16);
+#pragma unroll
+        for (int s = 0; s < TN; ++s) tot[a][s] = mfma16<DT>(af, bfrag[s], tot[a][s]);
       }
     }
   }
+  wait_vmcnt<0>();
+  __builtin_amdgcn_s_barrier();  // the spare loads are done and every wavefront has stopped reading
+
+  const int strip0 = strip_blk + wn * TN;
+  float sc[TN], bv[TN];
+#pragma unroll
+  for (int s = 0; s < TN; ++s) {
+    const int st = strip0 + s < nstrips ? strip0 + s : nstrips - 1;
+    const int n = st * 16 + j;
+    sc[s] = to_f32<DT>(scale[n]);
+    bv[s] = bias != nullptr ? to_f32<DT>(bias[n]) : 0.0f;
+  }
+  constexpr int kSlabRow = TN * 16 + 8;
+  uint16_t* slab = reinterpret_cast<uint16_t*>(smem) + wave * 16 * kSlabRow;
+  constexpr int kPieces = 16 * (TN * 16 / 8);
+#pragma unroll
+  for (int a = 0; a < TM; ++a) {
+#pragma unroll
+    for (int s = 0; s < TN; ++s)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        slab[(kb * 4 + r) * kSlabRow + s * 16 + j] = from_f32_rne<DT>(tot[a][s][r] * sc[s] + bv[s]);
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int p = lane; p < kPieces; p += 64) {
+      const int r = p / (TN * 2), c = p % (TN * 2);
+      const int m = m0 + (wm * TM + a) * 16 + r;
+      const int n = strip0 * 16 + c * 8;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(&slab[r * kSlabRow + c * 8]);
+      if (m < M && n < N) *reinterpret_cast<u32x4*>(out + static_cast<int64_t>(m) * N + n) = v;
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+#endif
 }
 
 struct Args {
   const void* x; const void* codes; const void* bias; const void* scale; void* out;
-  int64_t M, K, N; int group_size; int out_f32; hipStream_t stream;
+  int M, K, N, gshift, out_f32; hipStream_t stream;
 };
 
-template <int DT, int BITS, bool GROUPED, int WMT, int WNT>
+template <int DT, int BITS, bool GROUPED, int WM, int WN, int TM, int TN>
 void launch_one(const Args& a) {
-  constexpr int BM = 32 * WMT, BN = 32 * WNT;
-  const dim3 grid(static_cast<unsigned>((a.N + BN - 1) / BN), static_cast<unsigned>((a.M + BM - 1) / BM));
-  gemm_kernel<DT, BITS, GROUPED, WMT, WNT><<<grid, dim3(kThreads), 0, a.stream>>>(
+  constexpr int BM = WM * TM * 16, BN = WN * TN * 16, TK = BITS == 8 ? 64 : 128;
+  const int nbx = (a.N + BN - 1) / BN, nby = (a.M + BM - 1) / BM;
+  const size_t lds = 2 * static_cast<size_t>(BM) * (TK + 8) * sizeof(uint16_t);
+  auto kern = gemm_kernel<DT, BITS, GROUPED, WM, WN, TM, TN>;
+  static bool configured = false;  // per instantiation; the attribute is idempotent
+  if (!configured) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    configured = true;
+  }
+  kern<<<dim3(static_cast<unsigned>(nbx * nby)), dim3(64 * WM * WN), lds, a.stream>>>(
       static_cast<const uint16_t*>(a.x), static_cast<const uint8_t*>(a.codes),
       static_cast<const uint16_t*>(a.bias), static_cast<const uint16_t*>(a.scale), a.out, a.M, a.K,
-      a.N, a.group_size, a.out_f32);
+      a.N, a.gshift, a.out_f32, nbx, nby);
+}
+
+template <int DT, int BITS, int WM, int WN, int TM, int TN>
+void launch_dma(const Args& a) {
+  constexpr int BM = WM * TM * 16, BN = WN * TN * 16, TK = BITS == 8 ? 64 : 128;
+  const int nbx = (a.N + BN - 1) / BN, nby = (a.M + BM - 1) / BM;
+  const size_t lds = 3 * (static_cast<size_t>(BM) * TK * 2 + (BN / 16) * 1024);
+  auto kern = gemm_dma_kernel<DT, BITS, WM, WN, TM, TN>;
+  static bool configured = false;
+  if (!configured) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    configured = true;
+  }
+  kern<<<dim3(static_cast<unsigned>(nbx * nby)), dim3(64 * WM * WN), lds, a.stream>>>(
+      static_cast<const uint16_t*>(a.x), static_cast<const uint8_t*>(a.codes),
+      static_cast<const uint16_t*>(a.bias), static_cast<const uint16_t*>(a.scale),
+      static_cast<uint16_t*>(a.out), a.M, a.K, a.N, nbx, nby);
 }
 
 template <int DT, int BITS>
 void launch_cfg(const Args& a) {
-  if (a.group_size > 0) launch_one<DT, BITS, true, 4, 4>(a);
-  else launch_one<DT, BITS, false, 4, 4>(a);
+  constexpr int TK = BITS == 8 ? 64 : 128;
+  if (a.gshift < 0 && !a.out_f32 && a.K % TK == 0 && a.K / TK >= 2) {
+    if (BITS == 8) launch_dma<DT, BITS, 2, 4, 8, 4>(a);   // 256 x 256 x 64, 144 KiB of LDS
+    else launch_dma<DT, BITS, 2, 4, 4, 4>(a);             // 128 x 256 x 128
+    return;
+  }
+  if (a.gshift >= 0) {
+    launch_one<DT, BITS, true, 2, 4, 8, 2>(a);   // 256 x 128, partial accumulators per group
+  } else {
+    launch_one<DT, BITS, false, 2, 4, 8, 4>(a);  // 256 x 256
+  }
 }
 
 }  // namespace
@@ -248,7 +534,9 @@ void launch_cfg(const Args& a) {
 int launch_linear_gemm(const void* x, const void* codes, const void* bias, const void* scale,
                        int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
                        void* out, bool out_f32, hipStream_t stream) {
-  const Args a{x, codes, bias, scale, out, M, K, N, group_size, out_f32 ? 1 : 0, stream};
+  const int gshift = group_size == 64 ? 6 : (group_size == 128 ? 7 : -1);
+  const Args a{x, codes, bias, scale, out, static_cast<int>(M), static_cast<int>(K),
+               static_cast<int>(N), gshift, out_f32 ? 1 : 0, stream};
   if (dtype == WOL_DTYPE_BF16) {
     if (bits == 8) launch_cfg<WOL_DTYPE_BF16, 8>(a); else launch_cfg<WOL_DTYPE_BF16, 4>(a);
   } else {
