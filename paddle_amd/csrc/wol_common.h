@@ -167,6 +167,20 @@ __device__ inline uint16_t from_f32_rne(float f) {
   return DT == WOL_DTYPE_BF16 ? f32_to_bf16_rne(f) : f32_to_f16_rne(f);
 }
 
+// Output cast of the linear kernels: the hardware's round-to-nearest-even
+// conversions (v_cvt_pk_bf16_f32 / v_cvt_f16_f32), branch-free.  They agree
+// with from_f32_rne on every finite and infinite value; NaN payloads may differ.
+// The fp16 flavour hides its operand from the optimiser first: otherwise the
+// multiply-add that produced it is merged with the conversion into one
+// v_fma_mixlo_f16, which rounds once, and the result would no longer be the
+// cast of the fp32 value that the fp32 output mode reports.
+template <int DT>
+__device__ inline uint16_t cast_out(float f) {
+  if (DT == WOL_DTYPE_BF16) return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
+  asm volatile("" : "+v"(f));
+  return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
+}
+
 // Launchers implemented in the .hip files; each returns a wol_status.
 int launch_quantize(const void* w, int dtype, int64_t K, int64_t N, int bits, int group_size,
                     int round_mode, int layout, void* codes, void* scale, void* workspace,

@@ -301,7 +301,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(
     for (int s = 0; s < TN; ++s)
 #pragma unroll
       for (int r = 0; r < 4; ++r)
-        slab[(kb * 4 + r) * kSlabRow + s * 16 + j] = from_f32_rne<DT>(tot[a][s][r] * sc[s] + bv[s]);
+        slab[(kb * 4 + r) * kSlabRow + s * 16 + j] = cast_out<DT>(tot[a][s][r] * sc[s] + bv[s]);
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int p = lane; p < kPieces; p += 64) {
@@ -325,23 +325,52 @@ __device__ inline void wait_vmcnt() {
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
-// Fast path: per-channel scales, K a multiple of the tile depth.  Both operands
-// travel global -> LDS with direct-to-LDS loads (no registers, no LDS store
+// XOR applied to the 16-byte piece index of an A row in LDS (C pieces per
+// row).  A lane group reads the same piece of 16 consecutive rows; the XOR
+// spreads those reads over the banks whether the LDS serves 8 or 16 lanes of
+// a 128-bit read per cycle.
+template <int C>
+__device__ inline int a_swizzle(int row) {
+  if (C == 8) return (row & 7) ^ ((row >> 3) & 1);  // 128-byte rows
+  return row & (C - 1);                             // 256-byte rows
+}
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+template <int DT>
+__device__ inline f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+  if (DT == WOL_DTYPE_BF16)
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+
+// Fast path: per-channel scales, K a multiple of the tile depth.
+//
+// v_mfma_f32_32x32x16 is the instruction that reaches the matrix cores' full
+// rate on gfx950 (the 16x16x32 form issues at half of it), so the wavefront
+// tile is built from 32 x 32 blocks: TM x TN of them.  Both operands travel
+// global -> LDS with direct-to-LDS loads (no registers, no LDS store
 // instructions), three k tiles deep: while tile `it` is consumed the loads of
 // tiles it+1 and it+2 are in flight.  A lands in LDS as unpadded rows whose
-// 16-byte pieces are XOR-swizzled by row so the A-fragment reads of a lane
-// group fall into distinct banks; the raw packed B tiles land exactly as they
-// lie in memory and every lane reads back its own 16 bytes.
+// 16-byte pieces are XOR-swizzled by row so a lane group's fragment reads
+// fall into distinct banks.  The raw packed B tiles land exactly as they lie
+// in memory (16-column strips in 16x16x32 order); a 32x32x16 B operand is
+// assembled by letting lane l = 32*b + 16*sp + j read the 16 bytes that lane
+// j + 16*(2h + b) of strip sp owns: MFMA (step, h) then contracts over
+// k = 32*step + 16*h + 8*b + i, and the A fragment for it is simply piece
+// 4*step + 2*h + b of the row.
 template <int DT, int BITS, int WM, int WN, int TM, int TN>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
     const uint16_t* __restrict__ x, const uint8_t* __restrict__ codes,
-    const uint16_t* __restrict__ bias, const uint16_t* __restrict__ scale, uint16_t* __restrict__ out,
-    int M, int K, int N, int nbx, int nby) {
+    const uint16_t* __restrict__ bias, const uint16_t* __restrict__ scale, void* __restrict__ outv,
+    int M, int K, int N, int out_f32, int nbx, int nby) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   constexpr int NW = WM * WN;
-  constexpr int BM = WM * TM * 16, BN = WN * TN * 16;
-  constexpr int TK = BITS == 8 ? 64 : 128;
-  constexpr int kDw = BITS == 8 ? 2 : 1;
+  constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
+  constexpr int TK = BITS == 8 ? 64 : 128;       // k per 16-byte lane load of B
+  constexpr int kDw = BITS == 8 ? 2 : 1;         // dwords per 8 codes
   constexpr int C = TK / 8;                      // 16-byte pieces per A row
   constexpr int kABytes = BM * TK * 2;           // one A tile
   constexpr int kBBytes = (BN / 16) * 1024;      // one raw B tile (all strips of the workgroup)
@@ -356,7 +385,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WN, wn = wave % WN;
-  const int j = lane & 15, kb = lane >> 4;
+  const int j = lane & 15, sp = (lane >> 4) & 1, b = lane >> 5, r32 = lane & 31;
   int bx, by;
   tile_of_block(nbx, nby, &bx, &by);
   const int m0 = by * BM;
@@ -364,25 +393,26 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
   const int nstrips = N / kStripCols;
 
   // global source of this lane for each of its A loads: LDS piece p holds row
-  // p / C, piece (p % C) ^ f(row) of the tile
+  // p / C, piece (p % C) ^ swizzle(row) of the tile
   const uint16_t* asrc[kALoads];
 #pragma unroll
   for (int c = 0; c < kALoads; ++c) {
     const int p = (c * NW + wave) * 64 + lane;
     const int row = p / C, slot = p % C;
-    const int cc = slot ^ ((row / (16 / C)) % C);
+    const int cc = slot ^ a_swizzle<C>(row);
     int m = m0 + row;
-    m = m < M ? m : M - 1;
+    m = m < M ? m : M - 1;  // rows past M are computed on valid data and never stored
     asrc[c] = x + static_cast<int64_t>(m) * K + cc * 8;
   }
   const uint8_t* bsrc[kBLoads];
 #pragma unroll
   for (int c = 0; c < kBLoads; ++c) {
     int st = strip_blk + c * NW + wave;
-    st = st < nstrips ? st : nstrips - 1;
+    st = st < nstrips ? st : nstrips - 1;  // past N: valid data, never stored
     bsrc[c] = codes + static_cast<int64_t>(st) * strip_bytes(K, BITS) + lane * 16;
   }
   const int niter = K / TK;
+  const int swz = a_swizzle<C>(lane & 15);  // fragment rows are 32*t + r32; the swizzle has period 16
 
   auto issue = [&](int it) {
     const int t = it < niter ? it : niter - 1;  // past the end: reload the last tile into a spare stage
@@ -397,75 +427,148 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
                                          (lds_ptr_t)(stage + kABytes + (c * NW + wave) * 1024), 16, 0, 0);
   };
 
-  f32x4 tot[TM][TN];
+  f32x16 tot[TM][TN];
 #pragma unroll
   for (int a = 0; a < TM; ++a)
 #pragma unroll
-    for (int b = 0; b < TN; ++b) tot[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int c = 0; c < TN; ++c)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) tot[a][c][r] = 0.0f;
+
+  // byte offsets inside a stage that do not change from tile to tile
+  const int a_row_off = (wm * TM * 32 + r32) * (TK * 2);
+  const int b_off = kABytes + (wn * TN * 2 + sp) * 1024 + (j + 16 * b) * 16;
+  constexpr int Q = TK / 16;  // 16-k slices (one MFMA per 32x32 block each) per tile
+  constexpr int kValuPerMfma = (BITS == 8 ? 16 : 12) * TN / (TM * TN) + 2;
+
+  // The wavefront's pipeline registers: raw codes of the current tile, and
+  // two sets of operands -- the one the MFMAs of slice q use and the one being
+  // prepared for slice q+1 (A fragments read from LDS, B fragments dequantised).
+  u32x4 braw[TN][2];
+  u32x4 af[2][TM];
+  u32x4 bf[2][TN];
+  auto read_b = [&](const unsigned char* stage) {
+#pragma unroll
+    for (int c = 0; c < TN; ++c)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+        braw[c][h] = *reinterpret_cast<const u32x4*>(stage + b_off + c * 2048 + h * 512);
+  };
+  auto read_a = [&](const unsigned char* stage, u32x4 (&dst)[TM], int q) {
+#pragma unroll
+    for (int a = 0; a < TM; ++a) {
+      const int slot = (2 * q + b) ^ swz;
+      dst[a] = *reinterpret_cast<const u32x4*>(stage + a_row_off + a * 32 * (TK * 2) + slot * 16);
+    }
+  };
+  auto dequant = [&](u32x4 (&dst)[TN], int q) {
+    const int step = q / 2, h = q % 2;
+#pragma unroll
+    for (int c = 0; c < TN; ++c) {
+      const uint32_t w4[4] = {braw[c][h].x, braw[c][h].y, braw[c][h].z, braw[c][h].w};
+      dst[c] = DequantExact<DT, BITS>::run(&w4[step * kDw]);
+    }
+  };
+  auto mfmas = [&](const u32x4 (&a4)[TM], const u32x4 (&b4)[TN]) {
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+      for (int c = 0; c < TN; ++c) tot[a][c] = mfma32<DT>(a4[a], b4[c], tot[a][c]);
+  };
 
   issue(0);
   issue(1);
+  issue(2);
+  wait_vmcnt<2 * kPerStage>();  // tile 0 has landed
+  __builtin_amdgcn_s_barrier();
+  read_b(smem);
+  read_a(smem, af[0], 0);
+  dequant(bf[0], 0);
   for (int it = 0; it < niter; ++it) {
-    wait_vmcnt<kPerStage>();           // everything but the newest stage has landed
-    __builtin_amdgcn_s_barrier();    // ... for every wavefront; and stage it-1 is free
-    issue(it + 2);
     const unsigned char* stage = smem + (it % kStages) * kStage;
-    const unsigned char* Bs = stage + kABytes + (wn * TN) * 1024 + lane * 16;
 #pragma unroll
-    for (int step = 0; step < TK / 32; ++step) {
-      u32x4 bfrag[TN];
+    for (int q = 0; q < Q; ++q) {
+      if (q + 1 < Q) {
+        // prepare slice q+1 of this tile while the MFMAs of slice q run: the
+        // scheduler is told to put the LDS reads and a share of the dequantising
+        // VALU work behind every MFMA so they execute in its shadow
+        read_a(stage, af[(q + 1) & 1], q + 1);
+        dequant(bf[(q + 1) & 1], q + 1);
+        mfmas(af[q & 1], bf[q & 1]);
 #pragma unroll
-      for (int s = 0; s < TN; ++s) {
-        uint32_t w[2];
-        if (BITS == 8) {
-          const u32x2 q = *reinterpret_cast<const u32x2*>(Bs + s * 1024 + step * 8);
-          w[0] = q.x; w[1] = q.y;
-        } else {
-          w[0] = *reinterpret_cast<const uint32_t*>(Bs + s * 1024 + step * 4);
-          w[1] = 0;
+        for (int i = 0; i < TM * TN; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                   // one MFMA
+          if (i < TM) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);       // one LDS read
+          __builtin_amdgcn_sched_group_barrier(0x002, kValuPerMfma, 0);        // VALU
         }
-        bfrag[s] = DequantExact<DT, BITS>::run(w);
-      }
-#pragma unroll
-      for (int a = 0; a < TM; ++a) {
-        const int row = (wm * TM + a) * 16 + j;
-        const int kc = step * 4 + kb;
-        const int slot = kc ^ ((row / (16 / C)) % C);
-        const u32x4 af = *reinterpret_cast<const u32x4*>(stage + row * (TK * 2) + slot * 16);
-#pragma unroll
-        for (int s = 0; s < TN; ++s) tot[a][s] = mfma16<DT>(af, bfrag[s], tot[a][s]);
+        __builtin_amdgcn_sched_barrier(0);
+      } else {
+        // last slice: this wavefront needs nothing more from the tile's LDS
+        // stage.  Once every wavefront is there, tile it+1 (landed by now) may
+        // be read and the stage refilled with tile it+3.
+        __builtin_amdgcn_s_waitcnt(0x0070 | (0xF << 0) | (3 << 14));  // lgkmcnt(0): my LDS reads are done
+        wait_vmcnt<kPerStage>();
+        __builtin_amdgcn_s_barrier();
+        issue(it + 3);
+        const unsigned char* next = smem + ((it + 1) % kStages) * kStage;
+        read_b(next);
+        read_a(next, af[(q + 1) & 1], 0);
+        __builtin_amdgcn_sched_barrier(0);
+        mfmas(af[q & 1], bf[q & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+        dequant(bf[(q + 1) & 1], 0);
       }
     }
   }
   wait_vmcnt<0>();
   __builtin_amdgcn_s_barrier();  // the spare loads are done and every wavefront has stopped reading
 
-  const int strip0 = strip_blk + wn * TN;
+  // ---- epilogue: scale, bias, cast; 32-row slabs leave through LDS as 16-byte stores ----
+  // accumulator element r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its block
+  const int col0 = (strip_blk + wn * TN * 2) * 16;  // first column of the wavefront
   float sc[TN], bv[TN];
 #pragma unroll
-  for (int s = 0; s < TN; ++s) {
-    const int st = strip0 + s < nstrips ? strip0 + s : nstrips - 1;
-    const int n = st * 16 + j;
-    sc[s] = to_f32<DT>(scale[n]);
-    bv[s] = bias != nullptr ? to_f32<DT>(bias[n]) : 0.0f;
+  for (int c = 0; c < TN; ++c) {
+    int n = col0 + c * 32 + r32;
+    n = n < N ? n : N - 1;
+    sc[c] = to_f32<DT>(scale[n]);
+    bv[c] = bias != nullptr ? to_f32<DT>(bias[n]) : 0.0f;
   }
-  constexpr int kSlabRow = TN * 16 + 8;
-  uint16_t* slab = reinterpret_cast<uint16_t*>(smem) + wave * 16 * kSlabRow;
-  constexpr int kPieces = 16 * (TN * 16 / 8);
+  if (out_f32) {  // verification mode: the accumulators themselves, plain stores
+    float* outf = static_cast<float*>(outv);
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+      for (int c = 0; c < TN; ++c) {
+        const int n = col0 + c * 32 + r32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = m0 + (wm * TM + a) * 32 + 8 * (r / 4) + 4 * b + r % 4;
+          if (m < M && n < N) outf[static_cast<int64_t>(m) * N + n] = tot[a][c][r] * sc[c] + bv[c];
+        }
+      }
+    return;
+  }
+  uint16_t* out = static_cast<uint16_t*>(outv);
+  constexpr int kSlabRow = TN * 32 + 8;  // padded, in elements
+  static_assert(NW * 32 * kSlabRow * 2 <= kStages * kStage, "slabs must fit in the stage buffers");
+  uint16_t* slab = reinterpret_cast<uint16_t*>(smem) + wave * 32 * kSlabRow;
+  constexpr int kPieces = 32 * (TN * 32 / 8);
 #pragma unroll
   for (int a = 0; a < TM; ++a) {
 #pragma unroll
-    for (int s = 0; s < TN; ++s)
+    for (int c = 0; c < TN; ++c)
 #pragma unroll
-      for (int r = 0; r < 4; ++r)
-        slab[(kb * 4 + r) * kSlabRow + s * 16 + j] = from_f32_rne<DT>(tot[a][s][r] * sc[s] + bv[s]);
+      for (int r = 0; r < 16; ++r)
+        slab[(8 * (r / 4) + 4 * b + r % 4) * kSlabRow + c * 32 + r32] =
+            cast_out<DT>(tot[a][c][r] * sc[c] + bv[c]);
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int p = lane; p < kPieces; p += 64) {
-      const int r = p / (TN * 2), c = p % (TN * 2);
-      const int m = m0 + (wm * TM + a) * 16 + r;
-      const int n = strip0 * 16 + c * 8;
-      const u32x4 v = *reinterpret_cast<const u32x4*>(&slab[r * kSlabRow + c * 8]);
+      const int r = p / (TN * 4), cc = p % (TN * 4);
+      const int m = m0 + (wm * TM + a) * 32 + r;
+      const int n = col0 + cc * 8;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(&slab[r * kSlabRow + cc * 8]);
       if (m < M && n < N) *reinterpret_cast<u32x4*>(out + static_cast<int64_t>(m) * N + n) = v;
     }
     __builtin_amdgcn_wave_barrier();
@@ -498,7 +601,7 @@ void launch_one(const Args& a) {
 
 template <int DT, int BITS, int WM, int WN, int TM, int TN>
 void launch_dma(const Args& a) {
-  constexpr int BM = WM * TM * 16, BN = WN * TN * 16, TK = BITS == 8 ? 64 : 128;
+  constexpr int BM = WM * TM * 32, BN = WN * TN * 32, TK = BITS == 8 ? 64 : 128;
   const int nbx = (a.N + BN - 1) / BN, nby = (a.M + BM - 1) / BM;
   const size_t lds = 3 * (static_cast<size_t>(BM) * TK * 2 + (BN / 16) * 1024);
   auto kern = gemm_dma_kernel<DT, BITS, WM, WN, TM, TN>;
@@ -511,15 +614,15 @@ void launch_dma(const Args& a) {
   kern<<<dim3(static_cast<unsigned>(nbx * nby)), dim3(64 * WM * WN), lds, a.stream>>>(
       static_cast<const uint16_t*>(a.x), static_cast<const uint8_t*>(a.codes),
       static_cast<const uint16_t*>(a.bias), static_cast<const uint16_t*>(a.scale),
-      static_cast<uint16_t*>(a.out), a.M, a.K, a.N, nbx, nby);
+      a.out, a.M, a.K, a.N, a.out_f32, nbx, nby);
 }
 
 template <int DT, int BITS>
 void launch_cfg(const Args& a) {
   constexpr int TK = BITS == 8 ? 64 : 128;
-  if (a.gshift < 0 && !a.out_f32 && a.K % TK == 0 && a.K / TK >= 2) {
-    if (BITS == 8) launch_dma<DT, BITS, 2, 4, 8, 4>(a);   // 256 x 256 x 64, 144 KiB of LDS
-    else launch_dma<DT, BITS, 2, 4, 4, 4>(a);             // 128 x 256 x 128
+  if (a.gshift < 0 && a.K % TK == 0 && a.K / TK >= 2) {
+    if (BITS == 8) launch_dma<DT, BITS, 2, 4, 4, 2>(a);   // 256 x 256 x 64: 144 KiB of LDS
+    else launch_dma<DT, BITS, 2, 4, 2, 2>(a);             // 128 x 256 x 128: 144 KiB of LDS
     return;
   }
   if (a.gshift >= 0) {

@@ -367,7 +367,7 @@ struct StreamKernel {
       if (out_f32)
         static_cast<float*>(out)[static_cast<int64_t>(m) * N + nn] = s;
       else
-        static_cast<uint16_t*>(out)[static_cast<int64_t>(m) * N + nn] = from_f32_rne<DT>(s);
+        static_cast<uint16_t*>(out)[static_cast<int64_t>(m) * N + nn] = cast_out<DT>(s);
     }
   }
 };
