@@ -365,7 +365,7 @@ template <int DT, int BITS, int WM, int WN, int TM, int TN>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
     const uint16_t* __restrict__ x, const uint8_t* __restrict__ codes,
     const uint16_t* __restrict__ bias, const uint16_t* __restrict__ scale, void* __restrict__ outv,
-    int M, int K, int N, int out_f32, int nbx, int nby) {
+    int M, int K, int N, int out_f32, int strip_lo, int strip_hi, int nbx, int nby) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   constexpr int NW = WM * WN;
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
@@ -389,8 +389,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
   int bx, by;
   tile_of_block(nbx, nby, &bx, &by);
   const int m0 = by * BM;
-  const int strip_blk = bx * (BN / 16);
-  const int nstrips = N / kStripCols;
+  // the launch covers the 16-column strips [strip_lo, strip_hi) of the weight
+  const int strip_blk = strip_lo + bx * (BN / 16);
+  const int nstrips = strip_hi;
+  const int n_hi = strip_hi * kStripCols;
 
   // global source of this lane for each of its A loads: LDS piece p holds row
   // p / C, piece (p % C) ^ swizzle(row) of the tile
@@ -444,15 +446,15 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
   // The wavefront's pipeline registers: raw codes of the current tile, and
   // two sets of operands -- the one the MFMAs of slice q use and the one being
   // prepared for slice q+1 (A fragments read from LDS, B fragments dequantised).
-  u32x4 braw[TN][2];
+  u32x4 braw[2][TN][2];
   u32x4 af[2][TM];
   u32x4 bf[2][TN];
-  auto read_b = [&](const unsigned char* stage) {
+  auto read_b = [&](const unsigned char* stage, u32x4 (&dst)[TN][2]) {
 #pragma unroll
     for (int c = 0; c < TN; ++c)
 #pragma unroll
       for (int h = 0; h < 2; ++h)
-        braw[c][h] = *reinterpret_cast<const u32x4*>(stage + b_off + c * 2048 + h * 512);
+        dst[c][h] = *reinterpret_cast<const u32x4*>(stage + b_off + c * 2048 + h * 512);
   };
   auto read_a = [&](const unsigned char* stage, u32x4 (&dst)[TM], int q) {
 #pragma unroll
@@ -461,19 +463,21 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
       dst[a] = *reinterpret_cast<const u32x4*>(stage + a_row_off + a * 32 * (TK * 2) + slot * 16);
     }
   };
-  auto dequant = [&](u32x4 (&dst)[TN], int q) {
+  auto dequant = [&](u32x4 (&dst)[TN], const u32x4 (&raw)[TN][2], int q) {
     const int step = q / 2, h = q % 2;
 #pragma unroll
     for (int c = 0; c < TN; ++c) {
-      const uint32_t w4[4] = {braw[c][h].x, braw[c][h].y, braw[c][h].z, braw[c][h].w};
+      const uint32_t w4[4] = {raw[c][h].x, raw[c][h].y, raw[c][h].z, raw[c][h].w};
       dst[c] = DequantExact<DT, BITS>::run(&w4[step * kDw]);
     }
   };
-  auto mfmas = [&](const u32x4 (&a4)[TM], const u32x4 (&b4)[TN]) {
+  // MFMAs of the A blocks [a_lo, a_hi) of a slice
+  auto mfmas = [&](const u32x4 (&a4)[TM], const u32x4 (&b4)[TN], int a_lo, int a_hi) {
 #pragma unroll
     for (int a = 0; a < TM; ++a)
+      if (a >= a_lo && a < a_hi)
 #pragma unroll
-      for (int c = 0; c < TN; ++c) tot[a][c] = mfma32<DT>(a4[a], b4[c], tot[a][c]);
+        for (int c = 0; c < TN; ++c) tot[a][c] = mfma32<DT>(a4[a], b4[c], tot[a][c]);
   };
 
   issue(0);
@@ -481,20 +485,27 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
   issue(2);
   wait_vmcnt<2 * kPerStage>();  // tile 0 has landed
   __builtin_amdgcn_s_barrier();
-  read_b(smem);
+  read_b(smem, braw[0]);
   read_a(smem, af[0], 0);
-  dequant(bf[0], 0);
-  for (int it = 0; it < niter; ++it) {
+  dequant(bf[0], braw[0], 0);
+  // Every slice runs its MFMAs with the preparation of the next slice's
+  // operands (A fragments read from LDS, B fragments dequantised) spread
+  // between them, so that the VALU work executes in the shadow of the matrix
+  // pipe.  The workgroup barrier that hands the stage of tile `it` over to
+  // tile it+3 sits in the middle of the last but one slice, once the
+  // wavefront has fetched its last operands of the tile; the raw codes of tile
+  // it+1 are read right behind it and have a whole slice to arrive.
+  static_assert(Q >= 2 && TM % 2 == 0, "the pipeline needs two slices per tile and an even TM");
+  auto tile = [&](int it, u32x4 (&raw)[TN][2], u32x4 (&raw_next)[TN][2]) {
     const unsigned char* stage = smem + (it % kStages) * kStage;
+    const unsigned char* next = smem + ((it + 1) % kStages) * kStage;
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
-      if (q + 1 < Q) {
-        // prepare slice q+1 of this tile while the MFMAs of slice q run: the
-        // scheduler is told to put the LDS reads and a share of the dequantising
-        // VALU work behind every MFMA so they execute in its shadow
-        read_a(stage, af[(q + 1) & 1], q + 1);
-        dequant(bf[(q + 1) & 1], q + 1);
-        mfmas(af[q & 1], bf[q & 1]);
+      if (q != Q - 2) {
+        const bool last = q == Q - 1;
+        read_a(last ? next : stage, af[(q + 1) & 1], last ? 0 : q + 1);
+        dequant(bf[(q + 1) & 1], last ? raw_next : raw, last ? 0 : q + 1);
+        mfmas(af[q & 1], bf[q & 1], 0, TM);
 #pragma unroll
         for (int i = 0; i < TM * TN; ++i) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                   // one MFMA
@@ -503,22 +514,37 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
         }
         __builtin_amdgcn_sched_barrier(0);
       } else {
-        // last slice: this wavefront needs nothing more from the tile's LDS
-        // stage.  Once every wavefront is there, tile it+1 (landed by now) may
-        // be read and the stage refilled with tile it+3.
-        __builtin_amdgcn_s_waitcnt(0x0070 | (0xF << 0) | (3 << 14));  // lgkmcnt(0): my LDS reads are done
+        read_a(stage, af[(q + 1) & 1], q + 1);
+        mfmas(af[q & 1], bf[q & 1], 0, TM / 2);
+#pragma unroll
+        for (int i = 0; i < TM * TN / 2; ++i) {
+          if (2 * i < TM) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // this wavefront needs nothing more from the tile's stage; once every
+        // wavefront is there, tile it+1 (landed by now) may be read and the
+        // stage refilled with tile it+3
+        __builtin_amdgcn_s_waitcnt(0x0070 | (0xF << 0) | (3 << 14));  // lgkmcnt(0)
         wait_vmcnt<kPerStage>();
         __builtin_amdgcn_s_barrier();
         issue(it + 3);
-        const unsigned char* next = smem + ((it + 1) % kStages) * kStage;
-        read_b(next);
-        read_a(next, af[(q + 1) & 1], 0);
+        read_b(next, raw_next);
+        dequant(bf[(q + 1) & 1], raw, q + 1);
+        mfmas(af[q & 1], bf[q & 1], TM / 2, TM);
+#pragma unroll
+        for (int i = 0; i < TM * TN / 2; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (i < 2 * TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, 2 * kValuPerMfma, 0);
+        }
         __builtin_amdgcn_sched_barrier(0);
-        mfmas(af[q & 1], bf[q & 1]);
-        __builtin_amdgcn_sched_barrier(0);
-        dequant(bf[(q + 1) & 1], 0);
       }
     }
+  };
+  for (int it = 0; it < niter; it += 2) {
+    tile(it, braw[0], braw[1]);
+    if (it + 1 < niter) tile(it + 1, braw[1], braw[0]);
   }
   wait_vmcnt<0>();
   __builtin_amdgcn_s_barrier();  // the spare loads are done and every wavefront has stopped reading
@@ -530,7 +556,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
 #pragma unroll
   for (int c = 0; c < TN; ++c) {
     int n = col0 + c * 32 + r32;
-    n = n < N ? n : N - 1;
+    n = n < n_hi ? n : n_hi - 1;
     sc[c] = to_f32<DT>(scale[n]);
     bv[c] = bias != nullptr ? to_f32<DT>(bias[n]) : 0.0f;
   }
@@ -544,7 +570,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int m = m0 + (wm * TM + a) * 32 + 8 * (r / 4) + 4 * b + r % 4;
-          if (m < M && n < N) outf[static_cast<int64_t>(m) * N + n] = tot[a][c][r] * sc[c] + bv[c];
+          if (m < M && n < n_hi) outf[static_cast<int64_t>(m) * N + n] = tot[a][c][r] * sc[c] + bv[c];
         }
       }
     return;
@@ -569,7 +595,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
       const int m = m0 + (wm * TM + a) * 32 + r;
       const int n = col0 + cc * 8;
       const u32x4 v = *reinterpret_cast<const u32x4*>(&slab[r * kSlabRow + cc * 8]);
-      if (m < M && n < N) *reinterpret_cast<u32x4*>(out + static_cast<int64_t>(m) * N + n) = v;
+      if (m < M && n < n_hi) *reinterpret_cast<u32x4*>(out + static_cast<int64_t>(m) * N + n) = v;
     }
     __builtin_amdgcn_wave_barrier();
   }
@@ -599,10 +625,12 @@ void launch_one(const Args& a) {
       a.N, a.gshift, a.out_f32, nbx, nby);
 }
 
+// Launches the fast kernel on the columns of strips [strip_lo, strip_hi).
 template <int DT, int BITS, int WM, int WN, int TM, int TN>
-void launch_dma(const Args& a) {
+void launch_dma(const Args& a, int strip_lo, int strip_hi) {
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32, TK = BITS == 8 ? 64 : 128;
-  const int nbx = (a.N + BN - 1) / BN, nby = (a.M + BM - 1) / BM;
+  if (strip_hi <= strip_lo) return;
+  const int nbx = ((strip_hi - strip_lo) * kStripCols + BN - 1) / BN, nby = (a.M + BM - 1) / BM;
   const size_t lds = 3 * (static_cast<size_t>(BM) * TK * 2 + (BN / 16) * 1024);
   auto kern = gemm_dma_kernel<DT, BITS, WM, WN, TM, TN>;
   static bool configured = false;
@@ -614,15 +642,50 @@ void launch_dma(const Args& a) {
   kern<<<dim3(static_cast<unsigned>(nbx * nby)), dim3(64 * WM * WN), lds, a.stream>>>(
       static_cast<const uint16_t*>(a.x), static_cast<const uint8_t*>(a.codes),
       static_cast<const uint16_t*>(a.bias), static_cast<const uint16_t*>(a.scale),
-      a.out, a.M, a.K, a.N, a.out_f32, nbx, nby);
+      a.out, a.M, a.K, a.N, a.out_f32, strip_lo, strip_hi, nbx, nby);
+}
+
+// Number of 256-column tiles given to the 256-row kernel; the remaining
+// columns run with 128-row tiles.  Cost model: a workgroup owns its CU, so a
+// launch takes ceil(tiles / CUs) tile times; a 128-row tile costs kSmall of a
+// 256-row one (more than half: the dequantised B operand is shared by fewer
+// MFMAs).
+inline int plan_big_columns(int M, int N) {
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    return n;
+  }();
+  constexpr double kSmall = 0.56;
+  const int nbx = (N + 255) / 256, nby_big = (M + 255) / 256, nby_small = (M + 127) / 128;
+  int best = nbx;
+  double best_t = 1e30;
+  for (int c = nbx; c >= 0; --c) {
+    const double t = static_cast<double>((c * nby_big + cus - 1) / cus) +
+                     kSmall * static_cast<double>(((nbx - c) * nby_small + cus - 1) / cus);
+    if (t < best_t - 1e-9) { best_t = t; best = c; }
+  }
+  return best;
 }
 
 template <int DT, int BITS>
 void launch_cfg(const Args& a) {
   constexpr int TK = BITS == 8 ? 64 : 128;
   if (a.gshift < 0 && a.K % TK == 0 && a.K / TK >= 2) {
-    if (BITS == 8) launch_dma<DT, BITS, 2, 4, 4, 2>(a);   // 256 x 256 x 64: 144 KiB of LDS
-    else launch_dma<DT, BITS, 2, 4, 2, 2>(a);             // 128 x 256 x 128: 144 KiB of LDS
+    const int nstrips = a.N / kStripCols;
+    if constexpr (BITS == 8) {
+      // 256 x 256 x 64 tiles (144 KiB of LDS, one workgroup per CU) for as many
+      // column tiles as fill whole rounds of the CUs; the rest, which would
+      // leave CUs idle for a whole tile time, goes to 128 x 256 tiles.
+      const int c = plan_big_columns(a.M, a.N);
+      const int hi = c * 16 < nstrips ? c * 16 : nstrips;
+      launch_dma<DT, BITS, 2, 4, 4, 2>(a, 0, hi);
+      launch_dma<DT, BITS, 2, 4, 2, 2>(a, hi, nstrips);
+    } else {
+      launch_dma<DT, BITS, 2, 4, 2, 2>(a, 0, nstrips);   // 128 x 256 x 128: 144 KiB of LDS
+    }
     return;
   }
   if (a.gshift >= 0) {

@@ -154,6 +154,12 @@ struct StreamKernel {
   static constexpr int kRowsPerGroup = MP < 4 ? 4 / MP : 1;  // row groups inside one lane group
   static constexpr int kClasses = kS / kRowsPerGroup;        // lane groups that receive results
   static constexpr int kLive = MP == 1 ? 1 : (MP == 2 ? 2 : 4);  // accumulators left after folding
+  // Group-wise scales a lane loads per unit.  With MP < 16 a lane keeps only
+  // the steps of its own class (all others land in sums that are discarded),
+  // kRowsPerGroup consecutive steps per A operand, and two consecutive steps
+  // (64 k) always share a group: one load per pair.  MP = 16 keeps every step.
+  static constexpr int kPairs = kRowsPerGroup >= 2 ? kRowsPerGroup / 2 : 1;
+  static constexpr int kNS = MP == 16 ? kU / 2 : kNA * kPairs;
 
   const uint16_t* x;
   const uint16_t* scale;
@@ -170,7 +176,7 @@ struct StreamKernel {
   struct Unit {
     u32x4 wv[kNT];
     u32x4 av[kNA][MT];
-    uint16_t sraw[kU / 2];
+    uint16_t sraw[kNS];
   };
 
   // A operand whose row group `slot` holds k step (step0 + slot); with
@@ -191,18 +197,32 @@ struct StreamKernel {
     return row[n];
   }
 
+  // Index into Unit::sraw of the scale that step s of a unit uses.
+  __device__ static constexpr int scale_slot(int s) {
+    return MP == 16 ? s / 2 : (s / kS) * kPairs + ((s % kS) % kRowsPerGroup) / 2;
+  }
+
+  // The small loads (activations, scales) go first: the memory system returns
+  // loads in order, so the first weight tile can be consumed while the later
+  // ones are still on their way.
   __device__ inline void load_unit(Unit& d, const u32x4* tp, int u) const {
     const int step0 = u * kU;
-#pragma unroll
-    for (int i = 0; i < kNT; ++i) d.wv[i] = __builtin_nontemporal_load(tp + (step0 / kSPT + i) * 64);
 #pragma unroll
     for (int a = 0; a < kNA; ++a)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) d.av[a][mt] = load_a(mt, step0 + a * kS, true);
     if (GROUPED) {
+      const int mine = MP == 8 ? (kb >> 1) : kb;
 #pragma unroll
-      for (int p = 0; p < kU / 2; ++p) d.sraw[p] = load_scale_raw(step0 + 2 * p);
+      for (int p = 0; p < kNS; ++p) {
+        const int step = MP == 16 ? step0 + 2 * p
+                                  : step0 + (p / kPairs) * kS + mine * kRowsPerGroup + 2 * (p % kPairs);
+        d.sraw[p] = load_scale_raw(step);
+      }
     }
+    if (NU > 0) __builtin_amdgcn_sched_barrier(0);  // keep the compiler from moving them behind the weights
+#pragma unroll
+    for (int i = 0; i < kNT; ++i) d.wv[i] = __builtin_nontemporal_load(tp + (step0 / kSPT + i) * 64);
   }
 
   // mfma(A, constant B): the term that removes the dequantiser's offset.  It
@@ -243,7 +263,7 @@ struct StreamKernel {
     for (int s = 0; s < kU; ++s) {
       const u32x4 t = d.wv[s / kSPT];
       const uint32_t w[4] = {t.x, t.y, t.z, t.w};
-      const float sc = GROUPED ? to_f32<DT>(d.sraw[s / 2]) : 1.0f;
+      const float sc = GROUPED ? to_f32<DT>(d.sraw[scale_slot(s)]) : 1.0f;
       step_mfma(w + (s % kSPT) * kDw, d.av[s / kS], cc[s / kS], s % kS, sc);
     }
   }
@@ -266,11 +286,18 @@ struct StreamKernel {
 #pragma unroll
       for (int c = 0; c < kClasses; ++c) totc[mt][c] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+    // what the epilogue needs from memory, requested before the long loads:
+    // thread t always stores column t % 16 of the strip
+    // (raw bits; they are converted where they are used, after the long loads)
+    const uint16_t ep_sraw = scale[n];
+    const uint16_t ep_braw = (bias != nullptr ? bias : scale)[n];  // one unconditional load
+
     const u32x4* tp = reinterpret_cast<const u32x4*>(strip) + lane;
     if (NU > 0) {
       Unit d[NU > 0 ? NU : 1];
 #pragma unroll
       for (int i = 0; i < NU; ++i) load_unit(d[i], tp, wave * NU + i);
+      __builtin_amdgcn_sched_barrier(0);  // every load is in flight before the first wait
 #pragma unroll
       for (int i = 0; i < NU; ++i) compute_unit(d[i]);
     } else {
@@ -321,6 +348,11 @@ struct StreamKernel {
       }
     }
 
+    // The epilogue's operands were requested first and have arrived by now;
+    // naming them here keeps the compiler from sinking those loads (and the
+    // reads of the kernel arguments) into the tail of the kernel.
+    asm volatile("" ::"v"(ep_sraw), "v"(ep_braw), "s"(out), "s"(out_f32));
+
     // Merge the classes: every lane keeps the class of its own lane group.
     f32x4 tot[MT];
     {
@@ -361,9 +393,10 @@ struct StreamKernel {
 #pragma unroll
       for (int w = 0; w < WK; ++w)
         s += red[((w * MT + mt) * 4 + (row % 4)) * 64 + (row / 4) * 16 + nl];
-      const int nn = tn * kStripCols + nl;
-      if (!GROUPED) s *= to_f32<DT>(scale[nn]);
-      if (bias != nullptr) s += to_f32<DT>(bias[nn]);
+      const int nn = tn * kStripCols + nl;  // nl == j: the stride of idx is a multiple of 16
+      const float ep_scale = GROUPED ? 1.0f : to_f32<DT>(ep_sraw);
+      const float ep_bias = bias != nullptr ? to_f32<DT>(ep_braw) : 0.0f;
+      s = s * ep_scale + ep_bias;
       if (out_f32)
         static_cast<float*>(out)[static_cast<int64_t>(m) * N + nn] = s;
       else
