@@ -24,25 +24,47 @@ bool layout_ok(int layout) {
          layout == WOL_LAYOUT_GFX950;
 }
 
-// The streaming kernel covers M <= 64 (four 16-row MFMA tiles).
+// The streaming kernel takes M <= 64 (four 16-row MFMA tiles).  It streams
+// the weights best, but every 16-column strip re-reads its activations from
+// L2; the MFMA GEMM shares them through LDS at the price of a second launch
+// that adds the K runs.  Between 9 and 64 rows the cheaper of the two by a
+// two-term cost model (microseconds, fitted to measurements on MI355X) runs.
 constexpr int64_t kStreamMaxM = 64;
+constexpr int64_t kStreamAlwaysM = 8;
+
+bool gemm_fast_path(int64_t K, int bits) {
+  const int64_t tk = bits == 8 ? 64 : 128;
+  return K % tk == 0 && K / tk >= 2;
+}
+
+bool use_stream(int64_t M, int64_t K, int64_t N, int bits) {
+  if (M > kStreamMaxM) return false;
+  if (M <= kStreamAlwaysM || !gemm_fast_path(K, bits)) return true;
+  const double w = static_cast<double>(K) * N * bits / 8.0;           // weight bytes
+  const double rows = static_cast<double>((M + 15) / 16 * 16);
+  const double a = static_cast<double>(N / 16) * rows * K * 2.0;      // activation bytes re-read
+  const double t_stream = (w / 5.0e6 > a / 8.0e6 ? w / 5.0e6 : a / 8.0e6) + 3.0;
+  const double t_gemm = w / 4.3e6 + 11.0;
+  return t_stream <= t_gemm;
+}
 
 int linear_impl(const void* x, const void* codes, const void* bias, const void* scale, int dtype,
                 int64_t M, int64_t K, int64_t N, int bits, int group_size, void* out, bool out_f32,
-                void* stream) {
+                void* workspace, size_t workspace_bytes, void* stream) {
   const int rc = check_problem(dtype, K, N, bits, group_size);
   if (rc != WOL_OK) return rc;
   if (M < 0 || M > (int64_t{1} << 30)) return WOL_ERR_BAD_SHAPE;
   if (M == 0) return WOL_OK;  // empty batch: nothing to write
   if (x == nullptr || codes == nullptr || scale == nullptr || out == nullptr)
     return WOL_ERR_NULL_POINTER;
-  if (!aligned16(x) || !aligned16(codes)) return WOL_ERR_ALIGNMENT;
+  if (!aligned16(x) || !aligned16(codes) || !aligned16(scale)) return WOL_ERR_ALIGNMENT;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (M <= kStreamMaxM)
+  if (use_stream(M, K, N, bits))
     return wol::launch_linear_stream(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out,
                                      out_f32, s);
+  if (workspace == nullptr || !aligned16(workspace)) workspace_bytes = 0;  // optional: only speeds up
   return wol::launch_linear_gemm(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out,
-                                 out_f32, s);
+                                 out_f32, workspace, workspace_bytes, s);
 }
 
 }  // namespace
@@ -102,23 +124,23 @@ int wol_dequantize(const void* codes, int layout, const void* scale, int dtype, 
 }
 
 size_t wol_linear_workspace(int64_t M, int64_t K, int64_t N, int bits, int group_size) {
-  (void)M; (void)K; (void)N; (void)bits; (void)group_size;
-  return 0;  // both kernels keep their partial sums on chip
+  if (check_problem(WOL_DTYPE_F16, K, N, bits, group_size) != WOL_OK || M <= 0) return 0;
+  if (use_stream(M, K, N, bits)) return 0;  // partial sums stay on chip
+  return wol::linear_gemm_workspace(M, K, N, bits);
 }
 
 int wol_linear(const void* x, const void* codes, const void* bias, const void* scale, int dtype,
                int64_t M, int64_t K, int64_t N, int bits, int group_size, void* out,
                void* workspace, size_t workspace_bytes, void* stream) {
-  (void)workspace; (void)workspace_bytes;
-  return linear_impl(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out, false, stream);
+  return linear_impl(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out, false,
+                     workspace, workspace_bytes, stream);
 }
 
 int wol_linear_f32(const void* x, const void* codes, const void* bias, const void* scale,
                    int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
                    float* out_f32, void* workspace, size_t workspace_bytes, void* stream) {
-  (void)workspace; (void)workspace_bytes;
   return linear_impl(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out_f32, true,
-                     stream);
+                     workspace, workspace_bytes, stream);
 }
 
 int wol_repack(const void* codes_in, int layout_in, void* codes_out, int layout_out, int64_t K,

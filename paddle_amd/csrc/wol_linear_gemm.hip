@@ -14,6 +14,9 @@
 // 16-byte stores.  Workgroups are numbered so that each XCD (one L2 each)
 // works on a compact block of neighbouring tiles.
 #include "wol_common.h"
+#include "wol_dequant.h"
+
+#include <climits>
 
 namespace wol {
 namespace {
@@ -22,7 +25,6 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 template <int DT>
@@ -113,8 +115,8 @@ struct DequantExact<WOL_DTYPE_BF16, 4> {
 // Workgroup -> output tile.  Hardware deals consecutive workgroup ids to the
 // 8 XCDs in turn; give XCD x the ids that form a compact block of tiles so
 // that its L2 sees every A row block and B column block of that block once.
-__device__ inline void tile_of_block(int nbx, int nby, int* bx, int* by) {
-  const int id = blockIdx.x, total = nbx * nby;
+__device__ inline void tile_of_block(int id, int nbx, int nby, int* bx, int* by) {
+  const int total = nbx * nby;
   constexpr int kXcd = 8;
   int t = id;
   if (total % kXcd == 0) {
@@ -145,7 +147,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(
   const int wm = wave / WN, wn = wave % WN;
   const int j = lane & 15, kb = lane >> 4;
   int bx, by;
-  tile_of_block(nbx, nby, &bx, &by);
+  tile_of_block(blockIdx.x, nbx, nby, &bx, &by);
   const int m0 = by * BM;
   const int strip0 = bx * (BN / 16) + wn * TN;
   const int nstrips = N / kStripCols;
@@ -346,7 +348,22 @@ __device__ inline f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
                                                 __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
 }
 
-// Fast path: per-channel scales, K a multiple of the tile depth.
+// What one launch of the fast kernel works on.
+struct DmaParams {
+  const uint16_t* x;
+  const uint8_t* codes;
+  const uint16_t* bias;
+  const uint16_t* scale;
+  void* out;                    // T or fp32 [M, N]; with nsplit > 1 fp32 partial sums [nsplit][M][N]
+  int M, K, N;
+  int out_f32;
+  int strip_lo, strip_hi;       // the launch covers the 16-column strips [strip_lo, strip_hi)
+  int nbx, nby;                 // output tiles of the launch
+  int nsplit, tiles_per_split;  // K is cut into nsplit runs of k tiles, one workgroup each
+  int rotate;                   // start each column tile's run at a different k tile
+};
+
+// Fast path: K a multiple of the tile depth.
 //
 // v_mfma_f32_32x32x16 is the instruction that reaches the matrix cores' full
 // rate on gfx950 (the 16x16x32 form issues at half of it), so the wavefront
@@ -361,11 +378,23 @@ __device__ inline f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
 // j + 16*(2h + b) of strip sp owns: MFMA (step, h) then contracts over
 // k = 32*step + 16*h + 8*b + i, and the A fragment for it is simply piece
 // 4*step + 2*h + b of the row.
-template <int DT, int BITS, int WM, int WN, int TM, int TN>
-__global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
-    const uint16_t* __restrict__ x, const uint8_t* __restrict__ codes,
-    const uint16_t* __restrict__ bias, const uint16_t* __restrict__ scale, void* __restrict__ outv,
-    int M, int K, int N, int out_f32, int strip_lo, int strip_hi, int nbx, int nby) {
+//
+// G = 0: per-channel scales, applied in the epilogue.  G = 64 or 128:
+// group-wise scales; the MFMAs of a group accumulate into `part`, which is
+// folded into the running sum with the group's scale (an fp32 FMA per
+// accumulator element), so code * scale is never rounded to T.
+//
+// OFFS selects the offset dequantiser: a fraction of the VALU work, paid for
+// with one more MFMA per A fragment and slice (into `canc`, which holds
+// -offset * sum of the activations and is added when the scale is applied).
+// It is the right trade when M is small: the matrix pipe idles, the VALU does
+// not.
+//
+// With nsplit > 1 a workgroup covers only a run of k tiles and leaves its
+// fp32 sums (scaled, without bias) in a partial buffer; reduce_partials_kernel
+// adds the runs.  That is what fills the CUs when M is small.
+template <int DT, int BITS, int G, bool OFFS, int WM, int WN, int TM, int TN>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   constexpr int NW = WM * WN;
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
@@ -374,79 +403,150 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
   constexpr int C = TK / 8;                      // 16-byte pieces per A row
   constexpr int kABytes = BM * TK * 2;           // one A tile
   constexpr int kBBytes = (BN / 16) * 1024;      // one raw B tile (all strips of the workgroup)
-  constexpr int kStage = kABytes + kBBytes;
+  constexpr int kSBytes = G == 0 ? 0 : NW * 256;  // the tile's group scales: 128 values per wavefront
+  constexpr int kStage = kABytes + kBBytes + kSBytes;
   constexpr int kStages = 3;
   constexpr int kALoads = kABytes / 1024 / NW;   // wave-level loads (1 KiB each) per wavefront
-  constexpr int kBLoads = (BN / 16 + NW - 1) / NW;
-  static_assert(kABytes / 1024 % NW == 0, "A tile must split evenly over the wavefronts");
-  constexpr int kPerStage = kALoads + kBLoads;   // loads every lane issues per stage
+  constexpr int kBLoads = BN / 16 / NW;
+  static_assert(kABytes / 1024 % NW == 0 && kALoads >= 1, "A tile must split evenly over the wavefronts");
+  static_assert(BN / 16 % NW == 0 && kBLoads >= 1, "B tile must split evenly over the wavefronts");
+  constexpr int Q = TK / 16;  // 16-k slices (one MFMA per 32x32 block each) per tile
+  // group-wise scales: a fold every kFold slices, kGT folds (groups or halves of one) per tile
+  constexpr int kFoldK = G == 0 ? TK : (G < TK ? G : TK);
+  constexpr int kFold = kFoldK / 16;
+  constexpr int kGT = TK / kFoldK;
+  constexpr int kGShift = G == 128 ? 7 : 6;
+  static_assert(kGT * BN <= NW * 128, "the tile's scales must fit the wavefronts' 4-byte loads");
+  // direct-to-LDS loads every lane issues per stage.  They are the only vector
+  // memory loads of the main loop, so they complete in issue order and
+  // s_waitcnt vmcnt(n) can tell which stages have landed.
+  constexpr int kPerStage = kALoads + kBLoads + (G == 0 ? 0 : 1);
+  static_assert(Q >= 2 && (Q - 2) % kFold != 0 && (Q - 2) % kFold != kFold - 1,
+                "the slice that holds the barrier neither starts nor ends a group");
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
+  const uint16_t* __restrict__ x = p.x;
+  const uint16_t* __restrict__ scale = p.scale;
+  const int M = p.M, K = p.K, N = p.N;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WN, wn = wave % WN;
   const int j = lane & 15, sp = (lane >> 4) & 1, b = lane >> 5, r32 = lane & 31;
+  const int ntiles = p.nbx * p.nby;
+  const int split = blockIdx.x / ntiles;
   int bx, by;
-  tile_of_block(nbx, nby, &bx, &by);
+  tile_of_block(blockIdx.x - split * ntiles, p.nbx, p.nby, &bx, &by);
   const int m0 = by * BM;
-  // the launch covers the 16-column strips [strip_lo, strip_hi) of the weight
-  const int strip_blk = strip_lo + bx * (BN / 16);
-  const int nstrips = strip_hi;
-  const int n_hi = strip_hi * kStripCols;
+  const int strip_blk = p.strip_lo + bx * (BN / 16);
+  const int nstrips = p.strip_hi;
+  const int n_hi = p.strip_hi * kStripCols;
+  // this workgroup's run of k tiles
+  const int t0 = split * p.tiles_per_split;
+  const int niter = (K / TK - t0) < p.tiles_per_split ? (K / TK - t0) : p.tiles_per_split;
+  // Strips lie a power of two apart when K is one, so workgroups that walk
+  // their k tiles in step would keep hitting the same few memory channels.
+  // With `rotate` each column tile starts its run somewhere else (the run
+  // wraps around; only the order of the fp32 additions changes).
+  const int rot = p.rotate ? (bx * 5 + split * 3) % niter : 0;
+  auto tile_index = [&](int it) {  // position in the run -> k tile of the run
+    int t = (it < niter ? it : niter - 1) + rot;
+    return t < niter ? t : t - niter;
+  };
 
-  // global source of this lane for each of its A loads: LDS piece p holds row
-  // p / C, piece (p % C) ^ swizzle(row) of the tile
+  // global source of this lane for each of its A loads: LDS piece q holds row
+  // q / C, piece (q % C) ^ swizzle(row) of the tile
   const uint16_t* asrc[kALoads];
 #pragma unroll
   for (int c = 0; c < kALoads; ++c) {
-    const int p = (c * NW + wave) * 64 + lane;
-    const int row = p / C, slot = p % C;
+    const int q = (c * NW + wave) * 64 + lane;
+    const int row = q / C, slot = q % C;
     const int cc = slot ^ a_swizzle<C>(row);
     int m = m0 + row;
     m = m < M ? m : M - 1;  // rows past M are computed on valid data and never stored
-    asrc[c] = x + static_cast<int64_t>(m) * K + cc * 8;
+    asrc[c] = x + static_cast<int64_t>(m) * K + static_cast<int64_t>(t0) * TK + cc * 8;
   }
   const uint8_t* bsrc[kBLoads];
 #pragma unroll
   for (int c = 0; c < kBLoads; ++c) {
     int st = strip_blk + c * NW + wave;
-    st = st < nstrips ? st : nstrips - 1;  // past N: valid data, never stored
-    bsrc[c] = codes + static_cast<int64_t>(st) * strip_bytes(K, BITS) + lane * 16;
+    st = st < nstrips ? st : nstrips - 1;  // past the last column: valid data, never stored
+    bsrc[c] = p.codes + static_cast<int64_t>(st) * strip_bytes(K, BITS) +
+              static_cast<int64_t>(t0) * 1024 + lane * 16;
   }
-  const int niter = K / TK;
   const int swz = a_swizzle<C>(lane & 15);  // fragment rows are 32*t + r32; the swizzle has period 16
 
+  // Group scales travel with the tile: value v = 2 * (64 * wave + lane) of the
+  // flattened [kGT][BN] block of the tile's scale rows, two values per lane.
+  const int sval = 2 * (wave * 64 + lane) < kGT * BN ? 2 * (wave * 64 + lane) : 0;
+  const int sfold = sval / BN;
+  int scol = strip_blk * kStripCols + sval % BN;
+  scol = scol < n_hi ? scol : n_hi - 2;  // past the last column: valid data, never used
   auto issue = [&](int it) {
-    const int t = it < niter ? it : niter - 1;  // past the end: reload the last tile into a spare stage
+    const int t = tile_index(it);  // past the end: reload the last tile into a spare stage
     unsigned char* stage = smem + (it % kStages) * kStage;
+    if (G != 0) {
+      const int64_t row = (static_cast<int64_t>(t0 + t) * TK + sfold * kFoldK) >> kGShift;
+      __builtin_amdgcn_global_load_lds(scale + row * N + scol,
+                                       (lds_ptr_t)(stage + kABytes + kBBytes + wave * 256), 4, 0, 0);
+    }
 #pragma unroll
     for (int c = 0; c < kALoads; ++c)
       __builtin_amdgcn_global_load_lds(asrc[c] + t * TK, (lds_ptr_t)(stage + (c * NW + wave) * 1024), 16, 0, 0);
 #pragma unroll
     for (int c = 0; c < kBLoads; ++c)
-      if (c * NW + wave < BN / 16)
-        __builtin_amdgcn_global_load_lds(bsrc[c] + t * 1024,
-                                         (lds_ptr_t)(stage + kABytes + (c * NW + wave) * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(bsrc[c] + t * 1024,
+                                       (lds_ptr_t)(stage + kABytes + (c * NW + wave) * 1024), 16, 0, 0);
+  };
+
+  // columns of this lane's accumulators: block c of the wavefront, column r32
+  const int col0 = (strip_blk + wn * TN * 2) * 16;
+  int ncol[TN];
+#pragma unroll
+  for (int c = 0; c < TN; ++c) {
+    const int n = col0 + c * 32 + r32;
+    ncol[c] = n < n_hi ? n : n_hi - 1;
+  }
+  // this lane's scales of the tile in `stage`, out of LDS
+  auto read_scales = [&](const unsigned char* stage, uint16_t (&dst)[kGT > 0 ? kGT : 1][TN]) {
+    if (G != 0) {
+#pragma unroll
+      for (int f = 0; f < kGT; ++f)
+#pragma unroll
+        for (int c = 0; c < TN; ++c)
+          dst[f][c] = *reinterpret_cast<const uint16_t*>(
+              stage + kABytes + kBBytes + (f * BN + (wn * TN + c) * 32 + r32) * 2);
+    }
   };
 
   f32x16 tot[TM][TN];
+  f32x16 part[G != 0 ? TM : 1][G != 0 ? TN : 1];
+  f32x16 canc[OFFS ? TM : 1];
 #pragma unroll
-  for (int a = 0; a < TM; ++a)
+  for (int a = 0; a < TM; ++a) {
 #pragma unroll
     for (int c = 0; c < TN; ++c)
 #pragma unroll
       for (int r = 0; r < 16; ++r) tot[a][c][r] = 0.0f;
+    if (OFFS) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) canc[a][r] = 0.0f;
+    }
+  }
+  uint32_t magic = Dequant<DT, BITS>::kMagic;
+  asm volatile("" : "+v"(magic));  // keep the constant in a VGPR
 
   // byte offsets inside a stage that do not change from tile to tile
   const int a_row_off = (wm * TM * 32 + r32) * (TK * 2);
   const int b_off = kABytes + (wn * TN * 2 + sp) * 1024 + (j + 16 * b) * 16;
-  constexpr int Q = TK / 16;  // 16-k slices (one MFMA per 32x32 block each) per tile
-  constexpr int kValuPerMfma = (BITS == 8 ? 16 : 12) * TN / (TM * TN) + 2;
+  constexpr int kValuPerMfma = ((BITS == 8 ? 16 : 12) * TN + TM * TN - 1) / (TM * TN) + 2;
+  constexpr int kHalf = (TM * TN + 1) / 2;  // MFMAs of a slice issued before the barrier
 
-  // The wavefront's pipeline registers: raw codes of the current tile, and
-  // two sets of operands -- the one the MFMAs of slice q use and the one being
-  // prepared for slice q+1 (A fragments read from LDS, B fragments dequantised).
+  // The wavefront's pipeline registers: raw codes of the current and the next
+  // tile, and two sets of operands -- the one the MFMAs of slice q use and the
+  // one being prepared for slice q+1 (A fragments read from LDS, B fragments
+  // dequantised).
   u32x4 braw[2][TN][2];
+  uint16_t sraw[kGT > 0 ? kGT : 1][TN];
   u32x4 af[2][TM];
   u32x4 bf[2][TN];
   auto read_b = [&](const unsigned char* stage, u32x4 (&dst)[TN][2]) {
@@ -468,16 +568,48 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
 #pragma unroll
     for (int c = 0; c < TN; ++c) {
       const uint32_t w4[4] = {raw[c][h].x, raw[c][h].y, raw[c][h].z, raw[c][h].w};
-      dst[c] = DequantExact<DT, BITS>::run(&w4[step * kDw]);
+      if (OFFS) dst[c] = Dequant<DT, BITS>::run(&w4[step * kDw], magic);
+      else dst[c] = DequantExact<DT, BITS>::run(&w4[step * kDw]);
     }
   };
-  // MFMAs of the A blocks [a_lo, a_hi) of a slice
-  auto mfmas = [&](const u32x4 (&a4)[TM], const u32x4 (&b4)[TN], int a_lo, int a_hi) {
+  // MFMAs lo .. hi-1 (numbered a * TN + c) of slice q
+  auto mfmas = [&](const u32x4 (&a4)[TM], const u32x4 (&b4)[TN], int q, int lo, int hi) {
+    const bool first = q % kFold == 0;
+    f32x16 zero;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) zero[r] = 0.0f;
 #pragma unroll
     for (int a = 0; a < TM; ++a)
-      if (a >= a_lo && a < a_hi)
 #pragma unroll
-        for (int c = 0; c < TN; ++c) tot[a][c] = mfma32<DT>(a4[a], b4[c], tot[a][c]);
+      for (int c = 0; c < TN; ++c)
+        if (a * TN + c >= lo && a * TN + c < hi) {
+          if (OFFS && c == 0) {
+            const u32x4 cb = {Dequant<DT, BITS>::kCancel, Dequant<DT, BITS>::kCancel,
+                              Dequant<DT, BITS>::kCancel, Dequant<DT, BITS>::kCancel};
+            canc[a] = mfma32<DT>(a4[a], cb, (G != 0 && first) ? zero : canc[a]);
+          }
+          if (G == 0) {
+            tot[a][c] = mfma32<DT>(a4[a], b4[c], tot[a][c]);
+          } else if (first) {
+            part[a][c] = mfma32<DT>(a4[a], b4[c], zero);
+          } else {
+            part[a][c] = mfma32<DT>(a4[a], b4[c], part[a][c]);
+          }
+        }
+  };
+  // after the last slice of a group: tot += part * scale
+  auto fold = [&](const uint16_t (&sr)[kGT > 0 ? kGT : 1][TN], int q) {
+    if (G != 0 && q % kFold == kFold - 1) {
+#pragma unroll
+      for (int c = 0; c < TN; ++c) {
+        const float sc = to_f32<DT>(sr[q / kFold][c]);
+#pragma unroll
+        for (int a = 0; a < TM; ++a)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            tot[a][c][r] = fmaf(OFFS ? part[a][c][r] + canc[a][r] : part[a][c][r], sc, tot[a][c][r]);
+      }
+    }
   };
 
   issue(0);
@@ -495,17 +627,17 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
   // tile it+3 sits in the middle of the last but one slice, once the
   // wavefront has fetched its last operands of the tile; the raw codes of tile
   // it+1 are read right behind it and have a whole slice to arrive.
-  static_assert(Q >= 2 && TM % 2 == 0, "the pipeline needs two slices per tile and an even TM");
   auto tile = [&](int it, u32x4 (&raw)[TN][2], u32x4 (&raw_next)[TN][2]) {
     const unsigned char* stage = smem + (it % kStages) * kStage;
     const unsigned char* next = smem + ((it + 1) % kStages) * kStage;
+    read_scales(stage, sraw);  // before the stage is handed over
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
       if (q != Q - 2) {
         const bool last = q == Q - 1;
         read_a(last ? next : stage, af[(q + 1) & 1], last ? 0 : q + 1);
         dequant(bf[(q + 1) & 1], last ? raw_next : raw, last ? 0 : q + 1);
-        mfmas(af[q & 1], bf[q & 1], 0, TM);
+        mfmas(af[q & 1], bf[q & 1], q, 0, TM * TN);
 #pragma unroll
         for (int i = 0; i < TM * TN; ++i) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                   // one MFMA
@@ -513,11 +645,12 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
           __builtin_amdgcn_sched_group_barrier(0x002, kValuPerMfma, 0);        // VALU
         }
         __builtin_amdgcn_sched_barrier(0);
+        fold(sraw, q);
       } else {
         read_a(stage, af[(q + 1) & 1], q + 1);
-        mfmas(af[q & 1], bf[q & 1], 0, TM / 2);
+        mfmas(af[q & 1], bf[q & 1], q, 0, kHalf);
 #pragma unroll
-        for (int i = 0; i < TM * TN / 2; ++i) {
+        for (int i = 0; i < kHalf; ++i) {
           if (2 * i < TM) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         }
@@ -531,10 +664,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
         issue(it + 3);
         read_b(next, raw_next);
         dequant(bf[(q + 1) & 1], raw, q + 1);
-        mfmas(af[q & 1], bf[q & 1], TM / 2, TM);
+        mfmas(af[q & 1], bf[q & 1], q, kHalf, TM * TN);
 #pragma unroll
-        for (int i = 0; i < TM * TN / 2; ++i) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        for (int i = 0; i < TM * TN - kHalf + 1; ++i) {
+          if (i < TM * TN - kHalf) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
           if (i < 2 * TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x002, 2 * kValuPerMfma, 0);
         }
@@ -551,17 +684,24 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
 
   // ---- epilogue: scale, bias, cast; 32-row slabs leave through LDS as 16-byte stores ----
   // accumulator element r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its block
-  const int col0 = (strip_blk + wn * TN * 2) * 16;  // first column of the wavefront
   float sc[TN], bv[TN];
 #pragma unroll
   for (int c = 0; c < TN; ++c) {
-    int n = col0 + c * 32 + r32;
-    n = n < n_hi ? n : n_hi - 1;
-    sc[c] = to_f32<DT>(scale[n]);
-    bv[c] = bias != nullptr ? to_f32<DT>(bias[n]) : 0.0f;
+    sc[c] = G == 0 ? to_f32<DT>(scale[ncol[c]]) : 1.0f;
+    bv[c] = (p.bias != nullptr && p.nsplit == 1) ? to_f32<DT>(p.bias[ncol[c]]) : 0.0f;
   }
-  if (out_f32) {  // verification mode: the accumulators themselves, plain stores
-    float* outf = static_cast<float*>(outv);
+  if (OFFS && G == 0) {
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+      for (int c = 0; c < TN; ++c)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) tot[a][c][r] += canc[a][r];
+  }
+  if (p.out_f32 || p.nsplit > 1) {
+    // fp32 results (verification mode) or partial sums of this run of k tiles: plain stores
+    float* outf = static_cast<float*>(p.out) +
+                  (p.nsplit > 1 ? static_cast<int64_t>(split) * M * N : 0);
 #pragma unroll
     for (int a = 0; a < TM; ++a)
 #pragma unroll
@@ -575,7 +715,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
       }
     return;
   }
-  uint16_t* out = static_cast<uint16_t*>(outv);
+  uint16_t* out = static_cast<uint16_t*>(p.out);
   constexpr int kSlabRow = TN * 32 + 8;  // padded, in elements
   static_assert(NW * 32 * kSlabRow * 2 <= kStages * kStage, "slabs must fit in the stage buffers");
   uint16_t* slab = reinterpret_cast<uint16_t*>(smem) + wave * 32 * kSlabRow;
@@ -590,8 +730,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
             cast_out<DT>(tot[a][c][r] * sc[c] + bv[c]);
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
-    for (int p = lane; p < kPieces; p += 64) {
-      const int r = p / (TN * 4), cc = p % (TN * 4);
+    for (int q = lane; q < kPieces; q += 64) {
+      const int r = q / (TN * 4), cc = q % (TN * 4);
       const int m = m0 + (wm * TM + a) * 32 + r;
       const int n = col0 + cc * 8;
       const u32x4 v = *reinterpret_cast<const u32x4*>(&slab[r * kSlabRow + cc * 8]);
@@ -602,10 +742,60 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(
 #endif
 }
 
+// out[m, n] = T( sum over the runs of part[run][m][n] + bias[n] ), four columns per thread
+template <int DT>
+__global__ __launch_bounds__(256) void reduce_partials_kernel(
+    const float* __restrict__ part, int nsplit, const uint16_t* __restrict__ bias,
+    void* __restrict__ out, int out_f32, int64_t total, int N) {
+  const int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
+  if (i >= total) return;
+  f32x4 s = {0.f, 0.f, 0.f, 0.f};
+  for (int r0 = 0; r0 < nsplit; r0 += 4) {  // four loads in flight, added in run order
+    f32x4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int r = r0 + u < nsplit ? r0 + u : nsplit - 1;
+      v[u] = *reinterpret_cast<const f32x4*>(part + r * total + i);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (r0 + u < nsplit) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) s[e] += v[u][e];
+      }
+  }
+  if (bias != nullptr) {
+    const int n = static_cast<int>(i % N);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) s[e] += to_f32<DT>(bias[n + e]);
+  }
+  if (out_f32) {
+    *reinterpret_cast<f32x4*>(static_cast<float*>(out) + i) = s;
+  } else {
+    u32x2 v;
+    v.x = cast_out<DT>(s[0]) | (static_cast<uint32_t>(cast_out<DT>(s[1])) << 16);
+    v.y = cast_out<DT>(s[2]) | (static_cast<uint32_t>(cast_out<DT>(s[3])) << 16);
+    *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(out) + i) = v;
+  }
+}
+
 struct Args {
   const void* x; const void* codes; const void* bias; const void* scale; void* out;
-  int M, K, N, gshift, out_f32; hipStream_t stream;
+  int M, K, N, gshift, out_f32;
+  void* ws; size_t ws_bytes;  // scratch for split-K partial sums, may be null
+  hipStream_t stream;
 };
+
+inline int num_cus() {
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    return n;
+  }();
+  return cus;
+}
 
 template <int DT, int BITS, bool GROUPED, int WM, int WN, int TM, int TN>
 void launch_one(const Args& a) {
@@ -625,24 +815,50 @@ void launch_one(const Args& a) {
       a.N, a.gshift, a.out_f32, nbx, nby);
 }
 
-// Launches the fast kernel on the columns of strips [strip_lo, strip_hi).
-template <int DT, int BITS, int WM, int WN, int TM, int TN>
-void launch_dma(const Args& a, int strip_lo, int strip_hi) {
+template <int BITS, int G, int WM, int WN, int TM, int TN>
+constexpr size_t dma_lds_bytes() {
+  return 3 * (static_cast<size_t>(WM * TM * 32) * (BITS == 8 ? 64 : 128) * 2 +
+              (WN * TN * 32 / 16) * 1024 + (G == 0 ? 0 : WM * WN * 256));
+}
+
+// Launches the fast kernel on the columns of strips [strip_lo, strip_hi), K
+// cut into nsplit runs (nsplit > 1 needs a.ws and covers every column).
+template <int DT, int BITS, int G, bool OFFS, int WM, int WN, int TM, int TN>
+void launch_dma(const Args& a, int strip_lo, int strip_hi, int nsplit) {
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32, TK = BITS == 8 ? 64 : 128;
   if (strip_hi <= strip_lo) return;
-  const int nbx = ((strip_hi - strip_lo) * kStripCols + BN - 1) / BN, nby = (a.M + BM - 1) / BM;
-  const size_t lds = 3 * (static_cast<size_t>(BM) * TK * 2 + (BN / 16) * 1024);
-  auto kern = gemm_dma_kernel<DT, BITS, WM, WN, TM, TN>;
+  constexpr size_t lds = dma_lds_bytes<BITS, G, WM, WN, TM, TN>();
+  auto kern = gemm_dma_kernel<DT, BITS, G, OFFS, WM, WN, TM, TN>;
   static bool configured = false;
   if (!configured) {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                               hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
     configured = true;
   }
-  kern<<<dim3(static_cast<unsigned>(nbx * nby)), dim3(64 * WM * WN), lds, a.stream>>>(
-      static_cast<const uint16_t*>(a.x), static_cast<const uint8_t*>(a.codes),
-      static_cast<const uint16_t*>(a.bias), static_cast<const uint16_t*>(a.scale),
-      a.out, a.M, a.K, a.N, a.out_f32, strip_lo, strip_hi, nbx, nby);
+  if (nsplit > 1 && (a.ws == nullptr ||
+                     a.ws_bytes < static_cast<size_t>(nsplit) * a.M * a.N * sizeof(float)))
+    nsplit = 1;  // never write past the scratch buffer
+  DmaParams p;
+  p.x = static_cast<const uint16_t*>(a.x);
+  p.codes = static_cast<const uint8_t*>(a.codes);
+  p.bias = static_cast<const uint16_t*>(a.bias);
+  p.scale = static_cast<const uint16_t*>(a.scale);
+  p.out = nsplit > 1 ? a.ws : a.out;
+  p.M = a.M; p.K = a.K; p.N = a.N;
+  p.out_f32 = a.out_f32;
+  p.strip_lo = strip_lo; p.strip_hi = strip_hi;
+  p.nbx = ((strip_hi - strip_lo) * kStripCols + BN - 1) / BN;
+  p.nby = (a.M + BM - 1) / BM;
+  const int tiles = a.K / TK;
+  p.tiles_per_split = (tiles + nsplit - 1) / nsplit;
+  p.nsplit = (tiles + p.tiles_per_split - 1) / p.tiles_per_split;
+  p.rotate = p.nby == 1 ? 1 : 0;  // with several row blocks the L2 reuse of A wants them in step
+  kern<<<dim3(static_cast<unsigned>(p.nbx * p.nby * p.nsplit)), dim3(64 * WM * WN), lds, a.stream>>>(p);
+  if (nsplit > 1) {
+    const int64_t total = static_cast<int64_t>(a.M) * a.N;
+    reduce_partials_kernel<DT><<<dim3(static_cast<unsigned>((total / 4 + 255) / 256)), dim3(256), 0, a.stream>>>(
+        static_cast<const float*>(a.ws), p.nsplit, p.bias, a.out, a.out_f32, total, a.N);
+  }
 }
 
 // Number of 256-column tiles given to the 256-row kernel; the remaining
@@ -651,13 +867,7 @@ void launch_dma(const Args& a, int strip_lo, int strip_hi) {
 // 256-row one (more than half: the dequantised B operand is shared by fewer
 // MFMAs).
 inline int plan_big_columns(int M, int N) {
-  static const int cus = [] {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-      n = 256;
-    return n;
-  }();
+  const int cus = num_cus();
   constexpr double kSmall = 0.56;
   const int nbx = (N + 255) / 256, nby_big = (M + 255) / 256, nby_small = (M + 127) / 128;
   int best = nbx;
@@ -670,22 +880,72 @@ inline int plan_big_columns(int M, int N) {
   return best;
 }
 
+// Rows up to which the small-M configurations (one row block of 32 or 64
+// rows, 256 columns, K split across workgroups) are used.
+constexpr int kSkinnyMaxM = 64;
+
+// Split of K for the small-M configurations: the number of runs that
+// minimises rounds-of-workgroups x (k tiles per run + fixed cost), at most 16
+// runs of at least 4 k tiles, and no more than the scratch buffer allows.
+inline int plan_split(int M, int K, int N, int bits, size_t lds, size_t ws_bytes) {
+  const int tk = bits == 8 ? 64 : 128, tiles = K / tk;
+  const int nbx = (N + 255) / 256;
+  const int per_cu = static_cast<int>((160 * 1024) / lds) > 0 ? static_cast<int>((160 * 1024) / lds) : 1;
+  const int slots = num_cus() * per_cu;
+  const size_t per_run = static_cast<size_t>(M) * N * sizeof(float);
+  int best = 1;
+  int64_t best_cost = INT64_MAX;
+  for (int ns = 1; ns <= 16; ++ns) {
+    const int tps = (tiles + ns - 1) / ns;
+    const int eff = (tiles + tps - 1) / tps;
+    if (eff != ns || (ns > 1 && tps < 4)) continue;
+    if (ns > 1 && per_run * ns > ws_bytes) continue;
+    const int64_t rounds = (static_cast<int64_t>(nbx) * ns + slots - 1) / slots;
+    const int64_t cost = rounds * (tps + 2) * 8 + ns;  // the last term prefers fewer runs on ties
+    if (cost < best_cost) { best_cost = cost; best = ns; }
+  }
+  return best;
+}
+
+template <int BITS>
+size_t skinny_lds(int M) {  // with group scales (the larger footprint)
+  if (BITS == 4 && M <= 32) return dma_lds_bytes<4, 64, 1, 8, 1, 1>();
+  return dma_lds_bytes<BITS, 64, 1, 8, 2, 1>();
+}
+
+template <int DT, int BITS, int G>
+void launch_fast(const Args& a) {
+  const int nstrips = a.N / kStripCols;
+  if (a.M <= kSkinnyMaxM) {
+    const int ns = plan_split(a.M, a.K, a.N, BITS, skinny_lds<BITS>(a.M), a.ws != nullptr ? a.ws_bytes : 0);
+    if constexpr (BITS == 4) {
+      if (a.M <= 32) { launch_dma<DT, BITS, G, true, 1, 8, 1, 1>(a, 0, nstrips, ns); return; }
+    }
+    launch_dma<DT, BITS, G, false, 1, 8, 2, 1>(a, 0, nstrips, ns);
+    return;
+  }
+  if constexpr (BITS == 8 && G == 0) {
+    // 256 x 256 x 64 tiles (144 KiB of LDS, one workgroup per CU) for as many
+    // column tiles as fill whole rounds of the CUs; the rest, which would
+    // leave CUs idle for a whole tile time, goes to 128 x 256 tiles.
+    const int c = plan_big_columns(a.M, a.N);
+    const int hi = c * 16 < nstrips ? c * 16 : nstrips;
+    launch_dma<DT, BITS, G, false, 2, 4, 4, 2>(a, 0, hi, 1);
+    launch_dma<DT, BITS, G, false, 2, 4, 2, 2>(a, hi, nstrips, 1);
+  } else {
+    // int4 tiles are 128 k deep and group-wise scales need a second set of
+    // accumulators: 128 x 256 tiles
+    launch_dma<DT, BITS, G, false, 2, 4, 2, 2>(a, 0, nstrips, 1);
+  }
+}
+
 template <int DT, int BITS>
 void launch_cfg(const Args& a) {
   constexpr int TK = BITS == 8 ? 64 : 128;
-  if (a.gshift < 0 && a.K % TK == 0 && a.K / TK >= 2) {
-    const int nstrips = a.N / kStripCols;
-    if constexpr (BITS == 8) {
-      // 256 x 256 x 64 tiles (144 KiB of LDS, one workgroup per CU) for as many
-      // column tiles as fill whole rounds of the CUs; the rest, which would
-      // leave CUs idle for a whole tile time, goes to 128 x 256 tiles.
-      const int c = plan_big_columns(a.M, a.N);
-      const int hi = c * 16 < nstrips ? c * 16 : nstrips;
-      launch_dma<DT, BITS, 2, 4, 4, 2>(a, 0, hi);
-      launch_dma<DT, BITS, 2, 4, 2, 2>(a, hi, nstrips);
-    } else {
-      launch_dma<DT, BITS, 2, 4, 2, 2>(a, 0, nstrips);   // 128 x 256 x 128: 144 KiB of LDS
-    }
+  if (a.K % TK == 0 && a.K / TK >= 2) {
+    if (a.gshift < 0) launch_fast<DT, BITS, 0>(a);
+    else if (a.gshift == 6) launch_fast<DT, BITS, 64>(a);
+    else launch_fast<DT, BITS, 128>(a);
     return;
   }
   if (a.gshift >= 0) {
@@ -697,12 +957,21 @@ void launch_cfg(const Args& a) {
 
 }  // namespace
 
+size_t linear_gemm_workspace(int64_t M, int64_t K, int64_t N, int bits) {
+  const int tk = bits == 8 ? 64 : 128;
+  if (M > kSkinnyMaxM || K % tk != 0 || K / tk < 2) return 0;
+  const size_t lds = bits == 8 ? skinny_lds<8>(static_cast<int>(M)) : skinny_lds<4>(static_cast<int>(M));
+  const int ns = plan_split(static_cast<int>(M), static_cast<int>(K), static_cast<int>(N), bits, lds, SIZE_MAX);
+  return ns > 1 ? static_cast<size_t>(ns) * M * N * sizeof(float) : 0;
+}
+
 int launch_linear_gemm(const void* x, const void* codes, const void* bias, const void* scale,
                        int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
-                       void* out, bool out_f32, hipStream_t stream) {
+                       void* out, bool out_f32, void* workspace, size_t workspace_bytes,
+                       hipStream_t stream) {
   const int gshift = group_size == 64 ? 6 : (group_size == 128 ? 7 : -1);
   const Args a{x, codes, bias, scale, out, static_cast<int>(M), static_cast<int>(K),
-               static_cast<int>(N), gshift, out_f32 ? 1 : 0, stream};
+               static_cast<int>(N), gshift, out_f32 ? 1 : 0, workspace, workspace_bytes, stream};
   if (dtype == WOL_DTYPE_BF16) {
     if (bits == 8) launch_cfg<WOL_DTYPE_BF16, 8>(a); else launch_cfg<WOL_DTYPE_BF16, 4>(a);
   } else {

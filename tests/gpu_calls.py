@@ -41,7 +41,7 @@ def repack(codes_u8, layout_in, layout_out, K, N, bits):
     return o.cpu().numpy()
 
 
-def linear(x_bits, codes_u8, bias_bits, scale_bits, dt, N, bits, g, f32=False):
+def linear(x_bits, codes_u8, bias_bits, scale_bits, dt, N, bits, g, f32=False, no_workspace=False):
     """codes_u8 in gfx950 layout.  Returns fp32 numpy [M,N] (f32=True) or T bits."""
     x = H.bits_to_torch(x_bits, dt, DEV)
     M, K = x.shape
@@ -54,7 +54,9 @@ def linear(x_bits, codes_u8, bias_bits, scale_bits, dt, N, bits, g, f32=False):
     else:
         out = torch.full((M, N), float("nan"), dtype=x.dtype, device=DEV)
         fn = _lib.lib.wol_linear
+    wsb = 0 if no_workspace else _lib.lib.wol_linear_workspace(M, K, N, bits, g)
+    ws = torch.empty(wsb, dtype=torch.uint8, device=DEV) if wsb else None
     _lib.check(fn(x.data_ptr(), c.data_ptr(), None if b is None else b.data_ptr(), s.data_ptr(), dt, M, K, N, bits, g,
-                  out.data_ptr(), None, 0, None))
+                  out.data_ptr(), None if ws is None else ws.data_ptr(), wsb, None))
     torch.cuda.synchronize()
     return out.cpu().numpy() if f32 else H.torch_to_bits(out)
