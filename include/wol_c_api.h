@@ -118,7 +118,10 @@ int wol_dequantize(const void* codes, int layout, const void* scale, int dtype,
                    int64_t K, int64_t N, int bits, int group_size,
                    void* out_KN, void* stream);
 
-/* Bytes of device scratch wol_linear needs for this problem (may be 0). */
+/* Bytes of device scratch wol_linear can use for this problem (may be 0).  The
+ * scratch is optional: without it (NULL or fewer bytes) the result is the
+ * same to fp32 summation order and only the speed of small-M problems drops,
+ * because K can no longer be split across workgroups.  Must be 16-byte aligned. */
 size_t wol_linear_workspace(int64_t M, int64_t K, int64_t N, int bits,
                             int group_size);
 
@@ -127,8 +130,10 @@ size_t wol_linear_workspace(int64_t M, int64_t K, int64_t N, int bits,
  * fp32 accumulation, one round-to-nearest-even cast to T at the end.
  * codes must be in GFX950 layout.  bias may be NULL.
  * scale: [N] T (group_size -1) or [ceil(K/g),N] T, as wol_quantize wrote it.
- * M <= 64 takes the streaming (HBM-bound) kernel, larger M the MFMA GEMM; the
+ * M <= 8 takes the streaming (HBM-bound) kernel, M > 64 the MFMA GEMM, and in
+ * between whichever a cost model of the two predicts to be faster; the
  * reference's split is M <= 3 (gpu/weight_only_linear_kernel.cu:60-61).
+ * x, codes and scale must be 16-byte aligned.
  */
 int wol_linear(const void* x, const void* codes, const void* bias,
                const void* scale, int dtype, int64_t M, int64_t K, int64_t N,
@@ -142,6 +147,27 @@ int wol_linear_f32(const void* x, const void* codes, const void* bias,
                    const void* scale, int dtype, int64_t M, int64_t K,
                    int64_t N, int bits, int group_size, float* out_f32,
                    void* workspace, size_t workspace_bytes, void* stream);
+
+/* Kernel choice of wol_linear_on. */
+enum wol_kernel {
+  WOL_KERNEL_AUTO = 0,   /* what wol_linear does                                */
+  WOL_KERNEL_STREAM = 1, /* the streaming kernel; M <= 64 only                  */
+  WOL_KERNEL_GEMM = 2    /* the MFMA GEMM                                       */
+};
+
+/*
+ * wol_linear / wol_linear_f32 with the kernel choice pinned: out is [M,N] T
+ * (out_is_f32 == 0) or float.  No counterpart in the reference; it exists so
+ * that both kernels can be timed and verified on the same problem.
+ * wol_linear_workspace_for is the matching scratch query.
+ */
+size_t wol_linear_workspace_for(int64_t M, int64_t K, int64_t N, int bits,
+                                int group_size, int kernel);
+int wol_linear_on(const void* x, const void* codes, const void* bias,
+                  const void* scale, int dtype, int64_t M, int64_t K, int64_t N,
+                  int bits, int group_size, void* out, int out_is_f32,
+                  int kernel, void* workspace, size_t workspace_bytes,
+                  void* stream);
 
 /*
  * Re-lays a code tensor between layouts (any pair of the three).  It is a

@@ -23,6 +23,8 @@ SYMBOLS = (
     "wol_linear_workspace",
     "wol_linear",
     "wol_linear_f32",
+    "wol_linear_workspace_for",
+    "wol_linear_on",
     "wol_repack",
     "wol_code_offset",
 )
@@ -56,6 +58,10 @@ def _load():
     lib.wol_linear.restype = ci
     lib.wol_linear_f32.argtypes = [vp, vp, vp, vp, ci, i64, i64, i64, ci, ci, vp, vp, sz, vp]
     lib.wol_linear_f32.restype = ci
+    lib.wol_linear_workspace_for.argtypes = [i64, i64, i64, ci, ci, ci]
+    lib.wol_linear_workspace_for.restype = sz
+    lib.wol_linear_on.argtypes = [vp, vp, vp, vp, ci, i64, i64, i64, ci, ci, vp, ci, ci, vp, sz, vp]
+    lib.wol_linear_on.restype = ci
     lib.wol_repack.argtypes = [vp, ci, vp, ci, i64, i64, ci, vp]
     lib.wol_repack.restype = ci
     lib.wol_code_offset.argtypes = [ci, i64, i64, ci, i64, i64, ctypes.POINTER(ci)]
@@ -68,6 +74,9 @@ lib = _load()
 # statuses that are argument errors (the reference raises InvalidArgument,
 # which Paddle surfaces as ValueError)
 _ARG_ERRORS = {1, 2, 3, 4, 5, 6, 7, 8, 9}
+
+# wol_kernel
+KERNEL_AUTO, KERNEL_STREAM, KERNEL_GEMM = 0, 1, 2
 
 
 def check(status):

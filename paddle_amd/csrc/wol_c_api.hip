@@ -48,18 +48,28 @@ bool use_stream(int64_t M, int64_t K, int64_t N, int bits) {
   return t_stream <= t_gemm;
 }
 
+// kernel: a wol_kernel; AUTO resolves by M and the cost model
+bool resolve_stream(int kernel, int64_t M, int64_t K, int64_t N, int bits) {
+  if (kernel == WOL_KERNEL_STREAM) return true;
+  if (kernel == WOL_KERNEL_GEMM) return false;
+  return use_stream(M, K, N, bits);
+}
+
 int linear_impl(const void* x, const void* codes, const void* bias, const void* scale, int dtype,
                 int64_t M, int64_t K, int64_t N, int bits, int group_size, void* out, bool out_f32,
-                void* workspace, size_t workspace_bytes, void* stream) {
+                int kernel, void* workspace, size_t workspace_bytes, void* stream) {
   const int rc = check_problem(dtype, K, N, bits, group_size);
   if (rc != WOL_OK) return rc;
   if (M < 0 || M > (int64_t{1} << 30)) return WOL_ERR_BAD_SHAPE;
+  if (kernel != WOL_KERNEL_AUTO && kernel != WOL_KERNEL_STREAM && kernel != WOL_KERNEL_GEMM)
+    return WOL_ERR_BAD_SHAPE;
+  if (kernel == WOL_KERNEL_STREAM && M > kStreamMaxM) return WOL_ERR_BAD_SHAPE;
   if (M == 0) return WOL_OK;  // empty batch: nothing to write
   if (x == nullptr || codes == nullptr || scale == nullptr || out == nullptr)
     return WOL_ERR_NULL_POINTER;
   if (!aligned16(x) || !aligned16(codes) || !aligned16(scale)) return WOL_ERR_ALIGNMENT;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (use_stream(M, K, N, bits))
+  if (resolve_stream(kernel, M, K, N, bits))
     return wol::launch_linear_stream(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out,
                                      out_f32, s);
   if (workspace == nullptr || !aligned16(workspace)) workspace_bytes = 0;  // optional: only speeds up
@@ -124,8 +134,14 @@ int wol_dequantize(const void* codes, int layout, const void* scale, int dtype, 
 }
 
 size_t wol_linear_workspace(int64_t M, int64_t K, int64_t N, int bits, int group_size) {
+  return wol_linear_workspace_for(M, K, N, bits, group_size, WOL_KERNEL_AUTO);
+}
+
+size_t wol_linear_workspace_for(int64_t M, int64_t K, int64_t N, int bits, int group_size,
+                                int kernel) {
   if (check_problem(WOL_DTYPE_F16, K, N, bits, group_size) != WOL_OK || M <= 0) return 0;
-  if (use_stream(M, K, N, bits)) return 0;  // partial sums stay on chip
+  if (kernel == WOL_KERNEL_STREAM && M > kStreamMaxM) return 0;
+  if (resolve_stream(kernel, M, K, N, bits)) return 0;  // partial sums stay on chip
   return wol::linear_gemm_workspace(M, K, N, bits);
 }
 
@@ -133,14 +149,22 @@ int wol_linear(const void* x, const void* codes, const void* bias, const void* s
                int64_t M, int64_t K, int64_t N, int bits, int group_size, void* out,
                void* workspace, size_t workspace_bytes, void* stream) {
   return linear_impl(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out, false,
-                     workspace, workspace_bytes, stream);
+                     WOL_KERNEL_AUTO, workspace, workspace_bytes, stream);
 }
 
 int wol_linear_f32(const void* x, const void* codes, const void* bias, const void* scale,
                    int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
                    float* out_f32, void* workspace, size_t workspace_bytes, void* stream) {
   return linear_impl(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out_f32, true,
-                     workspace, workspace_bytes, stream);
+                     WOL_KERNEL_AUTO, workspace, workspace_bytes, stream);
+}
+
+int wol_linear_on(const void* x, const void* codes, const void* bias, const void* scale, int dtype,
+                  int64_t M, int64_t K, int64_t N, int bits, int group_size, void* out,
+                  int out_is_f32, int kernel, void* workspace, size_t workspace_bytes,
+                  void* stream) {
+  return linear_impl(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out,
+                     out_is_f32 != 0, kernel, workspace, workspace_bytes, stream);
 }
 
 int wol_repack(const void* codes_in, int layout_in, void* codes_out, int layout_out, int64_t K,

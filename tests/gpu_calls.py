@@ -41,22 +41,33 @@ def repack(codes_u8, layout_in, layout_out, K, N, bits):
     return o.cpu().numpy()
 
 
-def linear(x_bits, codes_u8, bias_bits, scale_bits, dt, N, bits, g, f32=False, no_workspace=False):
-    """codes_u8 in gfx950 layout.  Returns fp32 numpy [M,N] (f32=True) or T bits."""
+def linear(x_bits, codes_u8, bias_bits, scale_bits, dt, N, bits, g, f32=False, no_workspace=False,
+           kernel=None, ws_bytes=None):
+    """codes_u8 in gfx950 layout.  Returns fp32 numpy [M,N] (f32=True) or T bits.
+    kernel pins the streaming (1) or GEMM (2) kernel through wol_linear_on;
+    ws_bytes overrides the size of the scratch buffer handed in."""
     x = H.bits_to_torch(x_bits, dt, DEV)
     M, K = x.shape
     c = torch.from_numpy(np.ascontiguousarray(codes_u8)).to(DEV)
     s = H.bits_to_torch(scale_bits, dt, DEV)
     b = None if bias_bits is None else H.bits_to_torch(bias_bits, dt, DEV)
-    if f32:
-        out = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
-        fn = _lib.lib.wol_linear_f32
+    out = torch.full((M, N), float("nan"), dtype=torch.float32 if f32 else x.dtype, device=DEV)
+    if kernel is None:
+        wsb = _lib.lib.wol_linear_workspace(M, K, N, bits, g)
     else:
-        out = torch.full((M, N), float("nan"), dtype=x.dtype, device=DEV)
-        fn = _lib.lib.wol_linear
-    wsb = 0 if no_workspace else _lib.lib.wol_linear_workspace(M, K, N, bits, g)
-    ws = torch.empty(wsb, dtype=torch.uint8, device=DEV) if wsb else None
-    _lib.check(fn(x.data_ptr(), c.data_ptr(), None if b is None else b.data_ptr(), s.data_ptr(), dt, M, K, N, bits, g,
-                  out.data_ptr(), None if ws is None else ws.data_ptr(), wsb, None))
+        wsb = _lib.lib.wol_linear_workspace_for(M, K, N, bits, g, kernel)
+    if no_workspace:
+        wsb = 0
+    if ws_bytes is not None:
+        wsb = ws_bytes
+    ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device=DEV) if wsb else None
+    args = (x.data_ptr(), c.data_ptr(), None if b is None else b.data_ptr(), s.data_ptr(), dt, M, K, N, bits, g,
+            out.data_ptr())
+    tail = (None if ws is None else ws.data_ptr(), wsb, None)
+    if kernel is None:
+        fn = _lib.lib.wol_linear_f32 if f32 else _lib.lib.wol_linear
+        _lib.check(fn(*args, *tail))
+    else:
+        _lib.check(_lib.lib.wol_linear_on(*args, 1 if f32 else 0, kernel, *tail))
     torch.cuda.synchronize()
     return out.cpu().numpy() if f32 else H.torch_to_bits(out)

@@ -22,15 +22,15 @@ def G(device):
     return gpu_calls
 
 
-def check(G, oracle, dt, bits, g, M, K, N, bias=True, seed=0, outliers=0.0, tol32=2e-5):
+def check(G, oracle, dt, bits, g, M, K, N, bias=True, seed=0, outliers=0.0, tol32=2e-5, **kw):
     wb = H.make_weight(K, N, dt, seed=seed + K + N, outlier_cols=outliers)
     xb = H.make_act(M, K, dt, seed=seed + M)
     bb = H.make_bias(N, dt, seed=seed + 1) if bias else None
     oc, osc = oracle.weight_quantize(wb, dt, bits, g)
     packed = H.gfx950_from_q(H.q_from_canonical(oc, bits), bits)
     r32, rT = oracle.linear(xb, oc, osc, bb, dt, bits, g)
-    got32 = G.linear(xb, packed, bb, osc, dt, N, bits, g, f32=True)
-    gotT = G.linear(xb, packed, bb, osc, dt, N, bits, g, f32=False)
+    got32 = G.linear(xb, packed, bb, osc, dt, N, bits, g, f32=True, **kw)
+    gotT = G.linear(xb, packed, bb, osc, dt, N, bits, g, f32=False, **kw)
     e32 = H.rel_l2(got32, r32)
     eT = H.rel_l2(H.bits_to_f32(gotT, dt), H.bits_to_f32(rT, dt))
     assert np.isfinite(got32).all()
@@ -53,6 +53,60 @@ def test_linear_small_shapes_all_m(G, oracle, dt, bits, g):
         for M in (1, 2, 3, 4, 7, 8, 15, 16, 17, 33, 48, 64, 65, 100, 300):
             print("case", dt, bits, g, K, N, M, flush=True)
             check(G, oracle, dt, bits, g, M, K, N, bias=(M % 2 == 1), seed=M)
+
+
+KERNEL_STREAM, KERNEL_GEMM = 1, 2
+
+
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("g", [-1, 64, 128])
+def test_linear_gemm_kernel_small_m(G, oracle, dt, bits, g):
+    # the MFMA GEMM pinned on the row counts that the cost model would hand to
+    # the streaming kernel at these sizes: one row block of 32 or 64 rows, K
+    # split across workgroups (512 / 64 = 8 k tiles for int8, 1024 / 128 = 8 for
+    # int4), ragged N (not a multiple of the 256-column tile), with and without bias
+    for K, N in [(512, 1024), (1024, 288), (1024, 1056)]:
+        if bits == 4 and N % 32:
+            continue
+        for M in (1, 9, 16, 31, 32, 33, 64):
+            print("case", dt, bits, g, K, N, M, flush=True)
+            check(G, oracle, dt, bits, g, M, K, N, bias=(M % 2 == 1), seed=M, kernel=KERNEL_GEMM)
+
+
+def test_linear_gemm_split_k_scratch_sizes(G, oracle):
+    # the scratch buffer is optional: with none, or one that holds fewer runs
+    # than planned, the same problem still comes out right (K is split less)
+    dt, bits, g, M, K, N = H.BF16, 8, 64, 24, 2048, 512
+    from paddle_amd import _lib
+    full = _lib.lib.wol_linear_workspace_for(M, K, N, bits, g, KERNEL_GEMM)
+    assert full >= 2 * M * N * 4 and full % (M * N * 4) == 0
+    for wsb in (0, M * N * 4, 2 * M * N * 4, full - 4, full):
+        check(G, oracle, dt, bits, g, M, K, N, seed=3, kernel=KERNEL_GEMM, ws_bytes=wsb)
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+def test_linear_stream_kernel_pinned_large_m(G, oracle, bits):
+    # the streaming kernel up to its limit of 64 rows, and the refusal beyond
+    for M in (17, 48, 64):
+        check(G, oracle, H.F16, bits, 128, M, 512, 256, seed=M, kernel=KERNEL_STREAM)
+    with pytest.raises(ValueError):
+        check(G, oracle, H.F16, bits, 128, 65, 512, 256, seed=1, kernel=KERNEL_STREAM)
+
+
+def test_both_kernels_agree_on_full_size_decode_shape(G, oracle):
+    # LLaMA-7B FFN shape at M = 16 (where the two kernels' costs cross): the
+    # two fp32 results differ only by summation order
+    dt, bits, g, M, K, N = H.BF16, 4, 128, 16, 4096, 11008
+    wb = H.make_weight(K, N, dt, seed=77)
+    xb = H.make_act(M, K, dt, seed=78)
+    oc, osc = oracle.weight_quantize(wb, dt, bits, g)
+    packed = H.gfx950_from_q(H.q_from_canonical(oc, bits), bits)
+    a = G.linear(xb, packed, None, osc, dt, N, bits, g, f32=True, kernel=KERNEL_STREAM)
+    b = G.linear(xb, packed, None, osc, dt, N, bits, g, f32=True, kernel=KERNEL_GEMM)
+    assert H.rel_l2(a, b) <= 5e-6  # each carries ~1.5e-6 of offset-cancellation rounding
+    r32, _ = oracle.linear(xb, oc, osc, None, dt, bits, g)
+    assert H.rel_l2(b, r32) <= 2e-5
 
 
 # The reference's own test matrix (test/quantization/test_weight_only_linear.py:

@@ -46,7 +46,15 @@ def test_workspace_queries(lib):
     assert L.wol_quantize_workspace(4096, 11008, 4, -1) == 4 * 11008
     assert L.wol_quantize_workspace(4096, 11008, 4, 128) == 0
     assert L.wol_quantize_workspace(4095, 11008, 4, 128) == 0  # invalid shape
-    assert L.wol_linear_workspace(1, 4096, 11008, 4, 128) == 0
+    assert L.wol_linear_workspace(1, 4096, 11008, 4, 128) == 0       # streaming kernel
+    assert L.wol_linear_workspace(2048, 4096, 12288, 8, -1) == 0     # one workgroup per tile covers all of K
+    # small M on the GEMM: whole fp32 [M, N] partial buffers, at most 16 of them
+    for M, K, N, bits, g in [(64, 8192, 28672, 4, 128), (32, 4096, 11008, 4, -1), (16, 8192, 28672, 4, 128)]:
+        need = L.wol_linear_workspace(M, K, N, bits, g)
+        assert need == L.wol_linear_workspace_for(M, K, N, bits, g, lib.KERNEL_GEMM)
+        assert need % (M * N * 4) == 0 and 2 <= need // (M * N * 4) <= 16, (M, K, N, need)
+    assert L.wol_linear_workspace_for(16, 4096, 11008, 4, 128, lib.KERNEL_STREAM) == 0
+    assert L.wol_linear_workspace_for(16, 4160, 11008, 4, 128, lib.KERNEL_GEMM) == 0  # K not a multiple of the k tile
 
 
 def test_argument_errors_return_before_device_work(lib):
@@ -67,7 +75,13 @@ def test_argument_errors_return_before_device_work(lib):
                                     kw.get("N", 16), kw.get("bits", 4), kw.get("g", -1), p, None, 0, None)
     assert lin(dt=5) == 2 and lin(bits=2) == 3 and lin(g=100) == 4 and lin(K=100) == 5 and lin(M=-1) == 5
     assert lin(x=None) == 1
+    assert lin(x=ctypes.c_void_p(0x1004)) == 9
     assert lin(M=0) == 0  # empty batch is a no-op
+    on = lambda **kw: L.wol_linear_on(p, p, None, kw.get("scale", p), 1, kw.get("M", 1), 64, 16, 4, -1, p, 0,
+                                      kw.get("kernel", 0), None, 0, None)
+    assert on(kernel=3) == 5 and on(kernel=-1) == 5
+    assert on(kernel=lib.KERNEL_STREAM, M=65) == 5  # the streaming kernel stops at 64 rows
+    assert on(scale=ctypes.c_void_p(0x1002)) == 9
     assert L.wol_dequantize(p, 9, p, 0, 64, 16, 8, -1, p, None) == 6
     assert L.wol_repack(p, 0, p, 2, 64, 16, 8, None) == 6  # in-place is refused
     assert L.wol_repack(p, 0, ctypes.c_void_p(0x2000), 2, 64, 24, 8, None) == 5
