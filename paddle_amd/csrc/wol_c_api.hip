@@ -42,9 +42,10 @@ bool use_stream(int64_t M, int64_t K, int64_t N, int bits) {
   if (M <= kStreamAlwaysM || !gemm_fast_path(K, bits)) return true;
   const double w = static_cast<double>(K) * N * bits / 8.0;           // weight bytes
   const double rows = static_cast<double>((M + 15) / 16 * 16);
-  const double a = static_cast<double>(N / 16) * rows * K * 2.0;      // activation bytes re-read
-  const double t_stream = (w / 5.0e6 > a / 8.0e6 ? w / 5.0e6 : a / 8.0e6) + 3.0;
-  const double t_gemm = w / 4.3e6 + 11.0;
+  const double a = static_cast<double>(N / 16) * rows * K * 2.0 /     // activation bytes re-read
+                   wol::stream_strips_per_workgroup(M, N, bits);
+  const double t_stream = (w + a) / 8.8e6 + 4.5;  // everything through L2 at ~8.8 TB/s
+  const double t_gemm = w / 4.1e6 + 10.4;         // two launches, K runs of a few k tiles each
   return t_stream <= t_gemm;
 }
 

@@ -181,6 +181,20 @@ __device__ inline uint16_t cast_out(float f) {
   return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
 }
 
+// Strips (16 columns) that share a workgroup of the streaming linear kernel.
+// Two halve the activation traffic out of L2 (N/16 * rows * K * 2 bytes, rows
+// = M rounded up to a power of two, at most 16 per operand) but also the
+// number of workgroups: worth it once that traffic is at least twice the
+// weight bytes (rows / bits >= 2) and enough workgroups remain.
+inline int stream_strips_per_workgroup(int64_t M, int64_t N, int bits) {
+  int rows = 1;
+  while (rows < 16 && rows < M) rows *= 2;
+  const int64_t groups = N / kStripCols / 2;
+  if (rows >= 4 * bits) return groups >= 256 ? 2 : 1;
+  if (rows >= 2 * bits) return groups >= 384 ? 2 : 1;
+  return 1;
+}
+
 // Launchers implemented in the .hip files; each returns a wol_status.
 int launch_quantize(const void* w, int dtype, int64_t K, int64_t N, int bits, int group_size,
                     int round_mode, int layout, void* codes, void* scale, void* workspace,

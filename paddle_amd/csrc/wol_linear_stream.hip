@@ -62,7 +62,11 @@ __device__ inline float sum_lane_groups(float v, bool x16, bool x32) {
 // once (the whole problem is in flight from the first cycle; used when K is
 // small enough).  NU == 0: a wavefront walks its share of the units with the
 // loads of the next unit in flight while it consumes the current one.
-template <int DT, int BITS, int MP, int MT, int WK, int NU, bool GROUPED>
+//
+// TN strips (16 columns each) share one workgroup and with it every load of
+// the activations: the activation traffic out of L2, which grows with M, drops
+// by TN.
+template <int DT, int BITS, int MP, int MT, int WK, int NU, int TN, bool GROUPED>
 struct StreamKernel {
   static_assert(MT == 1 || MP == 16, "several M tiles only with full 16-row operands");
   static constexpr int kS = 16 / MP;                  // k steps sharing one A operand
@@ -85,18 +89,19 @@ struct StreamKernel {
   const uint16_t* scale;
   int M, K, N;
   int gshift;  // log2(group_size) when GROUPED
-  int lane, j, kb, n;
+  int lane, j, kb;
+  int n[TN];  // this lane's column in each strip (clamped to the last valid one)
   uint32_t magic;
   // totc[mt][c] gathers the steps whose results belong to lane group c (for
   // MP = 8: lane groups 2c, 2c+1); lanes outside that group accumulate sums
   // that are discarded when the classes are merged at the end.
-  f32x4 totc[MT][kClasses];
+  f32x4 totc[TN][MT][kClasses];
 
   // Everything one unit of work (kU k steps of this strip) reads from memory.
   struct Unit {
-    u32x4 wv[kNT];
+    u32x4 wv[TN][kNT];
     u32x4 av[kNA][MT];
-    uint16_t sraw[kNS];
+    uint16_t sraw[TN][kNS];
   };
 
   // A operand whose row group `slot` holds k step (step0 + slot); with
@@ -112,9 +117,9 @@ struct StreamKernel {
     return *reinterpret_cast<const u32x4*>(x + static_cast<int64_t>(m) * K + step * 32 + 8 * kb);
   }
 
-  __device__ inline uint16_t load_scale_raw(int step) const {
-    const uint16_t* row = scale + static_cast<int64_t>((step * 32) >> gshift) * N;  // uniform
-    return row[n];
+  __device__ inline uint16_t load_scale_raw(int step, int t) const {
+    const uint16_t* row = scale + static_cast<int64_t>((step * 32) >> gshift) * N;
+    return row[n[t]];
   }
 
   // Index into Unit::sraw of the scale that step s of a unit uses.
@@ -125,7 +130,7 @@ struct StreamKernel {
   // The small loads (activations, scales) go first: the memory system returns
   // loads in order, so the first weight tile can be consumed while the later
   // ones are still on their way.
-  __device__ inline void load_unit(Unit& d, const u32x4* tp, int u) const {
+  __device__ inline void load_unit(Unit& d, const u32x4* const (&tp)[TN], int u) const {
     const int step0 = u * kU;
 #pragma unroll
     for (int a = 0; a < kNA; ++a)
@@ -137,12 +142,15 @@ struct StreamKernel {
       for (int p = 0; p < kNS; ++p) {
         const int step = MP == 16 ? step0 + 2 * p
                                   : step0 + (p / kPairs) * kS + mine * kRowsPerGroup + 2 * (p % kPairs);
-        d.sraw[p] = load_scale_raw(step);
+#pragma unroll
+        for (int t = 0; t < TN; ++t) d.sraw[t][p] = load_scale_raw(step, t);
       }
     }
     if (NU > 0) __builtin_amdgcn_sched_barrier(0);  // keep the compiler from moving them behind the weights
 #pragma unroll
-    for (int i = 0; i < kNT; ++i) d.wv[i] = __builtin_nontemporal_load(tp + (step0 / kSPT + i) * 64);
+    for (int t = 0; t < TN; ++t)
+#pragma unroll
+      for (int i = 0; i < kNT; ++i) d.wv[t][i] = __builtin_nontemporal_load(tp[t] + (step0 / kSPT + i) * 64);
   }
 
   // mfma(A, constant B): the term that removes the dequantiser's offset.  It
@@ -157,7 +165,7 @@ struct StreamKernel {
   // One k step: dequantise, one MFMA per M tile, add the rows of row group
   // `slot` to that group's class.
   __device__ inline void step_mfma(const uint32_t* w, const u32x4 (&a)[MT], const f32x4 (&cc)[MT],
-                                   int slot, float sc) {
+                                   int slot, float sc, int t) {
     const u32x4 b = Dequant<DT, BITS>::run(w, magic);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
@@ -166,8 +174,8 @@ struct StreamKernel {
       for (int r = 0; r < 4; ++r) {
         const bool rsel = MP >= 4 ? true : (r / MP == slot % kRowsPerGroup);
         if (rsel) {
-          const float t = totc[mt][slot / kRowsPerGroup][r];
-          totc[mt][slot / kRowsPerGroup][r] = GROUPED ? fmaf(acc[r], sc, t) : t + acc[r];
+          const float v = totc[t][mt][slot / kRowsPerGroup][r];
+          totc[t][mt][slot / kRowsPerGroup][r] = GROUPED ? fmaf(acc[r], sc, v) : v + acc[r];
         }
       }
     }
@@ -180,12 +188,14 @@ struct StreamKernel {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) cc[a][mt] = cancel_term(d.av[a][mt]);
 #pragma unroll
-    for (int s = 0; s < kU; ++s) {
-      const u32x4 t = d.wv[s / kSPT];
-      const uint32_t w[4] = {t.x, t.y, t.z, t.w};
-      const float sc = GROUPED ? to_f32<DT>(d.sraw[scale_slot(s)]) : 1.0f;
-      step_mfma(w + (s % kSPT) * kDw, d.av[s / kS], cc[s / kS], s % kS, sc);
-    }
+    for (int s = 0; s < kU; ++s)
+#pragma unroll
+      for (int t = 0; t < TN; ++t) {
+        const u32x4 v = d.wv[t][s / kSPT];
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        const float sc = GROUPED ? to_f32<DT>(d.sraw[t][scale_slot(s)]) : 1.0f;
+        step_mfma(w + (s % kSPT) * kDw, d.av[s / kS], cc[s / kS], s % kS, sc, t);
+      }
   }
 
   __device__ inline void run(const uint8_t* codes, const uint16_t* bias, void* out, int out_f32,
@@ -194,25 +204,37 @@ struct StreamKernel {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     j = lane & 15;
     kb = lane >> 4;
-    const int tn = blockIdx.x;
-    n = tn * kStripCols + j;
-    const uint8_t* strip = codes + static_cast<int64_t>(tn) * strip_bytes(K, BITS);
+    const int nstrips = N / kStripCols;
+    const uint8_t* strip[TN];
+#pragma unroll
+    for (int t = 0; t < TN; ++t) {
+      int tn = blockIdx.x * TN + t;
+      tn = tn < nstrips ? tn : nstrips - 1;  // a strip past the end repeats the last one and is not stored
+      n[t] = tn * kStripCols + j;
+      strip[t] = codes + static_cast<int64_t>(tn) * strip_bytes(K, BITS);
+    }
     magic = Dequant<DT, BITS>::kMagic;
     asm volatile("" : "+v"(magic));  // keep the constant in a VGPR
     const int nsteps = K / 32;
     const int nunits = nsteps / kU;
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+    for (int t = 0; t < TN; ++t)
 #pragma unroll
-      for (int c = 0; c < kClasses; ++c) totc[mt][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int c = 0; c < kClasses; ++c) totc[t][mt][c] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     // what the epilogue needs from memory, requested before the long loads:
     // thread t always stores column t % 16 of the strip
     // (raw bits; they are converted where they are used, after the long loads)
-    const uint16_t ep_sraw = scale[n];
-    const uint16_t ep_braw = (bias != nullptr ? bias : scale)[n];  // one unconditional load
-
-    const u32x4* tp = reinterpret_cast<const u32x4*>(strip) + lane;
+    uint16_t ep_sraw[TN], ep_braw[TN];
+    const u32x4* tp[TN];
+#pragma unroll
+    for (int t = 0; t < TN; ++t) {
+      ep_sraw[t] = scale[n[t]];
+      ep_braw[t] = (bias != nullptr ? bias : scale)[n[t]];  // one unconditional load
+      tp[t] = reinterpret_cast<const u32x4*>(strip[t]) + lane;
+    }
     if (NU > 0) {
       Unit d[NU > 0 ? NU : 1];
 #pragma unroll
@@ -241,28 +263,31 @@ struct StreamKernel {
         // 64 mod 128) or one whole tile (int8).  Every row group carries the
         // same step, row group 0 is kept.
         for (int step = nunits * kU; step < nsteps; step += 2) {
-          uint32_t w[4];
-          if (BITS == 8) {
-            const u32x4 t = tp[(step / 2) * 64];
-            w[0] = t.x; w[1] = t.y; w[2] = t.z; w[3] = t.w;
-          } else {
-            const int tile = step / 4, nfull = K / 128;
-            const uint8_t* p = tile < nfull ? strip + tile * 1024 + lane * 16 + (step % 4) * 4
-                                            : strip + nfull * 1024 + lane * 8;
-            const u32x2 t = *reinterpret_cast<const u32x2*>(p);
-            w[0] = t.x; w[1] = t.y; w[2] = 0; w[3] = 0;
-          }
-          const float sc = GROUPED ? to_f32<DT>(load_scale_raw(step)) : 1.0f;
+          u32x4 a[2][MT];
+          f32x4 cc[2][MT];
 #pragma unroll
-          for (int st = 0; st < 2; ++st) {
-            u32x4 a[MT];
-            f32x4 cc[MT];
+          for (int st = 0; st < 2; ++st)
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
-              a[mt] = load_a(mt, step + st, false);
-              cc[mt] = cancel_term(a[mt]);
+              a[st][mt] = load_a(mt, step + st, false);
+              cc[st][mt] = cancel_term(a[st][mt]);
             }
-            step_mfma(w + st * kDw, a, cc, 0, sc);
+#pragma unroll
+          for (int t = 0; t < TN; ++t) {
+            uint32_t w[4];
+            if (BITS == 8) {
+              const u32x4 v = tp[t][(step / 2) * 64];
+              w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w;
+            } else {
+              const int tile = step / 4, nfull = K / 128;
+              const uint8_t* p = tile < nfull ? strip[t] + tile * 1024 + lane * 16 + (step % 4) * 4
+                                              : strip[t] + nfull * 1024 + lane * 8;
+              const u32x2 v = *reinterpret_cast<const u32x2*>(p);
+              w[0] = v.x; w[1] = v.y; w[2] = 0; w[3] = 0;
+            }
+            const float sc = GROUPED ? to_f32<DT>(load_scale_raw(step, t)) : 1.0f;
+#pragma unroll
+            for (int st = 0; st < 2; ++st) step_mfma(w + st * kDw, a[st], cc[st], 0, sc, t);
           }
         }
       }
@@ -271,67 +296,77 @@ struct StreamKernel {
     // The epilogue's operands were requested first and have arrived by now;
     // naming them here keeps the compiler from sinking those loads (and the
     // reads of the kernel arguments) into the tail of the kernel.
-    asm volatile("" ::"v"(ep_sraw), "v"(ep_braw), "s"(out), "s"(out_f32));
+#pragma unroll
+    for (int t = 0; t < TN; ++t) asm volatile("" ::"v"(ep_sraw[t]), "v"(ep_braw[t]));
+    asm volatile("" ::"s"(out), "s"(out_f32));
 
-    // Merge the classes: every lane keeps the class of its own lane group.
-    f32x4 tot[MT];
-    {
-      const int mine = MP == 8 ? (kb >> 1) : kb;
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        tot[mt] = totc[mt][0];
+    for (int t = 0; t < TN; ++t) {
+      // Merge the classes: every lane keeps the class of its own lane group.
+      f32x4 tot[MT];
+      {
+        const int mine = MP == 8 ? (kb >> 1) : kb;
 #pragma unroll
-        for (int c = 1; c < kClasses; ++c)
+        for (int mt = 0; mt < MT; ++mt) {
+          tot[mt] = totc[t][mt][0];
 #pragma unroll
-          for (int r = 0; r < 4; ++r) tot[mt][r] = mine == c ? totc[mt][c][r] : tot[mt][r];
+          for (int c = 1; c < kClasses; ++c)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) tot[mt][r] = mine == c ? totc[t][mt][c][r] : tot[mt][r];
+        }
       }
-    }
-    // Fold the kS row groups that carried the same output row: registers
-    // first (MP < 4 keeps several row groups in one lane), then across the
-    // lane groups.  Afterwards rows 0 .. MP-1 hold the wavefront's sums.
-    if (MP == 1) {
-      tot[0][0] = (tot[0][0] + tot[0][1]) + (tot[0][2] + tot[0][3]);
-    } else if (MP == 2) {
-      tot[0][0] += tot[0][2];
-      tot[0][1] += tot[0][3];
-    }
-    if (MP <= 8) {
+      // Fold the kS row groups that carried the same output row: registers
+      // first (MP < 4 keeps several row groups in one lane), then across the
+      // lane groups.  Afterwards rows 0 .. MP-1 hold the wavefront's sums.
+      if (MP == 1) {
+        tot[0][0] = (tot[0][0] + tot[0][1]) + (tot[0][2] + tot[0][3]);
+      } else if (MP == 2) {
+        tot[0][0] += tot[0][2];
+        tot[0][1] += tot[0][3];
+      }
+      if (MP <= 8) {
 #pragma unroll
-      for (int r = 0; r < kLive; ++r) tot[0][r] = sum_lane_groups(tot[0][r], MP <= 4, true);
+        for (int r = 0; r < kLive; ++r) tot[0][r] = sum_lane_groups(tot[0][r], MP <= 4, true);
+      }
+      // Meet in LDS: red[strip][wave][mt][r][lane], summed over wavefronts in order.
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < kLive; ++r)
+          red[(((t * WK + wave) * MT + mt) * 4 + r) * 64 + lane] = tot[mt][r];
     }
-    // Meet in LDS: red[wave][mt][r][lane], summed over wavefronts in order.
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-      for (int r = 0; r < kLive; ++r) red[((wave * MT + mt) * 4 + r) * 64 + lane] = tot[mt][r];
     __syncthreads();
     const int rows = M < 16 * MT ? M : 16 * MT;
-    for (int idx = threadIdx.x; idx < rows * 16; idx += WK * 64) {
-      const int m = idx / 16, nl = idx % 16;
-      const int mt = m / 16, row = m % 16;
-      float s = 0.0f;
 #pragma unroll
-      for (int w = 0; w < WK; ++w)
-        s += red[((w * MT + mt) * 4 + (row % 4)) * 64 + (row / 4) * 16 + nl];
-      const int nn = tn * kStripCols + nl;  // nl == j: the stride of idx is a multiple of 16
-      const float ep_scale = GROUPED ? 1.0f : to_f32<DT>(ep_sraw);
-      const float ep_bias = bias != nullptr ? to_f32<DT>(ep_braw) : 0.0f;
-      s = s * ep_scale + ep_bias;
-      if (out_f32)
-        static_cast<float*>(out)[static_cast<int64_t>(m) * N + nn] = s;
-      else
-        static_cast<uint16_t*>(out)[static_cast<int64_t>(m) * N + nn] = cast_out<DT>(s);
+    for (int t = 0; t < TN; ++t) {
+      if (static_cast<int>(blockIdx.x) * TN + t >= nstrips) break;  // the repeated last strip
+      const float ep_scale = GROUPED ? 1.0f : to_f32<DT>(ep_sraw[t]);
+      const float ep_bias = bias != nullptr ? to_f32<DT>(ep_braw[t]) : 0.0f;
+      for (int idx = threadIdx.x; idx < rows * 16; idx += WK * 64) {
+        const int m = idx / 16, nl = idx % 16;  // nl == j: the stride of idx is a multiple of 16
+        const int mt = m / 16, row = m % 16;
+        float s = 0.0f;
+#pragma unroll
+        for (int w = 0; w < WK; ++w)
+          s += red[(((t * WK + w) * MT + mt) * 4 + (row % 4)) * 64 + (row / 4) * 16 + nl];
+        s = s * ep_scale + ep_bias;
+        const int64_t o = static_cast<int64_t>(m) * N + n[t];
+        if (out_f32)
+          static_cast<float*>(out)[o] = s;
+        else
+          static_cast<uint16_t*>(out)[o] = cast_out<DT>(s);
+      }
     }
   }
 };
 
-template <int DT, int BITS, int MP, int MT, int WK, int NU, bool GROUPED>
+template <int DT, int BITS, int MP, int MT, int WK, int NU, int TN, bool GROUPED>
 __global__ __launch_bounds__(WK * 64) void stream_kernel(
     const uint16_t* __restrict__ x, const uint8_t* __restrict__ codes,
     const uint16_t* __restrict__ bias, const uint16_t* __restrict__ scale, void* __restrict__ out,
     int M, int K, int N, int gshift, int out_f32) {
   extern __shared__ float red[];
-  StreamKernel<DT, BITS, MP, MT, WK, NU, GROUPED> k;
+  StreamKernel<DT, BITS, MP, MT, WK, NU, TN, GROUPED> k;
   k.x = x;
   k.scale = scale;
   k.M = M;
@@ -343,23 +378,36 @@ __global__ __launch_bounds__(WK * 64) void stream_kernel(
 
 struct Args {
   const void* x; const void* codes; const void* bias; const void* scale; void* out;
-  int M, K, N, gshift, out_f32; hipStream_t stream;
+  int M, K, N, gshift, out_f32, tn; hipStream_t stream;
 };
 
-template <int DT, int BITS, int MP, int MT, int WK, int NU>
-void launch_one(const Args& a) {
-  const size_t lds = static_cast<size_t>(WK) * MT * 256 * sizeof(float);
-  const dim3 grid(static_cast<unsigned>(a.N / kStripCols)), block(WK * 64);
+template <int DT, int BITS, int MP, int MT, int WK, int NU, int TN>
+void launch_tn(const Args& a) {
+  const size_t lds = static_cast<size_t>(TN) * WK * MT * 256 * sizeof(float);
+  const dim3 grid(static_cast<unsigned>((a.N / kStripCols + TN - 1) / TN)), block(WK * 64);
   const uint16_t* x = static_cast<const uint16_t*>(a.x);
   const uint8_t* codes = static_cast<const uint8_t*>(a.codes);
   const uint16_t* bias = static_cast<const uint16_t*>(a.bias);
   const uint16_t* scale = static_cast<const uint16_t*>(a.scale);
   if (a.gshift >= 0)
-    stream_kernel<DT, BITS, MP, MT, WK, NU, true><<<grid, block, lds, a.stream>>>(
+    stream_kernel<DT, BITS, MP, MT, WK, NU, TN, true><<<grid, block, lds, a.stream>>>(
         x, codes, bias, scale, a.out, a.M, a.K, a.N, a.gshift, a.out_f32);
   else
-    stream_kernel<DT, BITS, MP, MT, WK, NU, false><<<grid, block, lds, a.stream>>>(
+    stream_kernel<DT, BITS, MP, MT, WK, NU, TN, false><<<grid, block, lds, a.stream>>>(
         x, codes, bias, scale, a.out, a.M, a.K, a.N, a.gshift, a.out_f32);
+}
+
+// Two strips per workgroup exist for the operand shapes whose activation
+// traffic matters (eight rows and up).
+template <int DT, int BITS, int MP, int MT, int WK, int NU>
+void launch_one(const Args& a) {
+  if constexpr (MP >= 8) {
+    if (a.tn == 2) {
+      launch_tn<DT, BITS, MP, MT, WK, NU, 2>(a);
+      return;
+    }
+  }
+  launch_tn<DT, BITS, MP, MT, WK, NU, 1>(a);
 }
 
 // wk in {1,2,4,8,16}; nu == 1 selects the all-loads-at-once variant (exactly
@@ -402,10 +450,11 @@ void launch_m(const Args& a, int wk, int nu) {
 // of two up to 16, each wavefront takes exactly one unit and loads it at once.
 // Otherwise wavefronts walk several units with two in flight, and WK aims at
 // about four wavefronts per SIMD.
-static void pick_split(int64_t M, int64_t K, int64_t N, int bits, int* wk, int* nu) {
-  const int64_t strips = N / kStripCols;
+static void pick_split(int64_t M, int64_t K, int64_t N, int bits, int* wk, int* nu, int* tn) {
   int mp = 1;
   while (mp < 16 && mp < M) mp *= 2;
+  *tn = stream_strips_per_workgroup(M, N, bits);
+  const int64_t strips = (N / kStripCols + *tn - 1) / *tn;  // workgroups
   const int s = 16 / mp, spt = bits == 8 ? 2 : 4;
   const int ku = s > spt ? s : spt;
   const int64_t nsteps = K / 32, nunits = nsteps / ku;
@@ -426,10 +475,10 @@ int launch_linear_stream(const void* x, const void* codes, const void* bias, con
                          int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
                          void* out, bool out_f32, hipStream_t stream) {
   const int gshift = group_size == 64 ? 6 : (group_size == 128 ? 7 : -1);
+  int wk = 1, nu = 0, tn = 1;
+  pick_split(M, K, N, bits, &wk, &nu, &tn);
   const Args a{x, codes, bias, scale, out, static_cast<int>(M), static_cast<int>(K),
-               static_cast<int>(N), gshift, out_f32 ? 1 : 0, stream};
-  int wk = 1, nu = 0;
-  pick_split(M, K, N, bits, &wk, &nu);
+               static_cast<int>(N), gshift, out_f32 ? 1 : 0, tn, stream};
   if (dtype == WOL_DTYPE_BF16) {
     if (bits == 8) launch_m<WOL_DTYPE_BF16, 8>(a, wk, nu); else launch_m<WOL_DTYPE_BF16, 4>(a, wk, nu);
   } else {
