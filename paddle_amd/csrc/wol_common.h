@@ -112,11 +112,11 @@ __device__ inline float to_f32(uint16_t h) {
 // paddle/phi/common/bfloat16.h:61-88: zero keeps only its sign, infinity
 // passes, NaN becomes 0x7FFF.
 __device__ inline uint16_t f32_to_bf16_rne(float f) {
+  // branch-free: the rounding add leaves zero and infinity as they are (their
+  // low half is zero), so only NaN needs a select
   const uint32_t u = __float_as_uint(f);
-  const uint32_t mag = u & 0x7FFFFFFFu;
-  if (mag > 0x7F800000u) return 0x7FFFu;
-  if (mag == 0x7F800000u || mag == 0) return static_cast<uint16_t>(u >> 16);
-  return static_cast<uint16_t>((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+  const uint32_t r = (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+  return static_cast<uint16_t>((u & 0x7FFFFFFFu) > 0x7F800000u ? 0x7FFFu : r);
 }
 
 // Round-to-nearest-even float -> fp16 (v_cvt_f16_f32 under the default
@@ -125,9 +125,9 @@ __device__ inline uint16_t f32_to_bf16_rne(float f) {
 __device__ inline uint16_t f32_to_f16_rne(float f) {
   const uint32_t u = __float_as_uint(f);
   const uint32_t mag = u & 0x7FFFFFFFu;
-  if (mag > 0x7F800000u)
-    return static_cast<uint16_t>(((u >> 16) & 0x8000u) | 0x7E00u | ((mag >> 13) & 0x3FFu));
-  return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
+  const uint16_t nan = static_cast<uint16_t>(((u >> 16) & 0x8000u) | 0x7E00u | ((mag >> 13) & 0x3FFu));
+  const uint16_t num = __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
+  return mag > 0x7F800000u ? nan : num;  // a select, not a branch
 }
 
 // The truncating flavours (WOL_ROUND_TRUNC): bf16 drops the low half

@@ -121,6 +121,82 @@ __device__ inline void load_block(Stage& st, int layout, int bits, int64_t K, in
   }
 }
 
+// Full blocks (128 k x 64 n) in the GFX950 layout move as whole 16-byte lane
+// pieces: a piece is the 16 (int8) or 32 (int4) codes one lane of the
+// consuming wavefront loads at once -- one column, rows as gfx950_offset()
+// lays them out.  512 (int8) or 256 (int4) pieces per block.
+template <int BITS>
+__device__ inline void store_block_gfx950(const Stage& st, int64_t K, int64_t k0, int64_t n0,
+                                          uint8_t* codes) {
+  constexpr int kPieces = BITS == 8 ? 512 : 256;
+  for (int q = threadIdx.x; q < kPieces; q += kThreads) {
+    const int lane = q % 64, c = (BITS == 8 ? q / 128 : q / 64) * 16 + lane % 16;
+    const int rb = (lane / 16) * 8;
+    uint32_t d[4];
+    int64_t off;
+    if (BITS == 8) {
+      const int t = (q / 64) % 2;
+#pragma unroll
+      for (int h = 0; h < 4; ++h) {  // dword h: k step h / 2, bytes 4 * (h % 2) ..
+        uint32_t v = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int r = t * 64 + (h / 2) * 32 + rb + 4 * (h % 2) + e;
+          v |= static_cast<uint32_t>((st.v[r][c] + 128) & 0xFF) << (8 * e);
+        }
+        d[h] = v;
+      }
+      off = (n0 / kStripCols + q / 128) * strip_bytes(K, 8) + (k0 / 64 + t) * 1024 + lane * 16;
+    } else {
+#pragma unroll
+      for (int step = 0; step < 4; ++step) {
+        uint32_t v = 0;
+#pragma unroll
+        for (int pn = 0; pn < 8; ++pn) {
+          const int i = pn < 4 ? 2 * pn : 2 * (pn - 4) + 1;
+          v |= static_cast<uint32_t>((st.v[step * 32 + rb + i][c] + 8) & 0xF) << (4 * pn);
+        }
+        d[step] = v;
+      }
+      off = (n0 / kStripCols + q / 64) * strip_bytes(K, 4) + (k0 / 128) * 1024 + lane * 16;
+    }
+    *reinterpret_cast<uint4*>(codes + off) = make_uint4(d[0], d[1], d[2], d[3]);
+  }
+}
+
+template <int BITS>
+__device__ inline void load_block_gfx950(Stage& st, int64_t K, int64_t k0, int64_t n0,
+                                         const uint8_t* codes) {
+  constexpr int kPieces = BITS == 8 ? 512 : 256;
+  for (int q = threadIdx.x; q < kPieces; q += kThreads) {
+    const int lane = q % 64, c = (BITS == 8 ? q / 128 : q / 64) * 16 + lane % 16;
+    const int rb = (lane / 16) * 8;
+    if (BITS == 8) {
+      const int t = (q / 64) % 2;
+      const int64_t off = (n0 / kStripCols + q / 128) * strip_bytes(K, 8) + (k0 / 64 + t) * 1024 + lane * 16;
+      const uint4 v = *reinterpret_cast<const uint4*>(codes + off);
+      const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int h = 0; h < 4; ++h)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          st.v[t * 64 + (h / 2) * 32 + rb + 4 * (h % 2) + e][c] =
+              static_cast<int8_t>(static_cast<int>((d[h] >> (8 * e)) & 0xFF) - 128);
+    } else {
+      const int64_t off = (n0 / kStripCols + q / 64) * strip_bytes(K, 4) + (k0 / 128) * 1024 + lane * 16;
+      const uint4 v = *reinterpret_cast<const uint4*>(codes + off);
+      const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int step = 0; step < 4; ++step)
+#pragma unroll
+        for (int pn = 0; pn < 8; ++pn) {
+          const int i = pn < 4 ? 2 * pn : 2 * (pn - 4) + 1;
+          st.v[step * 32 + rb + i][c] = static_cast<int8_t>(static_cast<int>((d[step] >> (4 * pn)) & 0xF) - 8);
+        }
+    }
+  }
+}
+
 union Pack8 {
   uint4 q;
   uint16_t h[8];
@@ -271,7 +347,10 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(
     }
   }
   __syncthreads();
-  store_block(st, layout, BITS, K, N, k0, n0, KR, NC, codes);
+  if (layout == WOL_LAYOUT_GFX950 && KR == kBlockK && NC == kBlockN)
+    store_block_gfx950<BITS>(st, K, k0, n0, codes);
+  else
+    store_block(st, layout, BITS, K, N, k0, n0, KR, NC, codes);
 }
 
 // out[k,n] = cast_T(float(code) * float(scale)), written as [K,N] rows.
@@ -285,7 +364,10 @@ __global__ __launch_bounds__(kThreads) void dequantize_kernel(
   const int64_t k0 = static_cast<int64_t>(blockIdx.y) * kBlockK;
   const int KR = static_cast<int>(K - k0 < kBlockK ? K - k0 : kBlockK);
   const int NC = static_cast<int>(N - n0 < kBlockN ? N - n0 : kBlockN);
-  load_block(st, layout, BITS, K, N, k0, n0, KR, NC, codes);
+  if (layout == WOL_LAYOUT_GFX950 && KR == kBlockK && NC == kBlockN)
+    load_block_gfx950<BITS>(st, K, k0, n0, codes);
+  else
+    load_block(st, layout, BITS, K, N, k0, n0, KR, NC, codes);
   __syncthreads();
   if (tx * 8 >= NC) return;
 #pragma unroll
@@ -312,9 +394,16 @@ __global__ __launch_bounds__(kThreads) void repack_kernel(const uint8_t* __restr
   const int64_t k0 = static_cast<int64_t>(blockIdx.y) * kBlockK;
   const int KR = static_cast<int>(K - k0 < kBlockK ? K - k0 : kBlockK);
   const int NC = static_cast<int>(N - n0 < kBlockN ? N - n0 : kBlockN);
-  load_block(st, layout_in, BITS, K, N, k0, n0, KR, NC, in);
+  const bool full = KR == kBlockK && NC == kBlockN;
+  if (layout_in == WOL_LAYOUT_GFX950 && full)
+    load_block_gfx950<BITS>(st, K, k0, n0, in);
+  else
+    load_block(st, layout_in, BITS, K, N, k0, n0, KR, NC, in);
   __syncthreads();
-  store_block(st, layout_out, BITS, K, N, k0, n0, KR, NC, out);
+  if (layout_out == WOL_LAYOUT_GFX950 && full)
+    store_block_gfx950<BITS>(st, K, k0, n0, out);
+  else
+    store_block(st, layout_out, BITS, K, N, k0, n0, KR, NC, out);
 }
 
 inline dim3 block_grid(int64_t K, int64_t N) {
