@@ -240,7 +240,7 @@ def main():
             "unit": "GB/s",
             "frac": round(dec_gbs / HBM_PEAK_GBS, 4),
             "traffic": traffic.get("decode_bytes_per_launch"),
-            "kernel": "wol::stream_kernel<1, 4, 1, 1, 8, 1, true>",
+            "kernel": "wol::stream_kernel<1, 4, 1, 1, 8, 1, 1, true>",
             "algorithmic_bytes_per_launch": wbytes,
             "total_bytes_per_launch": total_bytes,
         },
@@ -256,7 +256,7 @@ def main():
                 "unit": "TFLOP/s",
                 "frac": round(pre_tf / MFMA_BF16_PEAK_TF, 4),
                 "traffic": traffic.get("prefill_bytes_per_launch"),
-                "kernel": "wol::gemm_dma_kernel<1, 8, 2, 4, 4, 2>",
+                "kernel": "wol::gemm_dma_kernel<1, 8, 0, false, 2, 4, 4, 2> (256 of 384 tiles) + <1, 8, 0, false, 2, 4, 2, 2> (the rest as 128-row tiles)",
             },
         },
         "cpu_baseline": cpu,
