@@ -109,6 +109,20 @@ int wol_quantize(const void* w, int dtype, int64_t K, int64_t N, int bits,
                  void* stream);
 
 /*
+ * weight_quantize with algo = "llm.int8" (cpu/weight_quantize_kernel.cc:163-166,
+ * quant_compute<..., int8_t, 8, float>): int8 codes computed against the
+ * unrounded fp32 scale amax/127, which is also what is returned.
+ * scale_out: [N] or [ceil(K/g), N] float.  The reference returns the codes as
+ * [N,K] (a plain byte transpose, :108-111): that is WOL_LAYOUT_PADDLE_HIP.
+ * These tensors feed llm_int8_linear, not wol_linear (whose scales are T).
+ * Workspace as for wol_quantize with bits = 8.
+ */
+int wol_quantize_llm_int8(const void* w, int dtype, int64_t K, int64_t N,
+                          int group_size, int layout, void* codes_out,
+                          float* scale_out, void* workspace,
+                          size_t workspace_bytes, void* stream);
+
+/*
  * weight_dequantize.  out_KN[k,n] = cast_T( float(code[k,n]) * float(scale) ),
  * written directly as [K,N] row-major T (the reference writes [N,K] and then
  * transposes, gpu/weight_dequantize_kernel.cu:464-470).  `layout` names the

@@ -266,6 +266,45 @@ int wo_weight_quantize(const uint16_t* w, int64_t K, int64_t N, int dtype,
   return 0;
 }
 
+/* algo == "llm.int8" (paddle/phi/kernels/cpu/weight_quantize_kernel.cc:163-166:
+ * quant_compute<..., int8_t, 8, float>): the same loops with ScaleT = float,
+ * so the scale max/127 is not rounded to T and the codes divide by that fp32
+ * value (impl/weight_quantize_kernel_impl.h:45-57, :80-96 and the group-wise
+ * forms :59-78, :131-149).  codes [K,N] int8, scale [N] or [ceil(K/g),N] float.
+ * Pinned like the T-scale flavour (closed form, invariants, numpy
+ * restatement); the reference holds no vectors for it. */
+int wo_weight_quantize_llm_int8(const uint16_t* w, int64_t K, int64_t N,
+                                int dtype, int64_t group_size, int8_t* codes,
+                                float* scale) {
+  if (K % 64 != 0 || N % 16 != 0) return -1;
+  if (!(group_size == -1 || group_size == 64 || group_size == 128)) return -1;
+  for (int64_t n = 0; n < N; ++n) {
+    if (group_size == -1) {
+      float mx = wo_to_f32(w[n], dtype);
+      for (int64_t k = 0; k < K; ++k) {
+        float a = abs_like_ref(wo_to_f32(w[k * N + n], dtype));
+        mx = a > mx ? a : mx;
+      }
+      scale[n] = mx / 127.0f;
+    } else {
+      for (int64_t k0 = 0; k0 < K; k0 += group_size) {
+        float mx = 0.0f;
+        for (int64_t k = k0; k < k0 + group_size && k < K; ++k) {
+          float a = abs_like_ref(wo_to_f32(w[k * N + n], dtype));
+          mx = a > mx ? a : mx;
+        }
+        scale[(k0 / group_size) * N + n] = mx / 127.0f;
+      }
+    }
+  }
+  for (int64_t k = 0; k < K; ++k) {
+    const float* srow = group_size > 0 ? scale + (k / group_size) * N : scale;
+    for (int64_t n = 0; n < N; ++n)
+      codes[k * N + n] = quant_code_int8(wo_to_f32(w[k * N + n], dtype), srow[n]);
+  }
+  return 0;
+}
+
 /* The HIP-flavour layout step of quant_compute
  * (cpu/weight_quantize_kernel.cc:113-125): a byte transpose of the canonical
  * tensor, [K,N] -> [N,K] for int8 and [K,N/2] -> [N/2,K] for int4. */

@@ -52,6 +52,8 @@ def lib():
         L.wo_quant_codes.argtypes = [_u16p, _u16p, _i64, _i64, _int, _int, _i64, _int, _i8p]
         L.wo_weight_quantize.argtypes = [_u16p, _i64, _i64, _int, _int, _i64, _int, _int, _i8p, _u16p]
         L.wo_weight_quantize.restype = _int
+        L.wo_weight_quantize_llm_int8.argtypes = [_u16p, _i64, _i64, _int, _i64, _i8p, _f32p]
+        L.wo_weight_quantize_llm_int8.restype = _int
         L.wo_transpose_bytes.argtypes = [_i8p, _i64, _i64, _i8p]
         L.wo_dequantize.argtypes = [_i8p, _u16p, _i64, _i64, _int, _int, _i64, _int, _int,
                                     ctypes.c_void_p, ctypes.c_void_p]
@@ -88,6 +90,18 @@ def weight_quantize(w_bits, dtype, bits, group_size=-1, cast_mode=CAST_RNE, nibb
     rc = lib().wo_weight_quantize(w_bits, K, N, dtype, bits, group_size, cast_mode, nibble_bias,
                                   codes, scale)
     if rc != 0:
+        raise ValueError("oracle: shape/group_size outside the weight_quantize contract")
+    return codes, scale
+
+
+def weight_quantize_llm_int8(w_bits, dtype, group_size=-1):
+    """algo="llm.int8": canonical int8 codes [K,N] and fp32 scales [N] or [ceil(K/g),N]."""
+    w_bits = np.ascontiguousarray(w_bits, dtype=np.uint16)
+    K, N = w_bits.shape
+    codes = np.empty((K, N), np.int8)
+    shape = (N,) if group_size == -1 else ((K + group_size - 1) // group_size, N)
+    scale = np.empty(shape, np.float32)
+    if lib().wo_weight_quantize_llm_int8(w_bits, K, N, dtype, group_size, codes, scale) != 0:
         raise ValueError("oracle: shape/group_size outside the weight_quantize contract")
     return codes, scale
 

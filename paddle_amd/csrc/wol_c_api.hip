@@ -120,7 +120,21 @@ int wol_quantize(const void* w, int dtype, int64_t K, int64_t N, int bits, int g
   const size_t need = wol_quantize_workspace(K, N, bits, group_size);
   if (need > 0 && (workspace == nullptr || workspace_bytes < need)) return WOL_ERR_WORKSPACE;
   return wol::launch_quantize(w, dtype, K, N, bits, group_size, round_mode, layout, codes_out,
-                              scale_out, workspace, static_cast<hipStream_t>(stream));
+                              scale_out, false, workspace, static_cast<hipStream_t>(stream));
+}
+
+int wol_quantize_llm_int8(const void* w, int dtype, int64_t K, int64_t N, int group_size,
+                          int layout, void* codes_out, float* scale_out, void* workspace,
+                          size_t workspace_bytes, void* stream) {
+  const int rc = check_problem(dtype, K, N, 8, group_size);
+  if (rc != WOL_OK) return rc;
+  if (!layout_ok(layout)) return WOL_ERR_BAD_LAYOUT;
+  if (w == nullptr || codes_out == nullptr || scale_out == nullptr) return WOL_ERR_NULL_POINTER;
+  if (!aligned16(w) || !aligned16(codes_out)) return WOL_ERR_ALIGNMENT;
+  const size_t need = wol_quantize_workspace(K, N, 8, group_size);
+  if (need > 0 && (workspace == nullptr || workspace_bytes < need)) return WOL_ERR_WORKSPACE;
+  return wol::launch_quantize(w, dtype, K, N, 8, group_size, WOL_ROUND_RNE, layout, codes_out,
+                              scale_out, true, workspace, static_cast<hipStream_t>(stream));
 }
 
 int wol_dequantize(const void* codes, int layout, const void* scale, int dtype, int64_t K,

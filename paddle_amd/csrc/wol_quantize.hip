@@ -265,7 +265,11 @@ template <int DT, int BITS>
 __global__ __launch_bounds__(kThreads) void quantize_kernel(
     const uint16_t* __restrict__ w, int64_t K, int64_t N, int group_size, int round_mode,
     int layout, const uint32_t* __restrict__ amax, uint8_t* __restrict__ codes,
-    uint16_t* __restrict__ scale) {
+    void* __restrict__ scale_out, int scale_f32) {
+  // scale_f32: the "llm.int8" flavour -- the scale stays the fp32 quotient
+  // (paddle/phi/kernels/cpu/weight_quantize_kernel.cc:163-166, ScaleT = float)
+  uint16_t* scale = static_cast<uint16_t*>(scale_out);
+  float* scale32 = static_cast<float*>(scale_out);
   __shared__ Stage st;
   __shared__ float part[2][32][kBlockN];
   __shared__ float sc[2][kBlockN];
@@ -316,9 +320,15 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(
       if (g < ngroups && c < NC && g * 64 < KR) {
         float m = 0.0f;
         for (int r = 0; r < 32; ++r) m = part[g][r][c] > m ? part[g][r][c] : m;
-        const uint16_t sb = from_f32<DT>(m / bound, round_mode);
-        scale[(k0 / group_size + g) * N + n0 + c] = sb;
-        sc[g][c] = to_f32<DT>(sb);
+        const int64_t si = (k0 / group_size + g) * N + n0 + c;
+        if (scale_f32) {
+          scale32[si] = m / bound;
+          sc[g][c] = m / bound;
+        } else {
+          const uint16_t sb = from_f32<DT>(m / bound, round_mode);
+          scale[si] = sb;
+          sc[g][c] = to_f32<DT>(sb);
+        }
       }
     }
   } else {
@@ -329,9 +339,14 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(
       const float v0 = to_f32<DT>(w[n0 + c]);
       const float m = __uint_as_float(amax[n0 + c]);
       const float src = (v0 != v0) ? v0 : (m == 0.0f ? (v0 < 0.0f ? m : v0) : m);
-      const uint16_t sb = from_f32<DT>(src / bound, round_mode);
-      if (k0 == 0) scale[n0 + c] = sb;
-      sc[0][c] = to_f32<DT>(sb);
+      if (scale_f32) {
+        if (k0 == 0) scale32[n0 + c] = src / bound;
+        sc[0][c] = src / bound;
+      } else {
+        const uint16_t sb = from_f32<DT>(src / bound, round_mode);
+        if (k0 == 0) scale[n0 + c] = sb;
+        sc[0][c] = to_f32<DT>(sb);
+      }
     }
   }
   __syncthreads();
@@ -414,8 +429,8 @@ inline dim3 block_grid(int64_t K, int64_t N) {
 }  // namespace
 
 int launch_quantize(const void* w, int dtype, int64_t K, int64_t N, int bits, int group_size,
-                    int round_mode, int layout, void* codes, void* scale, void* workspace,
-                    hipStream_t stream) {
+                    int round_mode, int layout, void* codes, void* scale, bool scale_f32,
+                    void* workspace, hipStream_t stream) {
   const uint16_t* wp = static_cast<const uint16_t*>(w);
   uint32_t* amax = static_cast<uint32_t*>(workspace);
   if (group_size == -1) {
@@ -429,10 +444,10 @@ int launch_quantize(const void* w, int dtype, int64_t K, int64_t N, int bits, in
   }
   const dim3 grid = block_grid(K, N);
   uint8_t* cp = static_cast<uint8_t*>(codes);
-  uint16_t* sp = static_cast<uint16_t*>(scale);
+  const int sf = scale_f32 ? 1 : 0;
 #define WOL_Q(DT, B)                                                                   \
   quantize_kernel<DT, B><<<grid, dim3(kThreads), 0, stream>>>(wp, K, N, group_size,   \
-                                                              round_mode, layout, amax, cp, sp)
+                                                              round_mode, layout, amax, cp, scale, sf)
   if (dtype == WOL_DTYPE_BF16) {
     if (bits == 8) WOL_Q(WOL_DTYPE_BF16, 8); else WOL_Q(WOL_DTYPE_BF16, 4);
   } else {

@@ -56,10 +56,7 @@ def _algo_bits(algo):
     if algo == "weight_only_int4":
         return 4
     if algo == "llm.int8":
-        raise NotImplementedError(
-            "algo 'llm.int8' (fp32 scales for llm_int8_linear) is outside the weight-only path "
-            "this library replaces"
-        )
+        return 8
     raise ValueError(
         "(InvalidArgument) The algo must be in ['weight_only_int8', 'weight_only_int4', "
         "'llm.int8'], but got[%s]" % algo
@@ -204,6 +201,10 @@ def weight_quantize(x, algo="weight_only_int8", arch=None, group_size=-1):
     layout; scale is [N] or [ceil(K/group_size), N] in x's dtype.  Codes and
     scales equal the reference's CPU kernel bit for bit (before its own layout
     step).  arch is accepted and ignored, as in a ROCm build of the reference.
+
+    algo="llm.int8" (the input of llm_int8_linear, not of weight_only_linear)
+    keeps the scale in float32 and returns the codes as the reference does for
+    that algo: plain int8 [N, K], the transpose of the code matrix.
     """
     if arch is None:
         arch = _get_arch_info()
@@ -217,9 +218,19 @@ def weight_quantize(x, algo="weight_only_int8", arch=None, group_size=-1):
     x = x.contiguous()
     K, N = x.shape
     out = torch.empty(out_shape, dtype=torch.int8, device=x.device)
-    scale = torch.empty(scale_shape, dtype=x.dtype, device=x.device)
     ws_bytes = _lib.lib.wol_quantize_workspace(K, N, bits, group_size)
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=x.device)
+    if algo == "llm.int8":
+        scale = torch.empty(scale_shape, dtype=torch.float32, device=x.device)
+        with torch.cuda.device(x.device):
+            _lib.check(
+                _lib.lib.wol_quantize_llm_int8(
+                    x.data_ptr(), dt, K, N, group_size, _lib.LAYOUT_PADDLE_HIP, out.data_ptr(),
+                    scale.data_ptr(), ws.data_ptr(), ws_bytes, _stream_ptr(x),
+                )
+            )
+        return out, scale
+    scale = torch.empty(scale_shape, dtype=x.dtype, device=x.device)
     with torch.cuda.device(x.device):
         _lib.check(
             _lib.lib.wol_quantize(

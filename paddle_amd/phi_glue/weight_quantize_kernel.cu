@@ -2,8 +2,8 @@
 // gfx950.  Same template signature (paddle/phi/kernels/weight_quantize_kernel.h:
 // 21-28) and registration (gpu/weight_quantize_kernel.cu:118-123).  Unlike the
 // file it replaces, it produces the CPU kernel's codes and scales bit for bit,
-// supports group_size 64/128 and int4 on the device, and launches on
-// dev_ctx.stream() rather than the null stream.
+// supports group_size 64/128, int4 and the 'llm.int8' flavour on the device,
+// and launches on dev_ctx.stream() rather than the null stream.
 #include "paddle/phi/kernels/weight_quantize_kernel.h"
 
 #include "paddle/phi/core/kernel_registry.h"
@@ -19,17 +19,17 @@ void WeightQuantizeKernel(const Context& dev_ctx,
                           const int32_t group_size,
                           DenseTensor* out,
                           DenseTensor* scale) {
-  PADDLE_ENFORCE_EQ(algo == "weight_only_int8" || algo == "weight_only_int4",
+  PADDLE_ENFORCE_EQ(algo == "weight_only_int8" || algo == "weight_only_int4" || algo == "llm.int8",
                     true,
                     common::errors::Unimplemented(
-                        "gfx950 weight_quantize covers 'weight_only_int8' and 'weight_only_int4'; "
-                        "'llm.int8' keeps its own kernel. Got[%s]",
+                        "The algo must be in ['weight_only_int8', 'weight_only_int4', "
+                        "'llm.int8'], but got[%s]",
                         algo));
-  const int bits = wol_glue::Bits(algo, "weight_quantize");
+  const bool llm = algo == "llm.int8";
+  const int bits = llm ? 8 : wol_glue::Bits(algo, "weight_quantize");
   const auto dims = x.dims();
   const int64_t K = dims[0], N = dims[1];
   dev_ctx.template Alloc<int8_t>(out);   // [N, K] or [N/2, K], set by WeightQuantizeInferMeta
-  dev_ctx.template Alloc<T>(scale);      // [N] or [ceil(K/group_size), N]
   DenseTensor workspace;
   const size_t ws_bytes = wol_quantize_workspace(K, N, bits, group_size);
   void* ws = nullptr;
@@ -37,6 +37,25 @@ void WeightQuantizeKernel(const Context& dev_ctx,
     workspace.Resize({static_cast<int64_t>(ws_bytes)});
     ws = dev_ctx.template Alloc<uint8_t>(&workspace);
   }
+  if (llm) {
+    // fp32 scales and the plain [N, K] transpose, as the reference returns them
+    // for this algo (cpu/weight_quantize_kernel.cc:108-111, :163-166)
+    dev_ctx.template Alloc<float>(scale);
+    wol_glue::Check(wol_quantize_llm_int8(x.data<T>(),
+                                          wol_glue::DTypeTag<T>::value,
+                                          K,
+                                          N,
+                                          group_size,
+                                          WOL_LAYOUT_PADDLE_HIP,
+                                          out->data<int8_t>(),
+                                          scale->data<float>(),
+                                          ws,
+                                          ws_bytes,
+                                          dev_ctx.stream()),
+                    "weight_quantize");
+    return;
+  }
+  dev_ctx.template Alloc<T>(scale);      // [N] or [ceil(K/group_size), N]
   wol_glue::Check(wol_quantize(x.data<T>(),
                                wol_glue::DTypeTag<T>::value,
                                K,

@@ -41,6 +41,20 @@ def repack(codes_u8, layout_in, layout_out, K, N, bits):
     return o.cpu().numpy()
 
 
+def quantize_llm_int8(w_bits, dt, g, layout=1):
+    """algo="llm.int8" through the C ABI: (codes uint8 in `layout`, fp32 scale)."""
+    w = H.bits_to_torch(w_bits, dt, DEV)
+    K, N = w.shape
+    codes = torch.zeros(K * N, dtype=torch.uint8, device=DEV)
+    scale = torch.zeros((N,) if g == -1 else ((K + g - 1) // g, N), dtype=torch.float32, device=DEV)
+    wsb = _lib.lib.wol_quantize_workspace(K, N, 8, g)
+    ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device=DEV)
+    _lib.check(_lib.lib.wol_quantize_llm_int8(w.data_ptr(), dt, K, N, g, layout, codes.data_ptr(), scale.data_ptr(),
+                                              ws.data_ptr(), wsb, None))
+    torch.cuda.synchronize()
+    return codes.cpu().numpy(), scale.cpu().numpy()
+
+
 def linear(x_bits, codes_u8, bias_bits, scale_bits, dt, N, bits, g, f32=False, no_workspace=False,
            kernel=None, ws_bytes=None):
     """codes_u8 in gfx950 layout.  Returns fp32 numpy [M,N] (f32=True) or T bits.

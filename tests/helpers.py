@@ -137,6 +137,30 @@ def np_quantize(w_bits, dt, bits, group_size):
     return q, scale_bits
 
 
+def np_quantize_llm_int8(w_bits, dt, group_size):
+    """Independent statement of algo="llm.int8": np_quantize for int8 with the
+    scale left as the fp32 quotient.  Returns (codes int32 [K,N], scale fp32)."""
+    w = bits_to_f32(w_bits, dt)
+    K, N = w.shape
+    g = K if group_size == -1 else group_size
+    ng = (K + g - 1) // g
+    scale = np.empty((ng, N), np.float32)
+    q = np.empty((K, N), np.int32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        for gi in range(ng):
+            blk = w[gi * g:(gi + 1) * g]
+            amax = np.abs(blk).max(axis=0).astype(np.float32)
+            if group_size == -1:
+                amax = np.where(amax == 0, blk[0], amax).astype(np.float32)
+            s = (amax / np.float32(127.0)).astype(np.float32)
+            scale[gi] = s
+            r = (blk / s[None, :]).astype(np.float32).astype(np.float64)
+            rounded = np.where(r >= 0, np.floor(r + 0.5), np.ceil(r - 0.5))
+            c = np.where(np.isnan(rounded), 127.0, np.clip(rounded, -127.0, 127.0))
+            q[gi * g:(gi + 1) * g] = c.astype(np.int32)
+    return q, (scale[0] if group_size == -1 else scale)
+
+
 def canonical_from_q(q, bits):
     """signed codes [K,N] -> canonical tensor ([K,N] int8 or [K,N/2] nibbles)."""
     if bits == 8:

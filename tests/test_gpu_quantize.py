@@ -38,6 +38,39 @@ def test_quantize_bit_exact_all_layouts(G, oracle, dt, bits, g):
 
 
 @pytest.mark.parametrize("dt", [H.F16, H.BF16])
+@pytest.mark.parametrize("g", [-1, 64, 128])
+def test_quantize_llm_int8_flavour_bit_exact(G, oracle, dt, g):
+    # algo="llm.int8": fp32 scales, codes as the plain [N,K] transpose (what the
+    # reference returns for it) and in the other two layouts
+    for K, N in SHAPES:
+        for adv in (False, True):
+            wb = H.adversarial_weight(K, N, dt) if adv else H.make_weight(K, N, dt, seed=K + N)
+            oc, osc = oracle.weight_quantize_llm_int8(wb, dt, g)
+            gh, gs = G.quantize_llm_int8(wb, dt, g, layout=1)
+            assert np.array_equal(gs.view(np.uint32), osc.view(np.uint32))
+            assert np.array_equal(gh.view(np.int8).reshape(N, K), oc.T)
+            gc, _ = G.quantize_llm_int8(wb, dt, g, layout=0)
+            assert np.array_equal(gc.view(np.int8).reshape(K, N), oc)
+            gp, _ = G.quantize_llm_int8(wb, dt, g, layout=2)
+            assert np.array_equal(gp, H.gfx950_from_q(oc.astype(np.int32), 8))
+
+
+def test_python_api_llm_int8(device, oracle):
+    import torch
+    from paddle_amd.nn import quant as Q
+
+    wb = H.make_weight(256, 64, H.F16, seed=5)
+    w = H.bits_to_torch(wb, H.F16, torch.device("cuda:0"))
+    out, scale = Q.weight_quantize(w, algo="llm.int8")
+    oc, osc = oracle.weight_quantize_llm_int8(wb, H.F16, -1)
+    assert out.dtype == torch.int8 and tuple(out.shape) == (64, 256) and scale.dtype == torch.float32
+    assert np.array_equal(out.cpu().numpy(), oc.T)
+    assert np.array_equal(scale.cpu().numpy().view(np.uint32), osc.view(np.uint32))
+    with pytest.raises(ValueError):  # weight_dequantize refuses llm.int8 (binary.cc:4521-4525)
+        Q.weight_dequantize(out, scale.half(), algo="llm.int8")
+
+
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
 @pytest.mark.parametrize("bits", [8, 4])
 def test_quantize_truncating_scale_flavour(G, oracle, dt, bits):
     K, N = 256, 128

@@ -88,6 +88,35 @@ def test_quantize_matches_numpy_statement(oracle, dt, bits, g):
             assert np.array_equal(codes, H.canonical_from_q(q, bits))
 
 
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+@pytest.mark.parametrize("g", GROUPS)
+def test_llm_int8_flavour_matches_numpy_statement(oracle, dt, g):
+    # algo="llm.int8": fp32 scales (no cast), codes divided by them.  Beyond the
+    # numpy statement: scale * 127 returns the column maximum to one fp32 ulp,
+    # every non-degenerate group reaches |code| = 127, and the codes differ from
+    # the T-scale flavour's only where the scale rounding moved a quotient
+    # across a rounding boundary (never by more than one step).
+    for K, N in SHAPES:
+        wb = H.make_weight(K, N, dt, seed=K * 3 + N)
+        codes, scale = oracle.weight_quantize_llm_int8(wb, dt, g)
+        q, s = H.np_quantize_llm_int8(wb, dt, g)
+        assert scale.dtype == np.float32 and np.array_equal(scale.view(np.uint32), s.view(np.uint32))
+        assert np.array_equal(codes.astype(np.int32), q)
+        w = H.bits_to_f32(wb, dt)
+        gs = K if g == -1 else g
+        amax = np.stack([np.abs(w[i:i + gs]).max(axis=0) for i in range(0, K, gs)])
+        assert np.allclose(scale.reshape(amax.shape) * np.float32(127.0), amax, rtol=2e-7, atol=0)
+        top = np.stack([np.abs(codes[i:i + gs].astype(np.int32)).max(axis=0) for i in range(0, K, gs)])
+        assert (top[amax > 0] == 127).all()
+        tcodes, _ = oracle.weight_quantize(wb, dt, 8, g)
+        assert np.abs(codes.astype(np.int32) - tcodes.astype(np.int32)).max() <= 1
+    adv = H.adversarial_weight(128, 64, dt)
+    codes, scale = oracle.weight_quantize_llm_int8(adv, dt, g)
+    q, s = H.np_quantize_llm_int8(adv, dt, g)
+    assert np.array_equal(codes.astype(np.int32), q)
+    assert np.array_equal(scale.view(np.uint32), s.view(np.uint32))
+
+
 def test_zero_column_known_answers(oracle):
     # Recorded from the reference header: an all-zero column gives scale bits
     # 0x0000, int8 code 127 and int4 nibble 0x9 (-7), for fp16 and bf16.
