@@ -317,6 +317,46 @@ def _linear_call(fn, x, weight, bias, weight_scale, weight_dtype, group_size, ou
     return out
 
 
+def weight_only_linear_grad(x, weight, bias, weight_scale, out_grad, weight_dtype="int8", arch=None,
+                            group_size=-1):
+    """x_grad of weight_only_linear, composed as the reference composes it
+    (paddle/phi/kernels/gpu/weight_only_linear_grad_kernel.cu:52-69): the weight
+    is dequantised to T with this library's kernel and multiplied by the
+    library GEMM (torch.matmul standing in for phi::MatmulKernel):
+    x_grad[M,K] = out_grad[M,N] . dequant(W)[K,N]^T.  The reference restricts
+    this op to per-channel scales and arch 80/86; every group size works here.
+    x is only used for its shape (no_need_buffer in the reference's backward.yaml)."""
+    algo = "weight_only_int8" if weight_dtype == "int8" else "weight_only_int4"
+    names = {torch.float16: "float16", torch.bfloat16: "bfloat16"}
+    if out_grad.dtype not in names:
+        raise ValueError("(InvalidArgument) out_grad must be float16 or bfloat16")
+    wdq = weight_dequantize(weight, weight_scale, algo=algo, out_dtype=names[out_grad.dtype],
+                            group_size=group_size)
+    g2 = out_grad.reshape(-1, out_grad.shape[-1])
+    return torch.matmul(g2, wdq.t()).reshape(x.shape)
+
+
+class _WeightOnlyLinearFn(torch.autograd.Function):
+    """weight_only_linear with the reference's backward (x_grad only: the
+    quantised weight, its scale and the bias get no gradient, backward.yaml:3651-3661)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, weight_scale, weight_dtype, group_size):
+        ctx.save_for_backward(weight, weight_scale)
+        ctx.meta = (weight_dtype, group_size, x.shape)
+        return _linear_call(_lib.lib.wol_linear, x, weight, bias, weight_scale, weight_dtype,
+                            group_size, None)
+
+    @staticmethod
+    def backward(ctx, out_grad):
+        weight, weight_scale = ctx.saved_tensors
+        weight_dtype, group_size, x_shape = ctx.meta
+        x_like = torch.empty(x_shape, dtype=out_grad.dtype, device="meta")
+        gx = weight_only_linear_grad(x_like, weight, None, weight_scale, out_grad.contiguous(),
+                                     weight_dtype, None, group_size)
+        return gx, None, None, None, None, None
+
+
 def weight_only_linear(x, weight, bias=None, weight_scale=None, weight_dtype="int8", arch=None,
                        group_size=-1):
     """out = x . dequant(weight) + bias, in x's dtype (fp32 accumulation, one
@@ -329,6 +369,8 @@ def weight_only_linear(x, weight, bias=None, weight_scale=None, weight_dtype="in
     ), f"Currently weight_quantize only support group size of -1, 64 or 128. but got {group_size} "
     if weight_scale is None:
         raise ValueError("(InvalidArgument) weight_scale is required")
+    if x.requires_grad and torch.is_grad_enabled():
+        return _WeightOnlyLinearFn.apply(x, weight, bias, weight_scale, weight_dtype, group_size)
     return _linear_call(_lib.lib.wol_linear, x, weight, bias, weight_scale, weight_dtype,
                         group_size, None)
 
