@@ -907,6 +907,20 @@ inline int plan_split(int M, int K, int N, int bits, size_t lds, size_t ws_bytes
   return best;
 }
 
+// K runs for the 128 x 256 configuration when its tiles leave CUs idle: as
+// many runs as fit the idle CUs (2..4), each at least 8 k tiles long, and
+// only if the scratch buffer holds them.  The extra traffic (ns x M x N fp32,
+// written and read once) is worth it below half occupancy.
+inline int plan_split_large(int M, int K, int N, int bits, bool grouped, size_t ws_bytes) {
+  if (bits == 8 && !grouped && plan_big_columns(M, N) > 0) return 1;  // 256-row tiles are in play
+  const int tk = bits == 8 ? 64 : 128, tiles = K / tk;
+  const int blocks = ((N + 255) / 256) * ((M + 127) / 128);
+  int ns = num_cus() / blocks;
+  ns = ns > 4 ? 4 : ns;
+  while (ns > 1 && (tiles / ns < 8 || static_cast<size_t>(ns) * M * N * sizeof(float) > ws_bytes)) --ns;
+  return ns < 1 ? 1 : ns;
+}
+
 template <int BITS>
 size_t skinny_lds(int M) {  // with group scales (the larger footprint)
   if (BITS == 4 && M <= 32) return dma_lds_bytes<4, 64, 1, 8, 1, 1>();
@@ -931,11 +945,13 @@ void launch_fast(const Args& a) {
     const int c = plan_big_columns(a.M, a.N);
     const int hi = c * 16 < nstrips ? c * 16 : nstrips;
     launch_dma<DT, BITS, G, false, 2, 4, 4, 2>(a, 0, hi, 1);
-    launch_dma<DT, BITS, G, false, 2, 4, 2, 2>(a, hi, nstrips, 1);
+    const int ns = hi == 0 ? plan_split_large(a.M, a.K, a.N, BITS, false, a.ws != nullptr ? a.ws_bytes : 0) : 1;
+    launch_dma<DT, BITS, G, false, 2, 4, 2, 2>(a, hi, nstrips, ns);
   } else {
     // int4 tiles are 128 k deep and group-wise scales need a second set of
     // accumulators: 128 x 256 tiles
-    launch_dma<DT, BITS, G, false, 2, 4, 2, 2>(a, 0, nstrips, 1);
+    const int ns = plan_split_large(a.M, a.K, a.N, BITS, G != 0, a.ws != nullptr ? a.ws_bytes : 0);
+    launch_dma<DT, BITS, G, false, 2, 4, 2, 2>(a, 0, nstrips, ns);
   }
 }
 
@@ -957,9 +973,14 @@ void launch_cfg(const Args& a) {
 
 }  // namespace
 
-size_t linear_gemm_workspace(int64_t M, int64_t K, int64_t N, int bits) {
+size_t linear_gemm_workspace(int64_t M, int64_t K, int64_t N, int bits, bool grouped) {
   const int tk = bits == 8 ? 64 : 128;
-  if (M > kSkinnyMaxM || K % tk != 0 || K / tk < 2) return 0;
+  if (K % tk != 0 || K / tk < 2) return 0;
+  if (M > kSkinnyMaxM) {
+    const int ns = plan_split_large(static_cast<int>(M), static_cast<int>(K), static_cast<int>(N), bits,
+                                    grouped, SIZE_MAX);
+    return ns > 1 ? static_cast<size_t>(ns) * M * N * sizeof(float) : 0;
+  }
   const size_t lds = bits == 8 ? skinny_lds<8>(static_cast<int>(M)) : skinny_lds<4>(static_cast<int>(M));
   const int ns = plan_split(static_cast<int>(M), static_cast<int>(K), static_cast<int>(N), bits, lds, SIZE_MAX);
   return ns > 1 ? static_cast<size_t>(ns) * M * N * sizeof(float) : 0;

@@ -83,6 +83,12 @@ def test_linear_gemm_split_k_scratch_sizes(G, oracle):
     assert full >= 2 * M * N * 4 and full % (M * N * 4) == 0
     for wsb in (0, M * N * 4, 2 * M * N * 4, full - 4, full):
         check(G, oracle, dt, bits, g, M, K, N, seed=3, kernel=KERNEL_GEMM, ws_bytes=wsb)
+    # above 64 rows K is split only when the output tiles leave most CUs idle
+    for dt, bits, g, M, K, N in ((H.BF16, 8, -1, 100, 2048, 512), (H.F16, 4, 128, 130, 4096, 256)):
+        full = _lib.lib.wol_linear_workspace(M, K, N, bits, g)
+        assert full >= 2 * M * N * 4 and full % (M * N * 4) == 0
+        for wsb in (0, 2 * M * N * 4, full):
+            check(G, oracle, dt, bits, g, M, K, N, seed=4, ws_bytes=wsb)
 
 
 @pytest.mark.parametrize("bits", [8, 4])

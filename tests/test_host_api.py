@@ -48,6 +48,7 @@ def test_workspace_queries(lib):
     assert L.wol_quantize_workspace(4095, 11008, 4, 128) == 0  # invalid shape
     assert L.wol_linear_workspace(1, 4096, 11008, 4, 128) == 0       # streaming kernel
     assert L.wol_linear_workspace(2048, 4096, 12288, 8, -1) == 0     # one workgroup per tile covers all of K
+    assert L.wol_linear_workspace(1024, 4096, 4096, 8, 64) == 2 * 1024 * 4096 * 4  # 128 tiles: two K runs
     # small M on the GEMM: whole fp32 [M, N] partial buffers, at most 16 of them
     for M, K, N, bits, g in [(64, 8192, 28672, 4, 128), (32, 4096, 11008, 4, -1), (16, 8192, 28672, 4, 128)]:
         need = L.wol_linear_workspace(M, K, N, bits, g)
