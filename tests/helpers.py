@@ -68,7 +68,7 @@ def bits_to_f32(b, dt):
 
 def make_weight(K, N, dt, seed=1234, std=0.02, outlier_cols=0.0):
     """W ~ N(0, std) in fp32, optionally with a fraction of columns scaled x20,
-    then cast to T (RNE): the weight_quantize input of the BASELINE configs."""
+    then cast to T (RNE): the weight_quantize input of the benchmark configurations."""
     rng = np.random.default_rng(seed)
     w = rng.standard_normal((K, N), dtype=np.float32) * np.float32(std)
     if outlier_cols > 0:
