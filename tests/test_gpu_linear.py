@@ -115,6 +115,26 @@ def test_both_kernels_agree_on_full_size_decode_shape(G, oracle):
     assert H.rel_l2(b, r32) <= 2e-5
 
 
+def test_linear_random_shapes_all_kernels(G, oracle):
+    # seeded sweep over the whole contract: any M, K a multiple of 64 (so both
+    # the k-tile-aligned and the ragged GEMM paths, and int4 strips that end in
+    # a half tile), N a multiple of 16 (32 for int4), every kernel that accepts
+    # the shape, with and without bias
+    rng = np.random.default_rng(20240607)
+    for case in range(36):
+        dt = [H.F16, H.BF16][int(rng.integers(2))]
+        bits = [8, 4][int(rng.integers(2))]
+        g = [-1, 64, 128][int(rng.integers(3))]
+        M = int(rng.choice([1, 2, 5, 8, 9, 13, 16, 20, 31, 33, 50, 64, 65, 96, 129, 200, 257]))
+        K = 64 * int(rng.integers(1, 33))
+        N = (32 if bits == 4 else 16) * int(rng.integers(1, 41))
+        kernels = [None, KERNEL_GEMM] + ([KERNEL_STREAM] if M <= 64 else [])
+        kernel = kernels[int(rng.integers(len(kernels)))]
+        print("case", case, dt, bits, g, M, K, N, kernel, flush=True)
+        kw = {} if kernel is None else {"kernel": kernel}
+        check(G, oracle, dt, bits, g, M, K, N, bias=bool(rng.integers(2)), seed=case, **kw)
+
+
 @pytest.mark.parametrize("dt,bits,g", [(H.F16, 8, -1), (H.BF16, 4, 128), (H.F16, 4, 64)])
 def test_x_grad_through_autograd(device, oracle, dt, bits, g):
     # weight_only_linear_grad as the reference composes it (dequantise to T, then
