@@ -369,8 +369,8 @@ struct DmaParams {
 // rate on gfx950 (the 16x16x32 form issues at half of it), so the wavefront
 // tile is built from 32 x 32 blocks: TM x TN of them.  Both operands travel
 // global -> LDS with direct-to-LDS loads (no registers, no LDS store
-// instructions), three k tiles deep: while tile `it` is consumed the loads of
-// tiles it+1 and it+2 are in flight.  A lands in LDS as unpadded rows whose
+// instructions), STAGES k tiles deep: while tile `it` is consumed the loads of
+// tiles it+1 (and, with three stages, it+2) are in flight.  A lands in LDS as unpadded rows whose
 // 16-byte pieces are XOR-swizzled by row so a lane group's fragment reads
 // fall into distinct banks.  The raw packed B tiles land exactly as they lie
 // in memory (16-column strips in 16x16x32 order); a 32x32x16 B operand is
@@ -393,7 +393,7 @@ struct DmaParams {
 // With nsplit > 1 a workgroup covers only a run of k tiles and leaves its
 // fp32 sums (scaled, without bias) in a partial buffer; reduce_partials_kernel
 // adds the runs.  That is what fills the CUs when M is small.
-template <int DT, int BITS, int G, bool OFFS, int WM, int WN, int TM, int TN>
+template <int DT, int BITS, int G, bool OFFS, int WM, int WN, int TM, int TN, int STAGES>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   constexpr int NW = WM * WN;
@@ -405,7 +405,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   constexpr int kBBytes = (BN / 16) * 1024;      // one raw B tile (all strips of the workgroup)
   constexpr int kSBytes = G == 0 ? 0 : NW * 256;  // the tile's group scales: 128 values per wavefront
   constexpr int kStage = kABytes + kBBytes + kSBytes;
-  constexpr int kStages = 3;
+  constexpr int kStages = STAGES;  // k tiles resident or in flight
+  static_assert(kStages == 2 || kStages == 3, "two or three stages");
   constexpr int kALoads = kABytes / 1024 / NW;   // wave-level loads (1 KiB each) per wavefront
   constexpr int kBLoads = BN / 16 / NW;
   static_assert(kABytes / 1024 % NW == 0 && kALoads >= 1, "A tile must split evenly over the wavefronts");
@@ -614,8 +615,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
 
   issue(0);
   issue(1);
-  issue(2);
-  wait_vmcnt<2 * kPerStage>();  // tile 0 has landed
+  if (kStages == 3) issue(2);
+  wait_vmcnt<(kStages - 1) * kPerStage>();  // tile 0 has landed
   __builtin_amdgcn_s_barrier();
   read_b(smem, braw[0]);
   read_a(smem, af[0], 0);
@@ -659,9 +660,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
         // wavefront is there, tile it+1 (landed by now) may be read and the
         // stage refilled with tile it+3
         __builtin_amdgcn_s_waitcnt(0x0070 | (0xF << 0) | (3 << 14));  // lgkmcnt(0)
-        wait_vmcnt<kPerStage>();
+        wait_vmcnt<(kStages - 2) * kPerStage>();
         __builtin_amdgcn_s_barrier();
-        issue(it + 3);
+        issue(it + kStages);
         read_b(next, raw_next);
         dequant(bf[(q + 1) & 1], raw, q + 1);
         mfmas(af[q & 1], bf[q & 1], q, kHalf, TM * TN);
@@ -815,20 +816,20 @@ void launch_one(const Args& a) {
       a.N, a.gshift, a.out_f32, nbx, nby);
 }
 
-template <int BITS, int G, int WM, int WN, int TM, int TN>
+template <int BITS, int G, int WM, int WN, int TM, int TN, int STAGES = 3>
 constexpr size_t dma_lds_bytes() {
-  return 3 * (static_cast<size_t>(WM * TM * 32) * (BITS == 8 ? 64 : 128) * 2 +
+  return STAGES * (static_cast<size_t>(WM * TM * 32) * (BITS == 8 ? 64 : 128) * 2 +
               (WN * TN * 32 / 16) * 1024 + (G == 0 ? 0 : WM * WN * 256));
 }
 
 // Launches the fast kernel on the columns of strips [strip_lo, strip_hi), K
 // cut into nsplit runs (nsplit > 1 needs a.ws and covers every column).
-template <int DT, int BITS, int G, bool OFFS, int WM, int WN, int TM, int TN>
+template <int DT, int BITS, int G, bool OFFS, int WM, int WN, int TM, int TN, int STAGES = 3>
 void launch_dma(const Args& a, int strip_lo, int strip_hi, int nsplit) {
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32, TK = BITS == 8 ? 64 : 128;
   if (strip_hi <= strip_lo) return;
-  constexpr size_t lds = dma_lds_bytes<BITS, G, WM, WN, TM, TN>();
-  auto kern = gemm_dma_kernel<DT, BITS, G, OFFS, WM, WN, TM, TN>;
+  constexpr size_t lds = dma_lds_bytes<BITS, G, WM, WN, TM, TN, STAGES>();
+  auto kern = gemm_dma_kernel<DT, BITS, G, OFFS, WM, WN, TM, TN, STAGES>;
   static bool configured = false;
   if (!configured) {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -881,7 +882,10 @@ inline int plan_big_columns(int M, int N) {
 }
 
 // Rows up to which the small-M configurations (one row block of 32 or 64
-// rows, 256 columns, K split across workgroups) are used.
+// rows, 256 columns, K split across workgroups) are used.  They run two
+// stages deep instead of three: the smaller LDS footprint lets a third (32
+// rows) or second (64 rows, int4) workgroup share the CU, which hides more
+// latency than the third stage did.
 constexpr int kSkinnyMaxM = 64;
 
 // Split of K for the small-M configurations: the number of runs that
@@ -923,8 +927,8 @@ inline int plan_split_large(int M, int K, int N, int bits, bool grouped, size_t 
 
 template <int BITS>
 size_t skinny_lds(int M) {  // with group scales (the larger footprint)
-  if (BITS == 4 && M <= 32) return dma_lds_bytes<4, 64, 1, 8, 1, 1>();
-  return dma_lds_bytes<BITS, 64, 1, 8, 2, 1>();
+  if (BITS == 4 && M <= 32) return dma_lds_bytes<4, 64, 1, 8, 1, 1, 2>();
+  return dma_lds_bytes<BITS, 64, 1, 8, 2, 1, 2>();
 }
 
 template <int DT, int BITS, int G>
@@ -933,9 +937,9 @@ void launch_fast(const Args& a) {
   if (a.M <= kSkinnyMaxM) {
     const int ns = plan_split(a.M, a.K, a.N, BITS, skinny_lds<BITS>(a.M), a.ws != nullptr ? a.ws_bytes : 0);
     if constexpr (BITS == 4) {
-      if (a.M <= 32) { launch_dma<DT, BITS, G, true, 1, 8, 1, 1>(a, 0, nstrips, ns); return; }
+      if (a.M <= 32) { launch_dma<DT, BITS, G, true, 1, 8, 1, 1, 2>(a, 0, nstrips, ns); return; }
     }
-    launch_dma<DT, BITS, G, false, 1, 8, 2, 1>(a, 0, nstrips, ns);
+    launch_dma<DT, BITS, G, false, 1, 8, 2, 1, 2>(a, 0, nstrips, ns);
     return;
   }
   if constexpr (BITS == 8 && G == 0) {
