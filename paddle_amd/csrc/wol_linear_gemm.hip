@@ -128,6 +128,23 @@ __device__ inline void tile_of_block(int id, int nbx, int nby, int* bx, int* by)
   *bx = t / nby;
 }
 
+// The same with a two-dimensional split: the 8 XCDs form a grid of rg x 8/rg
+// and each owns nby/rg row blocks x nbx/(8/rg) column blocks, the shape that
+// makes the sum of the A rows and B columns an L2 has to fetch smallest
+// (plan_xcd_rows on the host).  rg == 0: plain order.
+__device__ inline void tile_of_block_2d(int id, int nbx, int nby, int rg, int* bx, int* by) {
+  if (rg == 0) {
+    *by = id % nby;
+    *bx = id / nby;
+    return;
+  }
+  constexpr int kXcd = 8;
+  const int x = id % kXcd, i = id / kXcd;
+  const int r = nby / rg, c = nbx / (kXcd / rg);
+  *by = (x % rg) * r + i % r;
+  *bx = (x / rg) * c + i / r;
+}
+
 template <int DT, int BITS, bool GROUPED, int WM, int WN, int TM, int TN>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(
     const uint16_t* __restrict__ x, const uint8_t* __restrict__ codes,
@@ -360,7 +377,7 @@ struct DmaParams {
   int strip_lo, strip_hi;       // the launch covers the 16-column strips [strip_lo, strip_hi)
   int nbx, nby;                 // output tiles of the launch
   int nsplit, tiles_per_split;  // K is cut into nsplit runs of k tiles, one workgroup each
-  int rotate;                   // start each column tile's run at a different k tile
+  int xcd_rows;                 // row groups of the XCD grid (tile_of_block), 0 = plain order
 };
 
 // Fast path: K a multiple of the tile depth.
@@ -436,7 +453,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   const int ntiles = p.nbx * p.nby;
   const int split = blockIdx.x / ntiles;
   int bx, by;
-  tile_of_block(blockIdx.x - split * ntiles, p.nbx, p.nby, &bx, &by);
+  tile_of_block_2d(blockIdx.x - split * ntiles, p.nbx, p.nby, p.xcd_rows, &bx, &by);
   const int m0 = by * BM;
   const int strip_blk = p.strip_lo + bx * (BN / 16);
   const int nstrips = p.strip_hi;
@@ -444,14 +461,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   // this workgroup's run of k tiles
   const int t0 = split * p.tiles_per_split;
   const int niter = (K / TK - t0) < p.tiles_per_split ? (K / TK - t0) : p.tiles_per_split;
-  // Strips lie a power of two apart when K is one, so workgroups that walk
-  // their k tiles in step would keep hitting the same few memory channels.
-  // With `rotate` each column tile starts its run somewhere else (the run
-  // wraps around; only the order of the fp32 additions changes).
-  const int rot = p.rotate ? (bx * 5 + split * 3) % niter : 0;
-  auto tile_index = [&](int it) {  // position in the run -> k tile of the run
-    int t = (it < niter ? it : niter - 1) + rot;
-    return t < niter ? t : t - niter;
+  auto tile_index = [&](int it) {  // past the end of the run: the last tile again
+    return it < niter ? it : niter - 1;
   };
 
   // global source of this lane for each of its A loads: LDS piece q holds row
@@ -816,6 +827,22 @@ void launch_one(const Args& a) {
       a.N, a.gshift, a.out_f32, nbx, nby);
 }
 
+// Row groups rg of the XCD grid for tile_of_block_2d: among the divisors of 8
+// that split both tile counts evenly, the one with the least bytes per XCD and
+// k step, rows * a_bytes + columns * b_bytes (bytes of one row block / column
+// block per k).  0 when the tiles do not divide over the XCDs.
+inline int plan_xcd_rows(int nbx, int nby, int a_bytes, int b_bytes) {
+  int best = 0;
+  int64_t best_cost = INT64_MAX;
+  for (int rg = 1; rg <= 8; rg *= 2) {
+    const int cg = 8 / rg;
+    if (nby % rg != 0 || nbx % cg != 0) continue;
+    const int64_t cost = static_cast<int64_t>(nby / rg) * a_bytes + static_cast<int64_t>(nbx / cg) * b_bytes;
+    if (cost < best_cost) { best_cost = cost; best = rg; }
+  }
+  return best;
+}
+
 template <int BITS, int G, int WM, int WN, int TM, int TN, int STAGES = 3>
 constexpr size_t dma_lds_bytes() {
   return STAGES * (static_cast<size_t>(WM * TM * 32) * (BITS == 8 ? 64 : 128) * 2 +
@@ -853,7 +880,7 @@ void launch_dma(const Args& a, int strip_lo, int strip_hi, int nsplit) {
   const int tiles = a.K / TK;
   p.tiles_per_split = (tiles + nsplit - 1) / nsplit;
   p.nsplit = (tiles + p.tiles_per_split - 1) / p.tiles_per_split;
-  p.rotate = p.nby == 1 ? 1 : 0;  // with several row blocks the L2 reuse of A wants them in step
+  p.xcd_rows = plan_xcd_rows(p.nbx, p.nby, BM * 2, BN * BITS / 8);
   kern<<<dim3(static_cast<unsigned>(p.nbx * p.nby * p.nsplit)), dim3(64 * WM * WN), lds, a.stream>>>(p);
   if (nsplit > 1) {
     const int64_t total = static_cast<int64_t>(a.M) * a.N;
