@@ -415,6 +415,11 @@ void launch_one(const Args& a) {
 template <int DT, int BITS, int MP, int MT>
 void launch_wk(const Args& a, int wk, int nu) {
   constexpr int kMaxWk = MT <= 2 ? 16 : 8;  // LDS for the cross-wavefront sums
+  if constexpr ((MP == 4 || MP == 8) && MT == 1) {
+    // several units per wavefront, still all in flight at once (8 wavefronts)
+    if (nu == 2) { launch_one<DT, BITS, MP, MT, 8, 2>(a); return; }
+    if (nu == 4) { launch_one<DT, BITS, MP, MT, 8, 4>(a); return; }
+  }
   if (nu == 1) {
     if (wk >= 16 && kMaxWk == 16) launch_one<DT, BITS, MP, MT, kMaxWk, 1>(a);
     else if (wk >= 8) launch_one<DT, BITS, MP, MT, 8, 1>(a);
@@ -463,6 +468,14 @@ static void pick_split(int64_t M, int64_t K, int64_t N, int bits, int* wk, int* 
       strips * nunits <= 6144) {
     *wk = static_cast<int>(nunits);
     *nu = 1;
+    return;
+  }
+  // 3 to 8 rows: units are short (4 k steps), so a strip has many of them;
+  // eight wavefronts with two or four units each still keep everything in flight
+  if (mp >= 4 && mp <= 8 && nunits * ku == nsteps && (nunits == 16 || nunits == 32) &&
+      strips * 8 <= 6144) {
+    *wk = 8;
+    *nu = static_cast<int>(nunits / 8);
     return;
   }
   int w = 1;
