@@ -453,8 +453,8 @@ void launch_m(const Args& a, int wk, int nu) {
 // enough that one unit per wavefront keeps every wavefront resident at once
 // (at most ~6 per SIMD on 1024 SIMDs) and the unit count per strip is a power
 // of two up to 16, each wavefront takes exactly one unit and loads it at once.
-// Otherwise wavefronts walk several units with two in flight, and WK aims at
-// about four wavefronts per SIMD.
+// Otherwise wavefronts walk several units with two in flight, and WK follows
+// a budget of resident wavefronts that shrinks with the row count.
 static void pick_split(int64_t M, int64_t K, int64_t N, int bits, int* wk, int* nu, int* tn) {
   int mp = 1;
   while (mp < 16 && mp < M) mp *= 2;
@@ -478,8 +478,11 @@ static void pick_split(int64_t M, int64_t K, int64_t N, int bits, int* wk, int* 
     *nu = static_cast<int>(nunits / 8);
     return;
   }
+  // measured: one or two rows want up to ~8 wavefronts per SIMD, full 16-row
+  // operands (more registers and LDS per wavefront) only one or two
+  const int64_t budget = mp <= 2 ? 8192 : (mp <= 8 ? 4096 : 2048);
   int w = 1;
-  while (w < maxwk && strips * w * 2 <= 4096 && w * 4 <= nunits) w *= 2;
+  while (w < maxwk && strips * w * 2 <= budget && w * 4 <= nunits) w *= 2;
   *wk = w;
   *nu = 0;
 }
