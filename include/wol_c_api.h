@@ -72,7 +72,7 @@ typedef enum wol_status {
   WOL_ERR_BAD_DTYPE = 2,      /* dtype not F16/BF16                             */
   WOL_ERR_BAD_BITS = 3,       /* bits not 8/4 (weight_dtype not int8/int4)      */
   WOL_ERR_BAD_GROUP_SIZE = 4, /* group_size not -1/64/128                       */
-  WOL_ERR_BAD_SHAPE = 5,      /* K % 64, N % 16, M < 0 ... (InferMeta contract) */
+  WOL_ERR_BAD_SHAPE = 5,      /* K % 64, N % 16, M < 0, a size above 2^24, ...   */
   WOL_ERR_BAD_LAYOUT = 6,     /* unknown layout id                              */
   WOL_ERR_BAD_ROUND_MODE = 7,
   WOL_ERR_WORKSPACE = 8,      /* workspace NULL or smaller than the query says  */

@@ -14,8 +14,9 @@ int check_problem(int dtype, int64_t K, int64_t N, int bits, int group_size) {
   if (bits != 8 && bits != 4) return WOL_ERR_BAD_BITS;
   if (!(group_size == -1 || group_size == 64 || group_size == 128)) return WOL_ERR_BAD_GROUP_SIZE;
   if (K <= 0 || N <= 0 || K % 64 != 0 || N % 16 != 0) return WOL_ERR_BAD_SHAPE;
-  // byte offsets inside a tensor are kept in int64; row indices in int32
-  if (K > (int64_t{1} << 30) || N > (int64_t{1} << 30)) return WOL_ERR_BAD_SHAPE;
+  // byte offsets inside a tensor are kept in int64; row, column and k-tile
+  // indices (and a k tile's byte offset inside a strip, K * 16) in int32
+  if (K > (int64_t{1} << 24) || N > (int64_t{1} << 24)) return WOL_ERR_BAD_SHAPE;
   return WOL_OK;
 }
 
@@ -61,7 +62,7 @@ int linear_impl(const void* x, const void* codes, const void* bias, const void* 
                 int kernel, void* workspace, size_t workspace_bytes, void* stream) {
   const int rc = check_problem(dtype, K, N, bits, group_size);
   if (rc != WOL_OK) return rc;
-  if (M < 0 || M > (int64_t{1} << 30)) return WOL_ERR_BAD_SHAPE;
+  if (M < 0 || M > (int64_t{1} << 24)) return WOL_ERR_BAD_SHAPE;
   if (kernel != WOL_KERNEL_AUTO && kernel != WOL_KERNEL_STREAM && kernel != WOL_KERNEL_GEMM)
     return WOL_ERR_BAD_SHAPE;
   if (kernel == WOL_KERNEL_STREAM && M > kStreamMaxM) return WOL_ERR_BAD_SHAPE;
@@ -90,7 +91,7 @@ const char* wol_status_str(int status) {
     case WOL_ERR_BAD_BITS: return "weight_dtype must be int8 or int4";
     case WOL_ERR_BAD_GROUP_SIZE: return "group_size must be -1, 64 or 128";
     case WOL_ERR_BAD_SHAPE:
-      return "shape outside the contract (K divisible by 64, N divisible by 16, sizes positive)";
+      return "shape outside the contract (K divisible by 64, N divisible by 16, sizes positive and at most 2^24)";
     case WOL_ERR_BAD_LAYOUT: return "unknown weight layout";
     case WOL_ERR_BAD_ROUND_MODE: return "round_mode must be RNE (0) or TRUNC (1)";
     case WOL_ERR_WORKSPACE: return "workspace missing or too small";

@@ -75,6 +75,7 @@ def test_argument_errors_return_before_device_work(lib):
     lin = lambda **kw: L.wol_linear(kw.get("x", p), p, None, p, kw.get("dt", 1), kw.get("M", 1), kw.get("K", 64),
                                     kw.get("N", 16), kw.get("bits", 4), kw.get("g", -1), p, None, 0, None)
     assert lin(dt=5) == 2 and lin(bits=2) == 3 and lin(g=100) == 4 and lin(K=100) == 5 and lin(M=-1) == 5
+    assert lin(K=(1 << 24) + 64) == 5 and lin(N=(1 << 24) + 16) == 5 and lin(M=(1 << 24) + 1) == 5
     assert lin(x=None) == 1
     assert lin(x=ctypes.c_void_p(0x1004)) == 9
     assert lin(M=0) == 0  # empty batch is a no-op
