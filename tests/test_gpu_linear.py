@@ -300,6 +300,33 @@ def _full_size_properties(dt, bits, g, M, K, N, outliers=0.0):
     assert torch.equal(outT, out32.to(tdt))
 
 
+def test_weight_larger_than_2_gib(device):
+    # byte offsets beyond 2^31: a 8192 x 327680 int8 weight (2.7 GB of codes).
+    # One-hot activations must read back the dequantised rows, also at the far
+    # end of the tensor, on the streaming kernel (M = 4) and the GEMM (M = 80).
+    import torch
+    from paddle_amd.nn import quant as Q
+    from paddle_amd.nn.quant import quantized_linear as QL
+
+    K, N = 8192, 327680
+    gen = torch.Generator(device="cuda").manual_seed(7)
+    w = torch.empty(K, N, device="cuda", dtype=torch.bfloat16)
+    for k0 in range(0, K, 1024):  # in slabs: randn has no bf16 generator path for 2.7 G elements at once
+        w[k0:k0 + 1024] = (torch.randn(1024, N, device="cuda", generator=gen) * 0.02).to(torch.bfloat16)
+    codes, scale = Q.weight_quantize(w, algo="weight_only_int8", group_size=128)
+    assert codes.numel() > 2 ** 31
+    wdq = Q.weight_dequantize(codes, scale, algo="weight_only_int8", out_dtype="bfloat16", group_size=128)
+    del w
+    for M in (4, 80):
+        ks = [0, 1, K // 2 + 3, K - 1][: min(4, M)]
+        onehot = torch.zeros(M, K, device="cuda", dtype=torch.bfloat16)
+        for i, k in enumerate(ks):
+            onehot[i, k] = 1.0
+        rows = QL.weight_only_linear_fp32(onehot, codes, None, scale, "int8", 128)
+        assert torch.equal(rows[: len(ks)].to(torch.bfloat16), wdq[ks])
+        assert not rows[len(ks):].any()
+
+
 @pytest.mark.parametrize("M", [1, 8, 32, 64])
 def test_config_3_full_size_properties(device, M):
     _full_size_properties(H.F16, 4, 128, M, 8192, 28672, outliers=0.01)
