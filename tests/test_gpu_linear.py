@@ -300,6 +300,43 @@ def _full_size_properties(dt, bits, g, M, K, N, outliers=0.0):
     assert torch.equal(outT, out32.to(tdt))
 
 
+def test_calls_replay_correctly_from_a_hip_graph(device):
+    # Every entry point is stream-ordered and allocation-free, so a captured
+    # sequence must replay to the eager results: quantise (per-channel, with its
+    # scratch), decode, the small-M GEMM with its K runs and reduction, the
+    # prefill GEMM.  Replayed three times with eager work in between.
+    import torch
+    from paddle_amd.nn import quant as Q
+
+    dev = torch.device("cuda:0")
+    K, N = 2048, 1024
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    w = (torch.randn(K, N, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+    xs = {M: torch.randn(M, K, device=dev, generator=gen).to(torch.bfloat16) for M in (1, 40, 300)}
+
+    def work():
+        codes, scale = Q.weight_quantize(w, algo="weight_only_int8", group_size=-1)
+        c4, s4 = Q.weight_quantize(w, algo="weight_only_int4", group_size=128)
+        outs = [Q.weight_only_linear(x, codes, None, scale, "int8", None, -1) for x in xs.values()]
+        outs += [Q.weight_only_linear(x, c4, None, s4, "int4", None, 128) for x in xs.values()]
+        return [codes, scale, c4, s4] + outs
+
+    eager = [t.clone() for t in work()]
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        captured = work()
+    for rep in range(3):
+        for t in captured:
+            t.zero_()
+        _ = work()  # eager work between the replays
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(eager, captured):
+            assert torch.equal(a, b), rep
+
+
 def test_weight_larger_than_2_gib(device):
     # byte offsets beyond 2^31: a 8192 x 327680 int8 weight (2.7 GB of codes).
     # One-hot activations must read back the dequantised rows, also at the far
