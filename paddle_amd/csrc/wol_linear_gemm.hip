@@ -889,7 +889,7 @@ void launch_dma(const Args& a, int strip_lo, int strip_hi, int nsplit) {
   }
 }
 
-// The half-size tile of the int8 per-channel path: 256 x 128 (four A blocks
+// The half-size tile of the int8 paths: 256 x 128 (four A blocks
 // share each dequantised B block: less VALU work per MFMA, 9 % faster than
 // 128 x 256 at M = 512) unless its 256-row blocks would pad M much further
 // than 128-row blocks do.
@@ -955,7 +955,7 @@ inline int plan_split(int M, int K, int N, int bits, size_t lds, size_t ws_bytes
 inline int plan_split_large(int M, int K, int N, int bits, bool grouped, size_t ws_bytes) {
   if (bits == 8 && !grouped && plan_big_columns(M, N) > 0) return 1;  // 256-row tiles are in play
   const int tk = bits == 8 ? 64 : 128, tiles = K / tk;
-  const bool tall = bits == 8 && !grouped && tall_half_tile(M);
+  const bool tall = bits == 8 && tall_half_tile(M);
   const int blocks = tall ? ((N + 127) / 128) * ((M + 255) / 256) : ((N + 255) / 256) * ((M + 127) / 128);
   int ns = num_cus() / blocks;
   ns = ns > 4 ? 4 : ns;
@@ -994,6 +994,9 @@ void launch_fast(const Args& a) {
     // int4 tiles are 128 k deep and group-wise scales need a second set of
     // accumulators: 128 x 256 tiles
     const int ns = plan_split_large(a.M, a.K, a.N, BITS, G != 0, a.ws != nullptr ? a.ws_bytes : 0);
+    if constexpr (BITS == 8) {
+      if (tall_half_tile(a.M)) { launch_dma<DT, BITS, G, false, 2, 4, 4, 1>(a, 0, nstrips, ns); return; }
+    }
     launch_dma<DT, BITS, G, false, 2, 4, 2, 2>(a, 0, nstrips, ns);
   }
 }
