@@ -158,7 +158,7 @@ size_t wol_linear_workspace_for(int64_t M, int64_t K, int64_t N, int bits, int g
   if (check_problem(WOL_DTYPE_F16, K, N, bits, group_size) != WOL_OK || M <= 0) return 0;
   if (kernel == WOL_KERNEL_STREAM && M > kStreamMaxM) return 0;
   if (resolve_stream(kernel, M, K, N, bits)) return 0;  // partial sums stay on chip
-  return wol::linear_gemm_workspace(M, K, N, bits, group_size > 0);
+  return wol::linear_gemm_workspace(M, K, N, bits, group_size);
 }
 
 int wol_linear(const void* x, const void* codes, const void* bias, const void* scale, int dtype,

@@ -211,7 +211,7 @@ int launch_linear_gemm(const void* x, const void* codes, const void* bias, const
                        void* out, bool out_f32, void* workspace, size_t workspace_bytes,
                        hipStream_t stream);
 // Scratch bytes with which launch_linear_gemm splits K across workgroups (0: none needed).
-size_t linear_gemm_workspace(int64_t M, int64_t K, int64_t N, int bits, bool grouped);
+size_t linear_gemm_workspace(int64_t M, int64_t K, int64_t N, int bits, int group_size);
 
 inline int check_launch() {
   return hipGetLastError() == hipSuccess ? WOL_OK : WOL_ERR_HIP;

@@ -952,11 +952,13 @@ inline int plan_split(int M, int K, int N, int bits, size_t lds, size_t ws_bytes
 // many runs as fit the idle CUs (2..4), each at least 8 k tiles long, and
 // only if the scratch buffer holds them.  The extra traffic (ns x M x N fp32,
 // written and read once) is worth it below half occupancy.
-inline int plan_split_large(int M, int K, int N, int bits, bool grouped, size_t ws_bytes) {
-  if (bits == 8 && !grouped && plan_big_columns(M, N) > 0) return 1;  // 256-row tiles are in play
+inline int plan_split_large(int M, int K, int N, int bits, int group, size_t ws_bytes) {
+  if (bits == 8 && group == 0 && plan_big_columns(M, N) > 0) return 1;  // 256-row tiles are in play
   const int tk = bits == 8 ? 64 : 128, tiles = K / tk;
-  const bool tall = bits == 8 && tall_half_tile(M);
-  const int blocks = tall ? ((N + 127) / 128) * ((M + 255) / 256) : ((N + 255) / 256) * ((M + 127) / 128);
+  // tile of the configuration launch_fast picks: 256 x 128 or 128 x 256 (int8), 128 x 128 (int4, group 64)
+  const int bm = bits == 8 && tall_half_tile(M) ? 256 : 128;
+  const int bn = bm == 256 || (bits == 4 && group == 64) ? 128 : 256;
+  const int blocks = ((N + bn - 1) / bn) * ((M + bm - 1) / bm);
   int ns = num_cus() / blocks;
   ns = ns > 4 ? 4 : ns;
   while (ns > 1 && (tiles / ns < 8 || static_cast<size_t>(ns) * M * N * sizeof(float) > ws_bytes)) --ns;
@@ -987,17 +989,28 @@ void launch_fast(const Args& a) {
     const int c = plan_big_columns(a.M, a.N);
     const int hi = c * 16 < nstrips ? c * 16 : nstrips;
     launch_dma<DT, BITS, G, false, 2, 4, 4, 2>(a, 0, hi, 1);
-    const int ns = hi == 0 ? plan_split_large(a.M, a.K, a.N, BITS, false, a.ws != nullptr ? a.ws_bytes : 0) : 1;
+    const int ns = hi == 0 ? plan_split_large(a.M, a.K, a.N, BITS, 0, a.ws != nullptr ? a.ws_bytes : 0) : 1;
     if (tall_half_tile(a.M)) launch_dma<DT, BITS, G, false, 2, 4, 4, 1>(a, hi, nstrips, ns);
     else launch_dma<DT, BITS, G, false, 2, 4, 2, 2>(a, hi, nstrips, ns);
   } else {
     // int4 tiles are 128 k deep and group-wise scales need a second set of
     // accumulators: 128 x 256 tiles
-    const int ns = plan_split_large(a.M, a.K, a.N, BITS, G != 0, a.ws != nullptr ? a.ws_bytes : 0);
+    const int ns = plan_split_large(a.M, a.K, a.N, BITS, G, a.ws != nullptr ? a.ws_bytes : 0);
     if constexpr (BITS == 8) {
       if (tall_half_tile(a.M)) { launch_dma<DT, BITS, G, false, 2, 4, 4, 1>(a, 0, nstrips, ns); return; }
+      launch_dma<DT, BITS, G, false, 2, 4, 2, 2>(a, 0, nstrips, ns);
+    } else if constexpr (G == 64) {
+      // two groups per k tile: two scale sets on top of two accumulator sets do
+      // not fit 256 registers at 128 x 256 (the spills, being memory loads,
+      // also break the in-order accounting of the tile loads): 128 x 128
+      launch_dma<DT, BITS, G, false, 2, 4, 2, 1>(a, 0, nstrips, ns);
+    } else if constexpr (G == 0 && DT == WOL_DTYPE_BF16) {
+      // the exact int4 -> bf16 dequantiser costs 32 VALU instructions per 8
+      // codes; the offset form plus one cancelling MFMA per A block is faster
+      launch_dma<DT, BITS, G, true, 2, 4, 2, 2>(a, 0, nstrips, ns);
+    } else {
+      launch_dma<DT, BITS, G, false, 2, 4, 2, 2>(a, 0, nstrips, ns);
     }
-    launch_dma<DT, BITS, G, false, 2, 4, 2, 2>(a, 0, nstrips, ns);
   }
 }
 
@@ -1019,12 +1032,12 @@ void launch_cfg(const Args& a) {
 
 }  // namespace
 
-size_t linear_gemm_workspace(int64_t M, int64_t K, int64_t N, int bits, bool grouped) {
+size_t linear_gemm_workspace(int64_t M, int64_t K, int64_t N, int bits, int group_size) {
   const int tk = bits == 8 ? 64 : 128;
   if (K % tk != 0 || K / tk < 2) return 0;
   if (M > kSkinnyMaxM) {
     const int ns = plan_split_large(static_cast<int>(M), static_cast<int>(K), static_cast<int>(N), bits,
-                                    grouped, SIZE_MAX);
+                                    group_size > 0 ? group_size : 0, SIZE_MAX);
     return ns > 1 ? static_cast<size_t>(ns) * M * N * sizeof(float) : 0;
   }
   const size_t lds = bits == 8 ? skinny_lds<8>(static_cast<int>(M)) : skinny_lds<4>(static_cast<int>(M));
