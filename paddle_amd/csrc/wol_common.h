@@ -187,6 +187,7 @@ __device__ inline uint16_t cast_out(float f) {
 // number of workgroups: worth it once that traffic is at least twice the
 // weight bytes (rows / bits >= 2) and enough workgroups remain.
 inline int stream_strips_per_workgroup(int64_t M, int64_t N, int bits) {
+  if (M > 16) return 1;  // several 16-row operands per strip already fill the registers
   int rows = 1;
   while (rows < 16 && rows < M) rows *= 2;
   const int64_t groups = N / kStripCols / 2;

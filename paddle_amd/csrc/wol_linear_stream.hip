@@ -398,10 +398,10 @@ void launch_tn(const Args& a) {
 }
 
 // Two strips per workgroup exist for the operand shapes whose activation
-// traffic matters (eight rows and up).
+// traffic matters and whose registers allow it (8 to 16 rows).
 template <int DT, int BITS, int MP, int MT, int WK, int NU>
 void launch_one(const Args& a) {
-  if constexpr (MP >= 8) {
+  if constexpr (MP >= 8 && MT == 1) {
     if (a.tn == 2) {
       launch_tn<DT, BITS, MP, MT, WK, NU, 2>(a);
       return;
@@ -427,8 +427,9 @@ void launch_wk(const Args& a, int wk, int nu) {
     else if (wk >= 2) launch_one<DT, BITS, MP, MT, 2, 1>(a);
     else launch_one<DT, BITS, MP, MT, 1, 1>(a);
   } else {
-    if (wk >= 16 && kMaxWk == 16) launch_one<DT, BITS, MP, MT, kMaxWk, 0>(a);
-    else if (wk >= 8) launch_one<DT, BITS, MP, MT, 8, 0>(a);
+    // (no 16-wavefront walking variant: 1024 threads leave 128 registers each,
+    // which the double-buffered units do not fit without spilling)
+    if (wk >= 8) launch_one<DT, BITS, MP, MT, 8, 0>(a);
     else if (wk >= 4) launch_one<DT, BITS, MP, MT, 4, 0>(a);
     else if (wk >= 2) launch_one<DT, BITS, MP, MT, 2, 0>(a);
     else launch_one<DT, BITS, MP, MT, 1, 0>(a);
@@ -482,7 +483,7 @@ static void pick_split(int64_t M, int64_t K, int64_t N, int bits, int* wk, int* 
   // operands (more registers and LDS per wavefront) only one or two
   const int64_t budget = mp <= 2 ? 8192 : (mp <= 8 ? 4096 : 2048);
   int w = 1;
-  while (w < maxwk && strips * w * 2 <= budget && w * 4 <= nunits) w *= 2;
+  while (w < 8 && strips * w * 2 <= budget && w * 4 <= nunits) w *= 2;
   *wk = w;
   *nu = 0;
 }

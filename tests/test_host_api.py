@@ -32,6 +32,23 @@ def test_library_exports_every_declared_symbol(lib):
         assert hasattr(raw, name), name
 
 
+def test_no_kernel_spills_registers():
+    # build.sh keeps the compiler's per-kernel resource remarks and refuses a
+    # build in which a kernel spills; this reads the same files (absent when the
+    # library was built elsewhere and only the .so travelled)
+    import glob
+
+    files = glob.glob(os.path.join(ROOT, "paddle_amd", "csrc", "build", "*.resources.txt"))
+    if not files:
+        pytest.skip("no resource remarks beside the build")
+    kernels = 0
+    for f in files:
+        text = open(f).read()
+        kernels += text.count("Function Name:")
+        assert not re.search(r"(VGPRs Spill|SGPRs Spill|ScratchSize \[bytes/lane\]): [1-9]", text), f
+    assert kernels > 500  # the streaming kernel alone has several hundred instantiations
+
+
 def test_status_strings_and_version(lib):
     L = lib.lib
     assert L.wol_layout_version() == 1
