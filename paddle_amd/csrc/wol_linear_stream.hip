@@ -427,8 +427,11 @@ void launch_wk(const Args& a, int wk, int nu) {
     else if (wk >= 2) launch_one<DT, BITS, MP, MT, 2, 1>(a);
     else launch_one<DT, BITS, MP, MT, 1, 1>(a);
   } else {
-    // (no 16-wavefront walking variant: 1024 threads leave 128 registers each,
-    // which the double-buffered units do not fit without spilling)
+    // 16 wavefronts (1024 threads) leave 128 registers each: enough for the
+    // double-buffered units of 2 to 8 rows, not for the others
+    if constexpr (MP >= 2 && MP <= 8) {
+      if (wk >= 16) { launch_one<DT, BITS, MP, MT, 16, 0>(a); return; }
+    }
     if (wk >= 8) launch_one<DT, BITS, MP, MT, 8, 0>(a);
     else if (wk >= 4) launch_one<DT, BITS, MP, MT, 4, 0>(a);
     else if (wk >= 2) launch_one<DT, BITS, MP, MT, 2, 0>(a);
@@ -483,7 +486,8 @@ static void pick_split(int64_t M, int64_t K, int64_t N, int bits, int* wk, int* 
   // operands (more registers and LDS per wavefront) only one or two
   const int64_t budget = mp <= 2 ? 8192 : (mp <= 8 ? 4096 : 2048);
   int w = 1;
-  while (w < 8 && strips * w * 2 <= budget && w * 4 <= nunits) w *= 2;
+  const int maxwalk = mp >= 2 && mp <= 8 ? 16 : 8;
+  while (w < maxwalk && strips * w * 2 <= budget && w * 4 <= nunits) w *= 2;
   *wk = w;
   *nu = 0;
 }
