@@ -256,7 +256,7 @@ def main():
                 "unit": "TFLOP/s",
                 "frac": round(pre_tf / MFMA_BF16_PEAK_TF, 4),
                 "traffic": traffic.get("prefill_bytes_per_launch"),
-                "kernel": "wol::gemm_dma_kernel<1, 8, 0, false, 2, 4, 4, 2, 3> (256 of 384 tiles) + <1, 8, 0, false, 2, 4, 2, 2, 3> (the rest as 128-row tiles)",
+                "kernel": "wol::gemm_dma_kernel<1, 8, 0, false, 2, 4, 4, 2, 3> (256x256 tiles on the columns that fill whole rounds of the 256 CUs) + <1, 8, 0, false, 2, 4, 4, 1, 3> (256x128 tiles on the rest)",
             },
         },
         "cpu_baseline": cpu,
