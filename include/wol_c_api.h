@@ -203,6 +203,23 @@ int wol_repack(const void* codes_in, int layout_in, void* codes_out,
 int64_t wol_code_offset(int layout, int64_t K, int64_t N, int bits, int64_t k,
                         int64_t n, int* nibble_shift);
 
+/*
+ * Replaces ApplyPerChannelScaleKernel<T, GPUContext>
+ * (paddle/phi/kernels/gpu/apply_per_channel_scale_kernel.cu:146-190, device
+ * kernel :93-126; shape contract ApplyPerChannelScaleInferMeta,
+ * paddle/phi/infermeta/binary.cc:3452-3481): the pre-quant smoothing of the
+ * activations in front of weight_only_linear,
+ *   out[r, c] = T( x[r, c] * scales[c] ),  one multiply rounded once (RNE).
+ * x and out are [rows, cols] T row-major, scales is [cols] T; out may be x.
+ * Any cols; rows and cols at most 2^24.  16-byte accesses are used when cols
+ * is a multiple of 8 and the three pointers are 16-byte aligned (the file it
+ * replaces supports only that case).  A NaN product is a NaN of unspecified
+ * payload.
+ */
+int wol_apply_per_channel_scale(const void* x, const void* scales, int dtype,
+                                int64_t rows, int64_t cols, void* out,
+                                void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -23,6 +23,10 @@
  *   dequant/linear: products of <=8-bit codes with <=11-bit scales are exact
  *                   in fp32, so dequant has one correct answer; the linear is
  *                   checked against a float64 matmul of the same operands.
+ *   pre-scale     : one correctly rounded multiply in T; pinned against the
+ *                   half-precision multiply of numpy (fp16) and torch (bf16),
+ *                   which are library routines with that definition, and by
+ *                   exactness cases (scale 1, powers of two).
  */
 #include <math.h>
 #include <stdint.h>
@@ -393,4 +397,20 @@ void wo_dequantize_f32(const int8_t* codes, const uint16_t* scale, int64_t K,
                        int nibble_bias, float* out32) {
   wo_dequantize(codes, scale, K, N, dtype, bits, group_size, nibble_bias,
                 WO_CAST_RNE, out32, NULL);
+}
+
+/* ---- pre-quant activation smoothing ------------------------------------ */
+
+/* out[r,c] = T(x[r,c] * scales[c]): ApplyPerChannelScaleKernel
+ * (paddle/phi/kernels/gpu/apply_per_channel_scale_kernel.cu:93-126), whose
+ * __hmul2 is the exact product rounded once to nearest even.  The product of
+ * two T values (at most 11 significant bits each) is exact in fp32. */
+void wo_apply_per_channel_scale(const uint16_t* x, const uint16_t* scales,
+                                int64_t rows, int64_t cols, int dtype,
+                                uint16_t* out) {
+  for (int64_t r = 0; r < rows; ++r)
+    for (int64_t c = 0; c < cols; ++c)
+      out[r * cols + c] = wo_from_f32(
+          wo_to_f32(x[r * cols + c], dtype) * wo_to_f32(scales[c], dtype), dtype,
+          WO_CAST_RNE);
 }

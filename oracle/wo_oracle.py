@@ -55,6 +55,8 @@ def lib():
         L.wo_weight_quantize_llm_int8.argtypes = [_u16p, _i64, _i64, _int, _i64, _i8p, _f32p]
         L.wo_weight_quantize_llm_int8.restype = _int
         L.wo_transpose_bytes.argtypes = [_i8p, _i64, _i64, _i8p]
+        L.wo_apply_per_channel_scale.argtypes = [_u16p, _u16p, _i64, _i64, _int, _u16p]
+        L.wo_apply_per_channel_scale.restype = None
         L.wo_dequantize.argtypes = [_i8p, _u16p, _i64, _i64, _int, _int, _i64, _int, _int,
                                     ctypes.c_void_p, ctypes.c_void_p]
         L.wo_linear.argtypes = [_u16p, _i8p, ctypes.c_void_p, _u16p, _i64, _i64, _i64, _int, _int,
@@ -104,6 +106,17 @@ def weight_quantize_llm_int8(w_bits, dtype, group_size=-1):
     if lib().wo_weight_quantize_llm_int8(w_bits, K, N, dtype, group_size, codes, scale) != 0:
         raise ValueError("oracle: shape/group_size outside the weight_quantize contract")
     return codes, scale
+
+
+def apply_per_channel_scale(x_bits, scale_bits, dtype):
+    """x_bits [rows, cols] uint16, scale_bits [cols] uint16 -> T-bits [rows, cols]."""
+    x_bits = np.ascontiguousarray(x_bits, dtype=np.uint16)
+    scale_bits = np.ascontiguousarray(scale_bits, dtype=np.uint16)
+    rows, cols = x_bits.shape
+    assert scale_bits.shape == (cols,)
+    out = np.empty((rows, cols), np.uint16)
+    lib().wo_apply_per_channel_scale(x_bits, scale_bits, rows, cols, dtype, out)
+    return out
 
 
 def transpose_bytes(a):

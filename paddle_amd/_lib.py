@@ -28,6 +28,7 @@ SYMBOLS = (
     "wol_linear_on",
     "wol_repack",
     "wol_code_offset",
+    "wol_apply_per_channel_scale",
 )
 
 
@@ -69,6 +70,8 @@ def _load():
     lib.wol_repack.restype = ci
     lib.wol_code_offset.argtypes = [ci, i64, i64, ci, i64, i64, ctypes.POINTER(ci)]
     lib.wol_code_offset.restype = i64
+    lib.wol_apply_per_channel_scale.argtypes = [vp, vp, ci, i64, i64, vp, vp]
+    lib.wol_apply_per_channel_scale.restype = ci
     return lib
 
 

@@ -204,4 +204,14 @@ int64_t wol_code_offset(int layout, int64_t K, int64_t N, int bits, int64_t k, i
   return off;
 }
 
+int wol_apply_per_channel_scale(const void* x, const void* scales, int dtype, int64_t rows,
+                                int64_t cols, void* out, void* stream) {
+  if (dtype != WOL_DTYPE_F16 && dtype != WOL_DTYPE_BF16) return WOL_ERR_BAD_DTYPE;
+  if (rows < 0 || cols <= 0 || rows > (int64_t{1} << 24) || cols > (int64_t{1} << 24))
+    return WOL_ERR_BAD_SHAPE;
+  if (rows == 0) return WOL_OK;
+  if (x == nullptr || scales == nullptr || out == nullptr) return WOL_ERR_NULL_POINTER;
+  return wol::launch_prescale(x, scales, dtype, rows, cols, out, static_cast<hipStream_t>(stream));
+}
+
 }  // extern "C"

@@ -1,7 +1,8 @@
-"""weight_quantize / weight_dequantize / weight_only_linear with the signatures,
-defaults, checks and error behaviour of paddle.nn.quant
-(python/paddle/nn/quant/quantized_linear.py:64-282 in the reference), computed
-by the gfx950 library through its C ABI.
+"""weight_quantize / weight_dequantize / weight_only_linear /
+apply_per_channel_scale with the signatures, defaults, checks and error
+behaviour of paddle.nn.quant (python/paddle/nn/quant/quantized_linear.py:64-282
+and :351-388 in the reference), computed by the gfx950 library through its C
+ABI.
 
 Tensors are torch tensors on the GPU; torch only provides the memory and the
 stream.  The shape checks restate the reference's InferMeta functions and raise
@@ -382,3 +383,47 @@ def weight_only_linear_fp32(x, weight, bias=None, weight_scale=None, weight_dtyp
     can be checked apart from the output rounding."""
     return _linear_call(_lib.lib.wol_linear_f32, x, weight, bias, weight_scale, weight_dtype,
                         group_size, torch.float32)
+
+
+def apply_per_channel_scale_infer_meta(x_shape, scales_shape):
+    """ApplyPerChannelScaleInferMeta (paddle/phi/infermeta/binary.cc:3452-3481):
+    x is 2-D, scales 1-D with x's second dimension; out has x's shape."""
+    if len(x_shape) != 2:
+        raise ValueError(
+            "(InvalidArgument) The rank of Input(x) must be 2, but received %d." % len(x_shape)
+        )
+    if len(scales_shape) != 1:
+        raise ValueError(
+            "(InvalidArgument) The rank of Input(scales) must be 1, but received %d."
+            % len(scales_shape)
+        )
+    if x_shape[1] != scales_shape[0]:
+        raise ValueError(
+            "(InvalidArgument) The second dim of Input(x) must be equal to the first dim of scales,"
+            "but received %d and %d." % (x_shape[1], scales_shape[0])
+        )
+    return tuple(x_shape)
+
+
+def apply_per_channel_scale(x, scales):
+    """Apply pre-quant per channel scale on activations: out = x * scales, in
+    x's dtype (python/paddle/nn/quant/quantized_linear.py:351-388)."""
+    out_shape = apply_per_channel_scale_infer_meta(tuple(x.shape), tuple(scales.shape))
+    dt = _dtype_id(x, "x")
+    if scales.dtype != x.dtype:
+        raise ValueError(
+            "(InvalidArgument) scales dtype %s does not match x dtype %s" % (scales.dtype, x.dtype)
+        )
+    _require_gpu(x, "x")
+    _require_gpu(scales, "scales")
+    x = x.contiguous()
+    scales = scales.contiguous()
+    out = torch.empty(out_shape, dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(
+            _lib.lib.wol_apply_per_channel_scale(
+                x.data_ptr(), scales.data_ptr(), dt, out_shape[0], out_shape[1], out.data_ptr(),
+                _stream_ptr(x),
+            )
+        )
+    return out
