@@ -84,11 +84,15 @@ struct StreamKernel {
   // (64 k) always share a group: one load per pair.  MP = 16 keeps every step.
   static constexpr int kPairs = kRowsPerGroup >= 2 ? kRowsPerGroup / 2 : 1;
   static constexpr int kNS = MP == 16 ? kU / 2 : kNA * kPairs;
+  // Walking wavefronts: K's whole weight tiles may end with a partial unit when
+  // a unit spans several tiles (otherwise they divide into whole units).
+  static constexpr bool kPartial = NU == 0 && kU > kSPT;
 
   const uint16_t* x;
   const uint16_t* scale;
   int M, K, N;
   int gshift;  // log2(group_size) when GROUPED
+  int vsteps;  // k steps that lie in whole 16-byte weight tiles (all but an int4 half tile)
   int lane, j, kb;
   int n[TN];  // this lane's column in each strip (clamped to the last valid one)
   uint32_t magic;
@@ -106,13 +110,18 @@ struct StreamKernel {
 
   // A operand whose row group `slot` holds k step (step0 + slot); with
   // spread == false every row group holds step0.
-  __device__ inline u32x4 load_a(int mt, int step0, bool spread) const {
+  // tail: the unit is the partial one that ends K.
+  __device__ inline u32x4 load_a(int mt, int step0, bool spread, bool tail = false) const {
     int m = mt * 16 + (j % MP);
     if (MP > 1 || MT > 1) m = m < M ? m : M - 1;  // rows past M are never stored
     int step = step0 + (spread ? j / MP : 0);
-    if (NU == 0) {  // a partial unit at the end of K must not read past the row
-      const int last = K / 32 - 1;
-      step = step < last ? step : last;
+    if (tail) {
+      // steps past the end read the
+      // last valid one (never past the row) and count as zero
+      const bool valid = step < vsteps;
+      step = valid ? step : vsteps - 1;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(x + static_cast<int64_t>(m) * K + step * 32 + 8 * kb);
+      return valid ? v : u32x4{0u, 0u, 0u, 0u};
     }
     return *reinterpret_cast<const u32x4*>(x + static_cast<int64_t>(m) * K + step * 32 + 8 * kb);
   }
@@ -130,27 +139,32 @@ struct StreamKernel {
   // The small loads (activations, scales) go first: the memory system returns
   // loads in order, so the first weight tile can be consumed while the later
   // ones are still on their way.
-  __device__ inline void load_unit(Unit& d, const u32x4* const (&tp)[TN], int u) const {
+  __device__ inline void load_unit(Unit& d, const u32x4* const (&tp)[TN], int u, bool tail = false) const {
     const int step0 = u * kU;
 #pragma unroll
     for (int a = 0; a < kNA; ++a)
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) d.av[a][mt] = load_a(mt, step0 + a * kS, true);
+      for (int mt = 0; mt < MT; ++mt) d.av[a][mt] = load_a(mt, step0 + a * kS, true, tail);
     if (GROUPED) {
       const int mine = MP == 8 ? (kb >> 1) : kb;
 #pragma unroll
       for (int p = 0; p < kNS; ++p) {
         const int step = MP == 16 ? step0 + 2 * p
                                   : step0 + (p / kPairs) * kS + mine * kRowsPerGroup + 2 * (p % kPairs);
+        const int sstep = tail ? (step < vsteps ? step : vsteps - 1) : step;
 #pragma unroll
-        for (int t = 0; t < TN; ++t) d.sraw[t][p] = load_scale_raw(step, t);
+        for (int t = 0; t < TN; ++t) d.sraw[t][p] = load_scale_raw(sstep, t);
       }
     }
     if (NU > 0) __builtin_amdgcn_sched_barrier(0);  // keep the compiler from moving them behind the weights
 #pragma unroll
     for (int t = 0; t < TN; ++t)
 #pragma unroll
-      for (int i = 0; i < kNT; ++i) d.wv[t][i] = __builtin_nontemporal_load(tp[t] + (step0 / kSPT + i) * 64);
+      for (int i = 0; i < kNT; ++i) {
+        int tile = step0 / kSPT + i;
+        if (tail) tile = tile < vsteps / kSPT ? tile : vsteps / kSPT - 1;
+        d.wv[t][i] = __builtin_nontemporal_load(tp[t] + tile * 64);
+      }
   }
 
   // mfma(A, constant B): the term that removes the dequantiser's offset.  It
@@ -216,7 +230,8 @@ struct StreamKernel {
     magic = Dequant<DT, BITS>::kMagic;
     asm volatile("" : "+v"(magic));  // keep the constant in a VGPR
     const int nsteps = K / 32;
-    const int nunits = nsteps / kU;
+    vsteps = BITS == 4 ? (K / 128) * 4 : nsteps;
+    const int nunits = (NU > 0 ? nsteps : vsteps) / kU;  // whole units
 #pragma unroll
     for (int t = 0; t < TN; ++t)
 #pragma unroll
@@ -244,11 +259,16 @@ struct StreamKernel {
       for (int i = 0; i < NU; ++i) compute_unit(d[i]);
     } else {
       const int u0 = nunits * wave / WK, u1 = nunits * (wave + 1) / WK;
-      if (u0 < u1) {
+      // the partial unit that ends K goes to wavefront 0 (the floor split
+      // gives it the fewest whole units), ahead of its walk
+      const bool tail = kPartial && wave == 0 && nunits * kU < vsteps;
+      if (u0 < u1 || tail) {
         Unit d0, d1;
         int u = u0;
-        load_unit(d0, tp, u);
-        while (true) {
+        if (tail) load_unit(d1, tp, nunits, true);
+        if (u0 < u1) load_unit(d0, tp, u);
+        if (tail) compute_unit(d1);
+        if (u0 < u1) while (true) {
           if (u + 1 < u1) load_unit(d1, tp, u + 1);
           compute_unit(d0);
           if (++u >= u1) break;
@@ -257,12 +277,11 @@ struct StreamKernel {
           if (++u >= u1) break;
         }
       }
-      if (wave == WK - 1) {
-        // k steps past the last whole unit, two at a time (64 k): 8 bytes of
-        // codes per lane (int4, including the half tile that ends a K that is
-        // 64 mod 128) or one whole tile (int8).  Every row group carries the
-        // same step, row group 0 is kept.
-        for (int step = nunits * kU; step < nsteps; step += 2) {
+      if (BITS == 4 && wave == 0) {
+        // the half tile that ends a K that is 64 mod 128: two k steps, 8 bytes
+        // of codes per lane.  Every row group carries the same step, row
+        // group 0 is kept.
+        for (int step = vsteps; step < nsteps; step += 2) {
           u32x4 a[2][MT];
           f32x4 cc[2][MT];
 #pragma unroll
@@ -274,17 +293,8 @@ struct StreamKernel {
             }
 #pragma unroll
           for (int t = 0; t < TN; ++t) {
-            uint32_t w[4];
-            if (BITS == 8) {
-              const u32x4 v = tp[t][(step / 2) * 64];
-              w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w;
-            } else {
-              const int tile = step / 4, nfull = K / 128;
-              const uint8_t* p = tile < nfull ? strip[t] + tile * 1024 + lane * 16 + (step % 4) * 4
-                                              : strip[t] + nfull * 1024 + lane * 8;
-              const u32x2 v = *reinterpret_cast<const u32x2*>(p);
-              w[0] = v.x; w[1] = v.y; w[2] = 0; w[3] = 0;
-            }
+            const u32x2 v = *reinterpret_cast<const u32x2*>(strip[t] + (K / 128) * 1024 + lane * 8);
+            const uint32_t w[4] = {v.x, v.y, 0, 0};
             const float sc = GROUPED ? to_f32<DT>(load_scale_raw(step, t)) : 1.0f;
 #pragma unroll
             for (int st = 0; st < 2; ++st) step_mfma(w + st * kDw, a[st], cc[st], 0, sc, t);
@@ -429,7 +439,7 @@ void launch_wk(const Args& a, int wk, int nu) {
   } else {
     // 16 wavefronts (1024 threads) leave 128 registers each: enough for the
     // double-buffered units of 2 to 8 rows, not for the others
-    if constexpr (MP >= 2 && MP <= 8) {
+    if constexpr ((MP >= 2 && MP <= 8) || (MP == 1 && BITS == 4)) {
       if (wk >= 16) { launch_one<DT, BITS, MP, MT, 16, 0>(a); return; }
     }
     if (wk >= 8) launch_one<DT, BITS, MP, MT, 8, 0>(a);
@@ -486,8 +496,11 @@ static void pick_split(int64_t M, int64_t K, int64_t N, int bits, int* wk, int* 
   // operands (more registers and LDS per wavefront) only one or two
   const int64_t budget = mp <= 2 ? 8192 : (mp <= 8 ? 4096 : 2048);
   int w = 1;
-  const int maxwalk = mp >= 2 && mp <= 8 ? 16 : 8;
-  while (w < maxwalk && strips * w * 2 <= budget && w * 4 <= nunits) w *= 2;
+  const int maxwalk = (mp >= 2 && mp <= 8) || (mp == 1 && bits == 4) ? 16 : 8;
+  // at least four units per wavefront, unless the strips leave CUs (256) with
+  // one workgroup at most: then only a wider workgroup puts more wavefronts on a SIMD
+  const int minu = strips <= 256 ? 1 : 4;
+  while (w < maxwalk && strips * w * 2 <= budget && w * minu <= nunits) w *= 2;
   *wk = w;
   *nu = 0;
 }
