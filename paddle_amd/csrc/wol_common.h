@@ -193,6 +193,8 @@ inline int stream_strips_per_workgroup(int64_t M, int64_t N, int bits) {
   const int64_t groups = N / kStripCols / 2;
   if (rows >= 4 * bits) return groups >= 256 ? 2 : 1;
   if (rows >= 2 * bits) return groups >= 384 ? 2 : 1;
+  // 8 rows of int8 (the kernels pair strips from 8 rows up): 19.0 against 21.7 us at N = 22016
+  if (rows >= 8 && rows >= bits) return groups >= 512 ? 2 : 1;
   return 1;
 }
 
