@@ -28,10 +28,13 @@ bool layout_ok(int layout) {
 // The streaming kernel takes M <= 64 (four 16-row MFMA tiles).  It streams
 // the weights best, but every 16-column strip re-reads its activations from
 // L2; the MFMA GEMM shares them through LDS at the price of a second launch
-// that adds the K runs.  Between 9 and 64 rows the cheaper of the two by a
-// two-term cost model (microseconds, fitted to measurements on MI355X) runs.
+// that adds the K runs.  Up to 16 rows the streaming kernel won every shape
+// measured (K and N from 4096 to 28672, both bit widths); from 17 to 64 rows
+// the cheaper of the two by a linear cost model runs (microseconds, least
+// squares over those measurements on MI355X; it picks the slower kernel in 1
+// of 96 cases, by 14 %).
 constexpr int64_t kStreamMaxM = 64;
-constexpr int64_t kStreamAlwaysM = 8;
+constexpr int64_t kStreamAlwaysM = 16;
 
 bool gemm_fast_path(int64_t K, int bits) {
   const int64_t tk = bits == 8 ? 64 : 128;
@@ -41,12 +44,17 @@ bool gemm_fast_path(int64_t K, int bits) {
 bool use_stream(int64_t M, int64_t K, int64_t N, int bits) {
   if (M > kStreamMaxM) return false;
   if (M <= kStreamAlwaysM || !gemm_fast_path(K, bits)) return true;
-  const double w = static_cast<double>(K) * N * bits / 8.0;           // weight bytes
-  const double rows = static_cast<double>((M + 15) / 16 * 16);
-  const double a = static_cast<double>(N / 16) * rows * K * 2.0 /     // activation bytes re-read
-                   wol::stream_strips_per_workgroup(M, N, bits);
-  const double t_stream = (w + a) / 8.8e6 + 4.5;  // everything through L2 at ~8.8 TB/s
-  const double t_gemm = w / 4.1e6 + 10.4;         // two launches, K runs of a few k tiles each
+  const double w = static_cast<double>(K) * N * bits / 8.0 * 1e-6;  // weight MB
+  // activation MB the strips re-read out of L2: the rows that exist, and the
+  // 16-row operands they are padded to (padding rows repeat the last row)
+  const double a = static_cast<double>(N / 16) * M * K * 2.0 * 1e-6;
+  const double a_pad = static_cast<double>(N / 16) * ((M + 15) / 16 * 16) * K * 2.0 * 1e-6;
+  const double t_stream = 3.0 + 0.0132 * w + 0.0829 * a + 0.0296 * a_pad;
+  // two launches; K runs of a few k tiles each; fp32 partial sums written and
+  // read back (M * N); MFMA work of the 32- or 64-row tile
+  const double tile_rows = bits == 4 && M <= 32 ? 32.0 : 64.0;
+  const double t_gemm = 10.1 + (bits == 8 ? 0.1535 : 0.108) * w + 15.6 * (M * N * 1e-6) +
+                        0.494 * (tile_rows * N * K * 1e-9);
   return t_stream <= t_gemm;
 }
 

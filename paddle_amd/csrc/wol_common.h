@@ -184,17 +184,18 @@ __device__ inline uint16_t cast_out(float f) {
 // Strips (16 columns) that share a workgroup of the streaming linear kernel.
 // Two halve the activation traffic out of L2 (N/16 * rows * K * 2 bytes, rows
 // = M rounded up to a power of two, at most 16 per operand) but also the
-// number of workgroups: worth it once that traffic is at least twice the
-// weight bytes (rows / bits >= 2) and enough workgroups remain.
+// number of workgroups: worth it once that traffic is at least the weight
+// bytes (rows >= bits) and enough workgroups remain (measured thresholds).
 inline int stream_strips_per_workgroup(int64_t M, int64_t N, int bits) {
   if (M > 16) return 1;  // several 16-row operands per strip already fill the registers
   int rows = 1;
   while (rows < 16 && rows < M) rows *= 2;
   const int64_t groups = N / kStripCols / 2;
-  if (rows >= 4 * bits) return groups >= 256 ? 2 : 1;
-  if (rows >= 2 * bits) return groups >= 384 ? 2 : 1;
-  // 8 rows of int8 (the kernels pair strips from 8 rows up): 19.0 against 21.7 us at N = 22016
-  if (rows >= 8 && rows >= bits) return groups >= 512 ? 2 : 1;
+  if (rows >= 2 * bits) return groups >= 256 ? 2 : 1;  // a workgroup for every CU must remain
+  // activation traffic equal to the weight bytes (8 rows of int8; the kernels
+  // pair strips from 8 rows up): 25.7 against 26.9 us at 448 pairs, 13.4
+  // against 12.8 us at 384
+  if (rows >= 8 && rows >= bits) return groups >= 448 ? 2 : 1;
   return 1;
 }
 

@@ -67,10 +67,12 @@ def test_workspace_queries(lib):
     assert L.wol_linear_workspace(2048, 4096, 12288, 8, -1) == 0     # one workgroup per tile covers all of K
     assert L.wol_linear_workspace(1024, 4096, 4096, 8, 64) == 2 * 1024 * 4096 * 4  # 128 tiles: two K runs
     # small M on the GEMM: whole fp32 [M, N] partial buffers, at most 16 of them
-    for M, K, N, bits, g in [(64, 8192, 28672, 4, 128), (32, 4096, 11008, 4, -1), (16, 8192, 28672, 4, 128)]:
+    for M, K, N, bits, g in [(64, 8192, 28672, 4, 128), (32, 4096, 11008, 4, -1), (24, 8192, 28672, 4, 128)]:
         need = L.wol_linear_workspace(M, K, N, bits, g)
         assert need == L.wol_linear_workspace_for(M, K, N, bits, g, lib.KERNEL_GEMM)
         assert need % (M * N * 4) == 0 and 2 <= need // (M * N * 4) <= 16, (M, K, N, need)
+    assert L.wol_linear_workspace(16, 8192, 28672, 4, 128) == 0  # up to 16 rows: always the streaming kernel
+    assert L.wol_linear_workspace_for(16, 8192, 28672, 4, 128, lib.KERNEL_GEMM) > 0
     assert L.wol_linear_workspace_for(16, 4096, 11008, 4, 128, lib.KERNEL_STREAM) == 0
     assert L.wol_linear_workspace_for(16, 4160, 11008, 4, 128, lib.KERNEL_GEMM) == 0  # K not a multiple of the k tile
 
