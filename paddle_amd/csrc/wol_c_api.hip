@@ -31,8 +31,8 @@ bool layout_ok(int layout) {
 // that adds the K runs.  Up to 16 rows the streaming kernel won every shape
 // measured (K and N from 4096 to 28672, both bit widths); from 17 to 64 rows
 // the cheaper of the two by a linear cost model runs (microseconds, least
-// squares over those measurements on MI355X; it picks the slower kernel in 1
-// of 96 cases, by 14 %).
+// squares over those measurements on MI355X; it picks the slower kernel in 2
+// of 96 cases, by 16 %).
 constexpr int64_t kStreamMaxM = 64;
 constexpr int64_t kStreamAlwaysM = 16;
 
@@ -53,8 +53,8 @@ bool use_stream(int64_t M, int64_t K, int64_t N, int bits) {
   // two launches; K runs of a few k tiles each; fp32 partial sums written and
   // read back (M * N); MFMA work of the 32- or 64-row tile
   const double tile_rows = bits == 4 && M <= 32 ? 32.0 : 64.0;
-  const double t_gemm = 10.1 + (bits == 8 ? 0.1535 : 0.108) * w + 15.6 * (M * N * 1e-6) +
-                        0.494 * (tile_rows * N * K * 1e-9);
+  const double t_gemm = 11.2 + (bits == 8 ? 0.035 : 0.0014) * w + 7.04 * (M * N * 1e-6) +
+                        2.184 * (tile_rows * N * K * 1e-9);
   return t_stream <= t_gemm;
 }
 

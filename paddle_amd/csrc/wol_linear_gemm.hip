@@ -928,9 +928,10 @@ constexpr int kSkinnyMaxM = 64;
 // Split of K for the small-M configurations: the number of runs that
 // minimises rounds-of-workgroups x (k tiles per run + fixed cost), at most 16
 // runs of at least 4 k tiles, and no more than the scratch buffer allows.
-inline int plan_split(int M, int K, int N, int bits, size_t lds, size_t ws_bytes) {
+// cols: columns per workgroup (256 or 512).
+inline int plan_split(int M, int K, int N, int bits, int cols, size_t lds, size_t ws_bytes) {
   const int tk = bits == 8 ? 64 : 128, tiles = K / tk;
-  const int nbx = (N + 255) / 256;
+  const int nbx = (N + cols - 1) / cols;
   const int per_cu = static_cast<int>((160 * 1024) / lds) > 0 ? static_cast<int>((160 * 1024) / lds) : 1;
   const int slots = num_cus() * per_cu;
   const size_t per_run = static_cast<size_t>(M) * N * sizeof(float);
@@ -946,6 +947,21 @@ inline int plan_split(int M, int K, int N, int bits, size_t lds, size_t ws_bytes
     if (cost < best_cost) { best_cost = cost; best = ns; }
   }
   return best;
+}
+
+// The small-M configurations take 256 columns per workgroup, or 512 (two
+// 32-column blocks per wavefront): half the activation bytes out of L2 and
+// half the A-fragment reads out of LDS per MFMA (each workgroup fetches its
+// rows of x for its K run, which at 64 rows of int4 equals its weight
+// bytes).  Worth it while K runs can still make at least one workgroup per
+// CU; measured -13..-21 % at N >= 12288, +5..+20 % at N <= 4096 or K = 4096
+// int4 at N = 11008.  int4 with group size 64 and 64-row tiles does not fit
+// the registers at 512 columns.
+inline bool skinny_wide(int M, int K, int N, int bits, int group) {
+  if (bits == 4 && group == 64 && M > 32) return false;
+  const int tk = bits == 8 ? 64 : 128, tiles = K / tk;
+  const int max_runs = tiles / 4 < 16 ? (tiles / 4 < 1 ? 1 : tiles / 4) : 16;
+  return ((N + 511) / 512) * max_runs >= num_cus();
 }
 
 // K runs for the half-size configurations when their tiles leave CUs idle: as
@@ -966,18 +982,34 @@ inline int plan_split_large(int M, int K, int N, int bits, int group, size_t ws_
 }
 
 template <int BITS>
-size_t skinny_lds(int M) {  // with group scales (the larger footprint)
-  if (BITS == 4 && M <= 32) return dma_lds_bytes<4, 64, 1, 8, 1, 1, 2>();
-  return dma_lds_bytes<BITS, 64, 1, 8, 2, 1, 2>();
+size_t skinny_lds(int M, bool wide) {  // with group scales (the larger footprint)
+  if (BITS == 4 && M <= 32)
+    return wide ? dma_lds_bytes<4, 64, 1, 8, 1, 2, 2>() : dma_lds_bytes<4, 64, 1, 8, 1, 1, 2>();
+  return wide ? dma_lds_bytes<BITS, 64, 1, 8, 2, 2, 2>() : dma_lds_bytes<BITS, 64, 1, 8, 2, 1, 2>();
+}
+
+// K runs of the small-M configurations for a problem
+inline int plan_skinny(int M, int K, int N, int bits, int group, size_t ws_bytes, bool* wide) {
+  *wide = skinny_wide(M, K, N, bits, group);
+  const size_t lds = bits == 8 ? skinny_lds<8>(M, *wide) : skinny_lds<4>(M, *wide);
+  return plan_split(M, K, N, bits, *wide ? 512 : 256, lds, ws_bytes);
 }
 
 template <int DT, int BITS, int G>
 void launch_fast(const Args& a) {
   const int nstrips = a.N / kStripCols;
   if (a.M <= kSkinnyMaxM) {
-    const int ns = plan_split(a.M, a.K, a.N, BITS, skinny_lds<BITS>(a.M), a.ws != nullptr ? a.ws_bytes : 0);
+    bool wide = false;
+    const int ns = plan_skinny(a.M, a.K, a.N, BITS, G, a.ws != nullptr ? a.ws_bytes : 0, &wide);
     if constexpr (BITS == 4) {
-      if (a.M <= 32) { launch_dma<DT, BITS, G, true, 1, 8, 1, 1, 2>(a, 0, nstrips, ns); return; }
+      if (a.M <= 32) {
+        if (wide) launch_dma<DT, BITS, G, true, 1, 8, 1, 2, 2>(a, 0, nstrips, ns);
+        else launch_dma<DT, BITS, G, true, 1, 8, 1, 1, 2>(a, 0, nstrips, ns);
+        return;
+      }
+    }
+    if constexpr (!(BITS == 4 && G == 64)) {
+      if (wide) { launch_dma<DT, BITS, G, false, 1, 8, 2, 2, 2>(a, 0, nstrips, ns); return; }
     }
     launch_dma<DT, BITS, G, false, 1, 8, 2, 1, 2>(a, 0, nstrips, ns);
     return;
@@ -1040,8 +1072,9 @@ size_t linear_gemm_workspace(int64_t M, int64_t K, int64_t N, int bits, int grou
                                     group_size > 0 ? group_size : 0, SIZE_MAX);
     return ns > 1 ? static_cast<size_t>(ns) * M * N * sizeof(float) : 0;
   }
-  const size_t lds = bits == 8 ? skinny_lds<8>(static_cast<int>(M)) : skinny_lds<4>(static_cast<int>(M));
-  const int ns = plan_split(static_cast<int>(M), static_cast<int>(K), static_cast<int>(N), bits, lds, SIZE_MAX);
+  bool wide = false;
+  const int ns = plan_skinny(static_cast<int>(M), static_cast<int>(K), static_cast<int>(N), bits,
+                             group_size > 0 ? group_size : 0, SIZE_MAX, &wide);
   return ns > 1 ? static_cast<size_t>(ns) * M * N * sizeof(float) : 0;
 }
 
