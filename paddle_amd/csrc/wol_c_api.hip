@@ -41,7 +41,8 @@ bool gemm_fast_path(int64_t K, int bits) {
   return K % tk == 0 && K / tk >= 2;
 }
 
-bool use_stream(int64_t M, int64_t K, int64_t N, int bits) {
+// have_ws: the caller's scratch buffer holds at least two K runs of partial sums
+bool use_stream(int64_t M, int64_t K, int64_t N, int bits, bool have_ws) {
   if (M > kStreamMaxM) return false;
   if (M <= kStreamAlwaysM || !gemm_fast_path(K, bits)) return true;
   const double w = static_cast<double>(K) * N * bits / 8.0 * 1e-6;  // weight MB
@@ -53,16 +54,23 @@ bool use_stream(int64_t M, int64_t K, int64_t N, int bits) {
   // two launches; K runs of a few k tiles each; fp32 partial sums written and
   // read back (M * N); MFMA work of the 32- or 64-row tile
   const double tile_rows = bits == 4 && M <= 32 ? 32.0 : 64.0;
+  if (!have_ws) {
+    // without scratch every workgroup walks all of K: measured 0.75 us per k
+    // tile (1.17 us for 64 rows of int4), one workgroup per 256 columns
+    const double tiles = static_cast<double>(K / (bits == 8 ? 64 : 128));
+    const double rounds = static_cast<double>((N / 256 + 511) / 512);  // two workgroups fit a CU
+    return t_stream <= 3.0 + tiles * (bits == 4 && M > 32 ? 1.17 : 0.75) * rounds;
+  }
   const double t_gemm = 11.2 + (bits == 8 ? 0.035 : 0.0014) * w + 7.04 * (M * N * 1e-6) +
                         2.184 * (tile_rows * N * K * 1e-9);
   return t_stream <= t_gemm;
 }
 
 // kernel: a wol_kernel; AUTO resolves by M and the cost model
-bool resolve_stream(int kernel, int64_t M, int64_t K, int64_t N, int bits) {
+bool resolve_stream(int kernel, int64_t M, int64_t K, int64_t N, int bits, bool have_ws = true) {
   if (kernel == WOL_KERNEL_STREAM) return true;
   if (kernel == WOL_KERNEL_GEMM) return false;
-  return use_stream(M, K, N, bits);
+  return use_stream(M, K, N, bits, have_ws);
 }
 
 int linear_impl(const void* x, const void* codes, const void* bias, const void* scale, int dtype,
@@ -79,10 +87,11 @@ int linear_impl(const void* x, const void* codes, const void* bias, const void* 
     return WOL_ERR_NULL_POINTER;
   if (!aligned16(x) || !aligned16(codes) || !aligned16(scale)) return WOL_ERR_ALIGNMENT;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (resolve_stream(kernel, M, K, N, bits))
+  if (workspace == nullptr || !aligned16(workspace)) workspace_bytes = 0;  // optional: only speeds up
+  const bool have_ws = workspace_bytes / sizeof(float) / 2 >= static_cast<size_t>(M) * static_cast<size_t>(N);
+  if (resolve_stream(kernel, M, K, N, bits, have_ws))
     return wol::launch_linear_stream(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out,
                                      out_f32, s);
-  if (workspace == nullptr || !aligned16(workspace)) workspace_bytes = 0;  // optional: only speeds up
   return wol::launch_linear_gemm(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out,
                                  out_f32, workspace, workspace_bytes, s);
 }

@@ -13,6 +13,8 @@
 // The epilogue passes each 16-row slab through LDS so that rows leave as
 // 16-byte stores.  Workgroups are numbered so that each XCD (one L2 each)
 // works on a compact block of neighbouring tiles.
+#include <atomic>
+
 #include "wol_common.h"
 #include "wol_dequant.h"
 
@@ -798,6 +800,17 @@ struct Args {
   hipStream_t stream;
 };
 
+// Raises a kernel's dynamic LDS limit once per device (the attribute belongs to
+// the device's copy of the function); safe to call from several threads.
+inline void allow_lds(const void* kern, size_t lds, std::atomic<uint32_t>& done) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+  const uint32_t bit = 1u << (dev & 31);
+  if (done.load(std::memory_order_acquire) & bit) return;
+  (void)hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+  done.fetch_or(bit, std::memory_order_release);
+}
+
 inline int num_cus() {
   static const int cus = [] {
     int dev = 0, n = 0;
@@ -815,12 +828,8 @@ void launch_one(const Args& a) {
   const int nbx = (a.N + BN - 1) / BN, nby = (a.M + BM - 1) / BM;
   const size_t lds = 2 * static_cast<size_t>(BM) * (TK + 8) * sizeof(uint16_t);
   auto kern = gemm_kernel<DT, BITS, GROUPED, WM, WN, TM, TN>;
-  static bool configured = false;  // per instantiation; the attribute is idempotent
-  if (!configured) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-    configured = true;
-  }
+  static std::atomic<uint32_t> configured{0};  // per instantiation
+  allow_lds(reinterpret_cast<const void*>(kern), lds, configured);
   kern<<<dim3(static_cast<unsigned>(nbx * nby)), dim3(64 * WM * WN), lds, a.stream>>>(
       static_cast<const uint16_t*>(a.x), static_cast<const uint8_t*>(a.codes),
       static_cast<const uint16_t*>(a.bias), static_cast<const uint16_t*>(a.scale), a.out, a.M, a.K,
@@ -857,12 +866,8 @@ void launch_dma(const Args& a, int strip_lo, int strip_hi, int nsplit) {
   if (strip_hi <= strip_lo) return;
   constexpr size_t lds = dma_lds_bytes<BITS, G, WM, WN, TM, TN, STAGES>();
   auto kern = gemm_dma_kernel<DT, BITS, G, OFFS, WM, WN, TM, TN, STAGES>;
-  static bool configured = false;
-  if (!configured) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-    configured = true;
-  }
+  static std::atomic<uint32_t> configured{0};  // per instantiation
+  allow_lds(reinterpret_cast<const void*>(kern), lds, configured);
   if (nsplit > 1 && (a.ws == nullptr ||
                      a.ws_bytes < static_cast<size_t>(nsplit) * a.M * a.N * sizeof(float)))
     nsplit = 1;  // never write past the scratch buffer
@@ -957,10 +962,12 @@ inline int plan_split(int M, int K, int N, int bits, int cols, size_t lds, size_
 // CU; measured -13..-21 % at N >= 12288, +5..+20 % at N <= 4096 or K = 4096
 // int4 at N = 11008.  int4 with group size 64 and 64-row tiles does not fit
 // the registers at 512 columns.
-inline bool skinny_wide(int M, int K, int N, int bits, int group) {
+inline bool skinny_wide(int M, int K, int N, int bits, int group, size_t ws_bytes) {
   if (bits == 4 && group == 64 && M > 32) return false;
   const int tk = bits == 8 ? 64 : 128, tiles = K / tk;
-  const int max_runs = tiles / 4 < 16 ? (tiles / 4 < 1 ? 1 : tiles / 4) : 16;
+  int max_runs = tiles / 4 < 16 ? (tiles / 4 < 1 ? 1 : tiles / 4) : 16;
+  const size_t fit = ws_bytes / sizeof(float) / (static_cast<size_t>(M) * N);  // runs the scratch holds
+  if (fit < static_cast<size_t>(max_runs)) max_runs = fit < 1 ? 1 : static_cast<int>(fit);
   return ((N + 511) / 512) * max_runs >= num_cus();
 }
 
@@ -990,7 +997,7 @@ size_t skinny_lds(int M, bool wide) {  // with group scales (the larger footprin
 
 // K runs of the small-M configurations for a problem
 inline int plan_skinny(int M, int K, int N, int bits, int group, size_t ws_bytes, bool* wide) {
-  *wide = skinny_wide(M, K, N, bits, group);
+  *wide = skinny_wide(M, K, N, bits, group, ws_bytes);
   const size_t lds = bits == 8 ? skinny_lds<8>(M, *wide) : skinny_lds<4>(M, *wide);
   return plan_split(M, K, N, bits, *wide ? 512 : 256, lds, ws_bytes);
 }
