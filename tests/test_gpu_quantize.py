@@ -100,6 +100,53 @@ def test_quantize_nan_and_inf_inputs(G, oracle, bits):
         assert np.array_equal(gc.view(np.int8).reshape(oc.shape), oc)
 
 
+def _near_tie_weight(dt, bits, K, N, seed):
+    """Columns whose quotients w / scale sit on and right next to the rounding
+    boundaries k + 0.5 (every k up to the bound, both signs, and the neighbours
+    one unit in the last place of T either side), under scales that span the
+    exponent range of T: where a quantiser that multiplies by a reciprocal
+    instead of dividing would go wrong first."""
+    rng = np.random.default_rng(seed)
+    bound = 127 if bits == 8 else 7
+    lo_e, hi_e = (-12, 14) if dt == H.F16 else (-110, 110)
+    wb = np.zeros((K, N), np.uint16)
+    for c in range(N):
+        amax = np.float32(rng.uniform(1.0, 2.0) * 2.0 ** int(rng.integers(lo_e, hi_e)))
+        a_bits = H.f32_to_bits(np.array([amax], np.float32), dt)[0]
+        a_val = H.bits_to_f32(np.array([a_bits], np.uint16), dt)[0]
+        s_val = H.bits_to_f32(H.f32_to_bits(np.array([a_val / np.float32(bound)], np.float32), dt), dt)[0]
+        ks = rng.integers(0, bound, K).astype(np.float32) + np.float32(0.5)
+        sign = np.where(rng.integers(0, 2, K) == 0, np.float32(1), np.float32(-1))
+        col = H.f32_to_bits((ks * s_val * sign).astype(np.float32), dt).astype(np.int32)
+        col += rng.integers(-1, 2, K)  # the value itself or a neighbour in T
+        col = col.astype(np.uint16)
+        col[int(rng.integers(K))] = a_bits  # the column maximum that fixes the scale
+        if c % 7 == 0:  # the maximum in every 64-row group, so group-wise scales match too
+            col[::64] = a_bits
+        wb[:, c] = col
+    return wb
+
+
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+@pytest.mark.parametrize("bits", [8, 4])
+def test_quantize_near_rounding_boundaries(G, oracle, dt, bits):
+    K, N = 512, 128
+    for seed, g in ((1, -1), (2, 64), (3, 128), (4, -1)):
+        print("case", dt, bits, g, seed, flush=True)
+        wb = _near_tie_weight(dt, bits, K, N, seed)
+        oc, osc = oracle.weight_quantize(wb, dt, bits, g)
+        gc, gs = G.quantize(wb, dt, bits, g, layout=0)
+        assert np.array_equal(gs, osc)
+        got = gc.view(np.int8).reshape(oc.shape)
+        assert np.array_equal(got, oc), np.argwhere(got != oc)[:5]
+    # the construction does what it says: hundreds of quotients are exact ties
+    # (the rest lie within a few units in the last place of T of one)
+    w32 = H.bits_to_f32(wb, dt)
+    s32 = H.bits_to_f32(osc, dt)
+    frac = np.abs(np.abs(w32 / s32[None, :]) % 1.0 - 0.5)
+    assert (frac == 0).sum() > 300, (frac == 0).sum()
+
+
 @pytest.mark.parametrize("bits", [8, 4])
 def test_repack_round_trips(G, bits):
     rng = np.random.default_rng(bits)
