@@ -192,6 +192,17 @@ def main():
     y = decode_step(0)
     torch.cuda.synchronize()
 
+    # the floor of this launch shape on this machine: the same weight copies read
+    # by a kernel of the decode kernel's shape that computes nothing
+    from paddle_amd import _lib
+    floor_out = torch.empty(c["N"] // 16 * 8, dtype=torch.int32, device=dev)
+
+    def floor_step(i):
+        _lib.check(_lib.lib.wol_read_floor(copies[i % ncopies].data_ptr(), c["K"], c["N"], c["bits"],
+                                           floor_out.data_ptr(), torch.cuda.current_stream().cuda_stream))
+
+    floor_s = timer(torch, floor_step, args.steps, args.warmup) / args.steps
+
     # ---------------- prefill ----------------
     p = PREFILL
     pw_bits = H.make_weight(p["K"], p["N"], dt, seed=1236)
@@ -247,6 +258,13 @@ def main():
             "kernel": "wol::stream_kernel<1, 4, 1, 1, 8, 1, 1, true>",
             "algorithmic_bytes_per_launch": wbytes,
             "total_bytes_per_launch": total_bytes,
+            "read_floor": {
+                "what": "wol_read_floor: the same weight copies read by a kernel of the same launch shape "
+                        "that computes nothing (no scales, activations, MFMAs or output)",
+                "ms_per_step": round(floor_s * 1e3, 6),
+                "GB/s": round(wbytes / floor_s / 1e9, 1),
+                "decode_over_floor": round(dec_s / floor_s, 3),
+            },
         },
         "prefill": {
             "value": round(pre_tf, 2),

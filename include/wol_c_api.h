@@ -220,6 +220,18 @@ int wol_apply_per_channel_scale(const void* x, const void* scales, int dtype,
                                 int64_t rows, int64_t cols, void* out,
                                 void* stream);
 
+/*
+ * Measurement aid with no counterpart in the reference: reads a GFX950-layout
+ * weight with the launch shape of the one-row decode kernel (one workgroup of
+ * eight wavefronts per 16-column strip, 16-byte non-temporal loads, all of a
+ * wavefront's loads requested at once) and computes nothing.  Its duration is
+ * the floor a decode call of that shape has on the machine at hand; bench.py
+ * reports it beside the decode time.  out receives N/16*8 uint32 (an XOR of
+ * what each wavefront read).  K*bits/8*16 must be a multiple of 8 KiB.
+ */
+int wol_read_floor(const void* codes, int64_t K, int64_t N, int bits, void* out,
+                   void* stream);
+
 #ifdef __cplusplus
 }
 #endif

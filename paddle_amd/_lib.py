@@ -29,6 +29,7 @@ SYMBOLS = (
     "wol_repack",
     "wol_code_offset",
     "wol_apply_per_channel_scale",
+    "wol_read_floor",
 )
 
 
@@ -72,6 +73,8 @@ def _load():
     lib.wol_code_offset.restype = i64
     lib.wol_apply_per_channel_scale.argtypes = [vp, vp, ci, i64, i64, vp, vp]
     lib.wol_apply_per_channel_scale.restype = ci
+    lib.wol_read_floor.argtypes = [vp, i64, i64, ci, vp, vp]
+    lib.wol_read_floor.restype = ci
     return lib
 
 

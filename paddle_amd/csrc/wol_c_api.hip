@@ -231,4 +231,13 @@ int wol_apply_per_channel_scale(const void* x, const void* scales, int dtype, in
   return wol::launch_prescale(x, scales, dtype, rows, cols, out, static_cast<hipStream_t>(stream));
 }
 
+int wol_read_floor(const void* codes, int64_t K, int64_t N, int bits, void* out, void* stream) {
+  const int rc = check_problem(WOL_DTYPE_F16, K, N, bits, -1);
+  if (rc != WOL_OK) return rc;
+  if (K * bits % (8 * 1024 * 8 / 16) != 0) return WOL_ERR_BAD_SHAPE;  // whole 1 KiB pieces per wavefront
+  if (codes == nullptr || out == nullptr) return WOL_ERR_NULL_POINTER;
+  if (!aligned16(codes)) return WOL_ERR_ALIGNMENT;
+  return wol::launch_read_floor(codes, K, N, bits, out, static_cast<hipStream_t>(stream));
+}
+
 }  // extern "C"

@@ -214,6 +214,8 @@ int launch_linear_gemm(const void* x, const void* codes, const void* bias, const
                        int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
                        void* out, bool out_f32, void* workspace, size_t workspace_bytes,
                        hipStream_t stream);
+int launch_read_floor(const void* codes, int64_t K, int64_t N, int bits, void* out,
+                      hipStream_t stream);
 int launch_prescale(const void* x, const void* scales, int dtype, int64_t rows, int64_t cols,
                     void* out, hipStream_t stream);
 // Scratch bytes with which launch_linear_gemm splits K across workgroups (0: none needed).

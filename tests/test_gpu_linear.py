@@ -392,3 +392,23 @@ def test_empty_batch_and_leading_dims(device):
     out = Q.weight_only_linear(x, codes, weight_scale=scale)
     flat = Q.weight_only_linear(x.reshape(-1, 128), codes, weight_scale=scale)
     assert list(out.shape) == [2, 3, 5, 64] and torch.equal(out.reshape(-1, 64), flat)
+
+
+def test_read_floor_reads_every_byte_once(device):
+    # the measurement aid behind bench.py's read_floor: each wavefront XORs the
+    # dwords of its eighth of a strip
+    import torch
+    from paddle_amd import _lib
+
+    K, N, bits = 2048, 96, 8
+    rng = np.random.default_rng(5)
+    codes = rng.integers(0, 256, K * N, dtype=np.uint8)
+    d = torch.from_numpy(codes).to(device)
+    out = torch.zeros(N // 16 * 8, dtype=torch.int32, device=device)
+    _lib.check(_lib.lib.wol_read_floor(d.data_ptr(), K, N, bits, out.data_ptr(), None))
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().view(np.uint32)
+    # lane 0 of a wavefront holds the XOR over the lane-0 pieces only: 4 dwords of every 64 x 4
+    per_wave = codes.view(np.uint32).reshape(N // 16 * 8, -1, 64, 4)[:, :, 0, :]
+    want = np.bitwise_xor.reduce(per_wave.reshape(per_wave.shape[0], -1), axis=1)
+    assert np.array_equal(got, want)

@@ -209,3 +209,11 @@ def test_python_api_argument_checks():
     assert Q.weight_quantize.__defaults__ == ("weight_only_int8", None, -1)
     assert Q.weight_dequantize.__defaults__ == ("weight_only_int8", "float16", -1)
     assert Q.weight_only_linear.__defaults__ == (None, None, "int8", None, -1)
+
+
+def test_read_floor_argument_errors(lib):
+    f = lib.lib.wol_read_floor
+    assert f(None, 4096, 11008, 4, None, None) == 1  # null pointers
+    assert f(None, 4096, 11008, 5, None, None) == 3  # bits
+    assert f(None, 4096, 11000, 4, None, None) == 5  # N % 16
+    assert f(None, 64, 16, 4, None, None) == 5  # a strip smaller than one piece per wavefront
