@@ -412,3 +412,17 @@ def test_read_floor_reads_every_byte_once(device):
     per_wave = codes.view(np.uint32).reshape(N // 16 * 8, -1, 64, 4)[:, :, 0, :]
     want = np.bitwise_xor.reduce(per_wave.reshape(per_wave.shape[0], -1), axis=1)
     assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+def test_stream_kernel_every_k_tail(G, oracle, bits):
+    # every K from 64 to 2560 in steps of 64 at the row counts whose units span
+    # several weight tiles (1, 2 and 4 rows): whole units, a partial unit, the
+    # int4 half tile and their combinations, with one wavefront and with many
+    # (N = 64 gives 4 strips, so K decides the wavefront count)
+    N = 64
+    for K in range(64, 2561, 64):
+        for M, g in ((1, -1), (2, 64), (4, 128 if K % 128 == 0 else 64)):
+            print("case", bits, K, M, g, flush=True)
+            check(G, oracle, H.BF16 if (K // 64) % 2 else H.F16, bits, g, M, K, N, bias=(K // 64) % 3 == 0,
+                  seed=K + M, kernel=KERNEL_STREAM)
