@@ -373,7 +373,8 @@ struct DmaParams {
   const uint8_t* codes;
   const uint16_t* bias;
   const uint16_t* scale;
-  void* out;                    // T or fp32 [M, N]; with nsplit > 1 fp32 partial sums [nsplit][M][N]
+  void* out;                    // T or fp32 [M, N]; with nsplit > 1 fp32 partial sums
+                                // [nsplit][M][columns of the launch]
   int M, K, N;
   int out_f32;
   int strip_lo, strip_hi;       // the launch covers the 16-column strips [strip_lo, strip_hi)
@@ -714,8 +715,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   }
   if (p.out_f32 || p.nsplit > 1) {
     // fp32 results (verification mode) or partial sums of this run of k tiles: plain stores
-    float* outf = static_cast<float*>(p.out) +
-                  (p.nsplit > 1 ? static_cast<int64_t>(split) * M * N : 0);
+    // partial sums are kept compact: row length = the columns of this launch
+    const int64_t ld = p.nsplit > 1 ? static_cast<int64_t>(p.strip_hi - p.strip_lo) * kStripCols : N;
+    const int ncol0 = p.nsplit > 1 ? p.strip_lo * kStripCols : 0;
+    float* outf = static_cast<float*>(p.out) + (p.nsplit > 1 ? static_cast<int64_t>(split) * M * ld : 0);
 #pragma unroll
     for (int a = 0; a < TM; ++a)
 #pragma unroll
@@ -724,7 +727,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int m = m0 + (wm * TM + a) * 32 + 8 * (r / 4) + 4 * b + r % 4;
-          if (m < M && n < n_hi) outf[static_cast<int64_t>(m) * N + n] = tot[a][c][r] * sc[c] + bv[c];
+          if (m < M && n < n_hi) outf[static_cast<int64_t>(m) * ld + (n - ncol0)] = tot[a][c][r] * sc[c] + bv[c];
         }
       }
     return;
@@ -756,13 +759,15 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
 #endif
 }
 
-// out[m, n] = T( sum over the runs of part[run][m][n] + bias[n] ), four columns per thread
+// out[m, col0 + c] = T( sum over the runs of part[run][m][c] + bias[col0 + c] ) for the ncols
+// columns from col0 on; four columns per thread; total = M * ncols
 template <int DT>
 __global__ __launch_bounds__(256) void reduce_partials_kernel(
     const float* __restrict__ part, int nsplit, const uint16_t* __restrict__ bias,
-    void* __restrict__ out, int out_f32, int64_t total, int N) {
+    void* __restrict__ out, int out_f32, int64_t total, int N, int col0, int ncols) {
   const int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
   if (i >= total) return;
+  const int64_t o = i / ncols * N + col0 + i % ncols;  // position in out
   f32x4 s = {0.f, 0.f, 0.f, 0.f};
   for (int r0 = 0; r0 < nsplit; r0 += 4) {  // four loads in flight, added in run order
     f32x4 v[4];
@@ -779,17 +784,17 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(
       }
   }
   if (bias != nullptr) {
-    const int n = static_cast<int>(i % N);
+    const int n = col0 + static_cast<int>(i % ncols);
 #pragma unroll
     for (int e = 0; e < 4; ++e) s[e] += to_f32<DT>(bias[n + e]);
   }
   if (out_f32) {
-    *reinterpret_cast<f32x4*>(static_cast<float*>(out) + i) = s;
+    *reinterpret_cast<f32x4*>(static_cast<float*>(out) + o) = s;
   } else {
     u32x2 v;
     v.x = cast_out<DT>(s[0]) | (static_cast<uint32_t>(cast_out<DT>(s[1])) << 16);
     v.y = cast_out<DT>(s[2]) | (static_cast<uint32_t>(cast_out<DT>(s[3])) << 16);
-    *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(out) + i) = v;
+    *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(out) + o) = v;
   }
 }
 
@@ -859,7 +864,7 @@ constexpr size_t dma_lds_bytes() {
 }
 
 // Launches the fast kernel on the columns of strips [strip_lo, strip_hi), K
-// cut into nsplit runs (nsplit > 1 needs a.ws and covers every column).
+// cut into nsplit runs (nsplit > 1 needs a.ws: nsplit x M x columns floats).
 template <int DT, int BITS, int G, bool OFFS, int WM, int WN, int TM, int TN, int STAGES = 3>
 void launch_dma(const Args& a, int strip_lo, int strip_hi, int nsplit) {
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32, TK = BITS == 8 ? 64 : 128;
@@ -868,8 +873,9 @@ void launch_dma(const Args& a, int strip_lo, int strip_hi, int nsplit) {
   auto kern = gemm_dma_kernel<DT, BITS, G, OFFS, WM, WN, TM, TN, STAGES>;
   static std::atomic<uint32_t> configured{0};  // per instantiation
   allow_lds(reinterpret_cast<const void*>(kern), lds, configured);
+  const int ncols = (strip_hi - strip_lo) * kStripCols;
   if (nsplit > 1 && (a.ws == nullptr ||
-                     a.ws_bytes < static_cast<size_t>(nsplit) * a.M * a.N * sizeof(float)))
+                     a.ws_bytes < static_cast<size_t>(nsplit) * a.M * ncols * sizeof(float)))
     nsplit = 1;  // never write past the scratch buffer
   DmaParams p;
   p.x = static_cast<const uint16_t*>(a.x);
@@ -888,9 +894,10 @@ void launch_dma(const Args& a, int strip_lo, int strip_hi, int nsplit) {
   p.xcd_rows = plan_xcd_rows(p.nbx, p.nby, BM * 2, BN * BITS / 8);
   kern<<<dim3(static_cast<unsigned>(p.nbx * p.nby * p.nsplit)), dim3(64 * WM * WN), lds, a.stream>>>(p);
   if (nsplit > 1) {
-    const int64_t total = static_cast<int64_t>(a.M) * a.N;
+    const int64_t total = static_cast<int64_t>(a.M) * ncols;
     reduce_partials_kernel<DT><<<dim3(static_cast<unsigned>((total / 4 + 255) / 256)), dim3(256), 0, a.stream>>>(
-        static_cast<const float*>(a.ws), p.nsplit, p.bias, a.out, a.out_f32, total, a.N);
+        static_cast<const float*>(a.ws), p.nsplit, p.bias, a.out, a.out_f32, total, a.N,
+        strip_lo * kStripCols, ncols);
   }
 }
 
@@ -971,21 +978,48 @@ inline bool skinny_wide(int M, int K, int N, int bits, int group, size_t ws_byte
   return ((N + 511) / 512) * max_runs >= num_cus();
 }
 
-// K runs for the half-size configurations when their tiles leave CUs idle: as
-// many runs as fit the idle CUs (2..4), each at least 8 k tiles long, and
-// only if the scratch buffer holds them.  The extra traffic (ns x M x N fp32,
-// written and read once) is worth it below half occupancy.
-inline int plan_split_large(int M, int K, int N, int bits, int group, size_t ws_bytes) {
-  if (bits == 8 && group == 0 && plan_big_columns(M, N) > 0) return 1;  // 256-row tiles are in play
-  const int tk = bits == 8 ? 64 : 128, tiles = K / tk;
-  // tile of the configuration launch_fast picks: 256 x 128 or 128 x 256 (int8), 128 x 128 (int4, group 64)
-  const int bm = bits == 8 && tall_half_tile(M) ? 256 : 128;
-  const int bn = bm == 256 || (bits == 4 && group == 64) ? 128 : 256;
-  const int blocks = ((N + bn - 1) / bn) * ((M + bm - 1) / bm);
-  int ns = num_cus() / blocks;
+// Tile of the configuration launch_fast gives the columns that do not get
+// 256 x 256 tiles (above 64 rows), and the first strip of those columns.
+inline void half_tile_config(int M, int N, int bits, int group, int* bm, int* bn, int* strip_lo) {
+  *strip_lo = 0;
+  if (bits == 8 && group == 0) {
+    const int c = plan_big_columns(M, N) * 16, nstrips = N / kStripCols;
+    *strip_lo = c < nstrips ? c : nstrips;
+  }
+  if (bits == 8) {
+    *bm = tall_half_tile(M) ? 256 : 128;
+    *bn = tall_half_tile(M) ? 128 : 256;
+  } else {
+    *bm = 128;
+    *bn = group == 64 ? 128 : 256;
+  }
+}
+
+// How a half-size configuration (one workgroup per CU) covers ncols columns:
+// the column tiles of whole rounds of the CUs run as they are; the tiles of
+// the last, partial round leave CUs idle for a whole tile time, so K is cut
+// into as many runs as fit the idle CUs (2..4, each at least 8 k tiles long,
+// and only if the scratch buffer holds ns x M x columns floats).  The extra
+// traffic is worth it below half occupancy.  full_tiles = 0 with ns = 1 means
+// one plain launch over everything.
+struct TailPlan {
+  int full_tiles;  // column tiles launched without a K split
+  int ns;          // K runs of the remaining column tiles
+};
+inline TailPlan plan_tail(int M, int K, int ncols, int bm, int bn, int tk, size_t ws_bytes) {
+  const int cus = num_cus(), tiles = K / tk;
+  const int nbx = (ncols + bn - 1) / bn, nby = (M + bm - 1) / bm;
+  const int blocks = nbx * nby;
+  if (blocks == 0) return {0, 1};
+  const int full = blocks > cus ? (blocks / cus) * cus / nby : 0;
+  const int rest = (nbx - full) * nby;
+  if (rest == 0) return {0, 1};
+  const size_t rest_cols = static_cast<size_t>(ncols) - static_cast<size_t>(full) * bn;
+  int ns = cus / rest;
   ns = ns > 4 ? 4 : ns;
-  while (ns > 1 && (tiles / ns < 8 || static_cast<size_t>(ns) * M * N * sizeof(float) > ws_bytes)) --ns;
-  return ns < 1 ? 1 : ns;
+  while (ns > 1 && (tiles / ns < 8 || static_cast<size_t>(ns) * M * rest_cols * sizeof(float) > ws_bytes)) --ns;
+  if (ns <= 1) return {0, 1};
+  return {full, ns};
 }
 
 template <int BITS>
@@ -1021,36 +1055,42 @@ void launch_fast(const Args& a) {
     launch_dma<DT, BITS, G, false, 1, 8, 2, 1, 2>(a, 0, nstrips, ns);
     return;
   }
+  constexpr int TK = BITS == 8 ? 64 : 128;
+  int bm = 0, bn = 0, lo = 0;
+  half_tile_config(a.M, a.N, BITS, G, &bm, &bn, &lo);
+  const TailPlan t = plan_tail(a.M, a.K, (nstrips - lo) * kStripCols, bm, bn, TK, a.ws != nullptr ? a.ws_bytes : 0);
+  const int mid = lo + t.full_tiles * (bn / kStripCols);  // strips [lo, mid) unsplit, [mid, nstrips) in t.ns runs
+  // launches a half-size configuration on both parts
+#define WOL_HALF(...)                                              \
+  do {                                                             \
+    launch_dma<DT, BITS, G, __VA_ARGS__>(a, lo, mid, 1);           \
+    launch_dma<DT, BITS, G, __VA_ARGS__>(a, mid, nstrips, t.ns);   \
+  } while (0)
   if constexpr (BITS == 8 && G == 0) {
     // 256 x 256 x 64 tiles (144 KiB of LDS, one workgroup per CU) for as many
     // column tiles as fill whole rounds of the CUs; the rest, which would
     // leave CUs idle for a whole tile time, goes to half-size tiles.
-    const int c = plan_big_columns(a.M, a.N);
-    const int hi = c * 16 < nstrips ? c * 16 : nstrips;
-    launch_dma<DT, BITS, G, false, 2, 4, 4, 2>(a, 0, hi, 1);
-    const int ns = hi == 0 ? plan_split_large(a.M, a.K, a.N, BITS, 0, a.ws != nullptr ? a.ws_bytes : 0) : 1;
-    if (tall_half_tile(a.M)) launch_dma<DT, BITS, G, false, 2, 4, 4, 1>(a, hi, nstrips, ns);
-    else launch_dma<DT, BITS, G, false, 2, 4, 2, 2>(a, hi, nstrips, ns);
+    launch_dma<DT, BITS, G, false, 2, 4, 4, 2>(a, 0, lo, 1);
+    if (bm == 256) WOL_HALF(false, 2, 4, 4, 1);
+    else WOL_HALF(false, 2, 4, 2, 2);
+  } else if constexpr (BITS == 8) {
+    // group-wise scales need a second set of accumulators: half-size tiles
+    if (bm == 256) WOL_HALF(false, 2, 4, 4, 1);
+    else WOL_HALF(false, 2, 4, 2, 2);
+  } else if constexpr (G == 64) {
+    // int4 tiles are 128 k deep; two groups per k tile: two scale sets on top
+    // of two accumulator sets do not fit 256 registers at 128 x 256 (the
+    // spills, being memory loads, also break the in-order accounting of the
+    // tile loads): 128 x 128
+    WOL_HALF(false, 2, 4, 2, 1);
+  } else if constexpr (G == 0 && DT == WOL_DTYPE_BF16) {
+    // the exact int4 -> bf16 dequantiser costs 32 VALU instructions per 8
+    // codes; the offset form plus one cancelling MFMA per A block is faster
+    WOL_HALF(true, 2, 4, 2, 2);
   } else {
-    // int4 tiles are 128 k deep and group-wise scales need a second set of
-    // accumulators: 128 x 256 tiles
-    const int ns = plan_split_large(a.M, a.K, a.N, BITS, G, a.ws != nullptr ? a.ws_bytes : 0);
-    if constexpr (BITS == 8) {
-      if (tall_half_tile(a.M)) { launch_dma<DT, BITS, G, false, 2, 4, 4, 1>(a, 0, nstrips, ns); return; }
-      launch_dma<DT, BITS, G, false, 2, 4, 2, 2>(a, 0, nstrips, ns);
-    } else if constexpr (G == 64) {
-      // two groups per k tile: two scale sets on top of two accumulator sets do
-      // not fit 256 registers at 128 x 256 (the spills, being memory loads,
-      // also break the in-order accounting of the tile loads): 128 x 128
-      launch_dma<DT, BITS, G, false, 2, 4, 2, 1>(a, 0, nstrips, ns);
-    } else if constexpr (G == 0 && DT == WOL_DTYPE_BF16) {
-      // the exact int4 -> bf16 dequantiser costs 32 VALU instructions per 8
-      // codes; the offset form plus one cancelling MFMA per A block is faster
-      launch_dma<DT, BITS, G, true, 2, 4, 2, 2>(a, 0, nstrips, ns);
-    } else {
-      launch_dma<DT, BITS, G, false, 2, 4, 2, 2>(a, 0, nstrips, ns);
-    }
+    WOL_HALF(false, 2, 4, 2, 2);
   }
+#undef WOL_HALF
 }
 
 template <int DT, int BITS>
@@ -1075,9 +1115,12 @@ size_t linear_gemm_workspace(int64_t M, int64_t K, int64_t N, int bits, int grou
   const int tk = bits == 8 ? 64 : 128;
   if (K % tk != 0 || K / tk < 2) return 0;
   if (M > kSkinnyMaxM) {
-    const int ns = plan_split_large(static_cast<int>(M), static_cast<int>(K), static_cast<int>(N), bits,
-                                    group_size > 0 ? group_size : 0, SIZE_MAX);
-    return ns > 1 ? static_cast<size_t>(ns) * M * N * sizeof(float) : 0;
+    int bm = 0, bn = 0, lo = 0;
+    const int g = group_size > 0 ? group_size : 0;
+    half_tile_config(static_cast<int>(M), static_cast<int>(N), bits, g, &bm, &bn, &lo);
+    const int ncols = static_cast<int>(N) - lo * kStripCols;
+    const TailPlan t = plan_tail(static_cast<int>(M), static_cast<int>(K), ncols, bm, bn, tk, SIZE_MAX);
+    return t.ns > 1 ? static_cast<size_t>(t.ns) * M * (ncols - t.full_tiles * bn) * sizeof(float) : 0;
   }
   bool wide = false;
   const int ns = plan_skinny(static_cast<int>(M), static_cast<int>(K), static_cast<int>(N), bits,

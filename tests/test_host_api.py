@@ -66,6 +66,8 @@ def test_workspace_queries(lib):
     assert L.wol_linear_workspace(1, 4096, 11008, 4, 128) == 0       # streaming kernel
     assert L.wol_linear_workspace(2048, 4096, 12288, 8, -1) == 0     # one workgroup per tile covers all of K
     assert L.wol_linear_workspace(1024, 4096, 4096, 8, 64) == 2 * 1024 * 4096 * 4  # 128 tiles: two K runs
+    # 384 tiles: the 256 of the whole round run as they are, the other 128 (4096 columns) in two K runs
+    assert L.wol_linear_workspace(1024, 4096, 12288, 8, 64) == 2 * 1024 * 4096 * 4
     # small M on the GEMM: whole fp32 [M, N] partial buffers, at most 16 of them
     for M, K, N, bits, g in [(64, 8192, 28672, 4, 128), (32, 4096, 11008, 4, -1), (24, 8192, 28672, 4, 128)]:
         need = L.wol_linear_workspace(M, K, N, bits, g)
