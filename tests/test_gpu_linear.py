@@ -426,3 +426,32 @@ def test_stream_kernel_every_k_tail(G, oracle, bits):
             print("case", bits, K, M, g, flush=True)
             check(G, oracle, H.BF16 if (K // 64) % 2 else H.F16, bits, g, M, K, N, bias=(K // 64) % 3 == 0,
                   seed=K + M, kernel=KERNEL_STREAM)
+
+
+@pytest.mark.parametrize("dt,bits,g,M,K,N", [(H.BF16, 8, 64, 300, 2048, 22016), (H.F16, 4, 128, 300, 4096, 22016)])
+def test_gemm_partial_last_round_split(G, oracle, dt, bits, g, M, K, N):
+    # above 64 rows the tiles of a partial last round are launched with K cut
+    # into runs: their columns go through fp32 partial sums and a reduce over
+    # that column range only.  Checked against the same call without scratch
+    # (one launch, no split) and, on a few rows, against the oracle.
+    from paddle_amd import _lib
+
+    need = _lib.lib.wol_linear_workspace(M, K, N, bits, g)
+    assert 0 < need < 2 * 4 * M * N  # a split of some of the columns only
+    wb = H.make_weight(K, N, dt, seed=31)
+    xb = H.make_act(M, K, dt, seed=32)
+    bb = H.make_bias(N, dt, seed=33)
+    oc, osc = oracle.weight_quantize(wb, dt, bits, g)
+    packed = H.gfx950_from_q(H.q_from_canonical(oc, bits), bits)
+    split32 = G.linear(xb, packed, bb, osc, dt, N, bits, g, f32=True)
+    plain32 = G.linear(xb, packed, bb, osc, dt, N, bits, g, f32=True, no_workspace=True)
+    assert np.isfinite(split32).all()
+    assert H.rel_l2(split32, plain32) < 2e-6  # the same products, summed in another order
+    # the columns outside the split are bit-identical
+    same = (split32 == plain32).all(axis=0)
+    assert same.sum() >= N // 2
+    splitT = G.linear(xb, packed, bb, osc, dt, N, bits, g)
+    assert np.array_equal(splitT, H.f32_to_bits(split32, dt))
+    rows = np.r_[0:3, M - 3:M]
+    r32, _ = oracle.linear(xb[rows], oc, osc, bb, dt, bits, g)
+    assert H.rel_l2(split32[rows], r32) < 2e-5
