@@ -221,6 +221,47 @@ int wol_apply_per_channel_scale(const void* x, const void* scales, int dtype,
                                 void* stream);
 
 /*
+ * Replaces LLMInt8LinearKernel<T, GPUContext>
+ * (paddle/phi/kernels/gpu/llm_int8_linear_kernel.cu:29-79, the stages of
+ * paddle/phi/kernels/impl/llm_int8_matmul_kernel_impl.h:560-690; shape
+ * contract LLMInt8LinearInferMeta, paddle/phi/infermeta/multiary.cc:3792-3837).
+ *   x [M,K] T; weight [N,K] int8 and weight_scale [N] float as
+ *   weight_quantize(algo="llm.int8") returns them (wol_quantize_llm_int8 with
+ *   WOL_LAYOUT_PADDLE_HIP, group_size -1); bias [N] T or NULL; out [M,N] T.
+ *   Column k is an outlier when any |x[m,k]| > T(threshold).
+ *   range[m]  = max_k |x[m,k]| over the elements not above the threshold
+ *   qx[m,k]   = 0 in outlier columns, else clip(round(x * 127 * (1 / range[m])), -127, 127)
+ *   acc[m,n]  = sum_k qx[m,k] * weight[n,k]                         (int32, exact)
+ *   sub[m,n]  = T( sum over outlier k, ascending, of x[m,k] * T(weight[n,k] * weight_scale[n]) )  (fp32 sum)
+ *   out[m,n]  = T( sub + T(acc * range[m] * weight_scale[n] / 127) ), then T(out + bias[n])
+ * The reference reads the weight of the outlier columns through the index
+ * permutation of another layout (impl/llm_int8_matmul_kernel_impl.h:351-362)
+ * than the one its quantiser writes; this library indexes weight[n,k] plainly,
+ * as the operator's description and the reference's own test
+ * (test/quantization/test_llm_int8_linear.py:84-111) have it.
+ * Requires K % 64 == 0 and N % 16 == 0 (what weight_quantize accepts); x,
+ * weight, weight_scale, out and workspace 16-byte aligned.  The workspace is
+ * required (wol_llm_int8_linear_workspace bytes); it holds the row ranges,
+ * the outlier mask and list, the activation codes and, for few rows, int32
+ * sums.  Nothing returns to the host: the reference's device-to-host copy of
+ * the outlier count has no counterpart here.
+ */
+size_t wol_llm_int8_linear_workspace(int64_t M, int64_t K, int64_t N);
+int wol_llm_int8_linear(const void* x, const void* weight, const void* bias,
+                        const float* weight_scale, float threshold, int dtype,
+                        int64_t M, int64_t K, int64_t N, void* out,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/* Where the intermediate results of wol_llm_int8_linear lie in its workspace
+ * after a call, as byte offsets: [0] range (float [M]), [1] outlier mask
+ * (bit k % 32 of int32 word k / 32), [2] outlier count (int32), [3] outlier
+ * columns (int32, ascending), [4] activation codes (int8 [M,K]), [5] int32
+ * sums [M,N] or -1 when the GEMM writes the output itself.  For tests that
+ * compare the stages with the reference's; no counterpart there. */
+int wol_llm_int8_linear_stage_offsets(int64_t M, int64_t K, int64_t N,
+                                      int64_t* offsets);
+
+/*
  * Measurement aid with no counterpart in the reference: reads a GFX950-layout
  * weight with the launch shape of the one-row decode kernel (one workgroup of
  * eight wavefronts per 16-column strip, 16-byte non-temporal loads, all of a

@@ -23,6 +23,15 @@
  *   dequant/linear: products of <=8-bit codes with <=11-bit scales are exact
  *                   in fp32, so dequant has one correct answer; the linear is
  *                   checked against a float64 matmul of the same operands.
+ *   llm.int8      : activation codes pinned by a numpy statement and invariants,
+ *                   the int32 accumulators by numpy's integer matmul, the merge
+ *                   by float64 evaluation.  PARITY UNPINNED for the outlier
+ *                   branch: the reference reads the weight there through the
+ *                   index permutation of another layout
+ *                   (impl/llm_int8_matmul_kernel_impl.h:351-362) that
+ *                   weight_quantize(algo="llm.int8") does not produce, and its
+ *                   own tests never reach the branch; this restatement indexes
+ *                   the weight plainly, as the op's description has it.
  *   pre-scale     : one correctly rounded multiply in T; pinned against the
  *                   half-precision multiply of numpy (fp16) and torch (bf16),
  *                   which are library routines with that definition, and by
@@ -413,4 +422,78 @@ void wo_apply_per_channel_scale(const uint16_t* x, const uint16_t* scales,
       out[r * cols + c] = wo_from_f32(
           wo_to_f32(x[r * cols + c], dtype) * wo_to_f32(scales[c], dtype), dtype,
           WO_CAST_RNE);
+}
+
+/* ---- llm.int8 linear --------------------------------------------------- */
+
+/* LLMGemm (paddle/phi/kernels/impl/llm_int8_matmul_kernel_impl.h:560-690) and
+ * llm_int8_compute (gpu/llm_int8_linear_kernel.cu:29-64), stage by stage:
+ *   ReduceAbsMaxKernel (:221-268): column k is an outlier if any |x[m,k]| >
+ *     T(threshold) (compared in T); range[m] = max over the row of |x| with
+ *     the elements above the threshold counted as 0.
+ *   QuantActKernel (:270-303), QuantFunc (:153-164): q = 0 in outlier columns,
+ *     else clip(round(x * 127 * (1 / range[m])), -127, 127), products left to
+ *     right in fp32, C round().
+ *   int8 GEMM: acc[m,n] = sum_k q[m,k] * w[n,k] in int32.
+ *   outlier columns (:593-640): sub[m,n] = T(sum_k x[m,k] * T(w[n,k] *
+ *     wscale[n])) over the outlier columns (fp32 accumulation), 0 without any.
+ *   DequantMergeKernel (:415-447), DequantFunc (:172-176): out = T(sub +
+ *     T(acc * range[m] * wscale[n] / 127)), products left to right.
+ *   bias: out = T(out + bias[n]).
+ * w is [N,K] signed int8, wscale fp32 [N].  qx (optional) receives the codes,
+ * acc (optional) the int32 sums, ranges (optional) the row maxima, outlier
+ * (optional, K bytes) the column flags. */
+void wo_llm_int8_linear(const uint16_t* x, const int8_t* w, const uint16_t* bias,
+                        const float* wscale, float threshold, int64_t M,
+                        int64_t K, int64_t N, int dtype, uint16_t* out,
+                        int8_t* qx_out, int32_t* acc_out, float* ranges_out,
+                        uint8_t* outlier_out) {
+  const float thr = wo_to_f32(wo_from_f32(threshold, dtype, WO_CAST_RNE), dtype);
+  uint8_t* outlier = (uint8_t*)calloc((size_t)K, 1);
+  float* range = (float*)malloc((size_t)M * sizeof(float));
+  int8_t* q = (int8_t*)malloc((size_t)M * K);
+  for (int64_t m = 0; m < M; ++m) {
+    float mx = 0.0f;
+    for (int64_t k = 0; k < K; ++k) {
+      float a = fabsf(wo_to_f32(x[m * K + k], dtype));
+      if (a > thr) { outlier[k] = 1; a = 0.0f; }
+      if (a > mx) mx = a;
+    }
+    range[m] = mx;
+  }
+  for (int64_t m = 0; m < M; ++m) {
+    const float inv = 1.0f / range[m];
+    for (int64_t k = 0; k < K; ++k) {
+      float t = 0.0f;
+      if (!outlier[k]) {
+        t = wo_to_f32(x[m * K + k], dtype) * 127.0f * inv;
+        t = roundf(t);
+        if (t > 127.0f) t = 127.0f; else if (t < -127.0f) t = -127.0f;
+        if (t != t) t = 0.0f; /* 0 * inf in an all-zero row: undefined in the reference */
+      }
+      q[m * K + k] = (int8_t)t;
+    }
+  }
+  for (int64_t m = 0; m < M; ++m)
+    for (int64_t n = 0; n < N; ++n) {
+      int32_t acc = 0;
+      float sub = 0.0f;
+      for (int64_t k = 0; k < K; ++k) {
+        acc += (int32_t)q[m * K + k] * (int32_t)w[n * K + k];
+        if (outlier[k]) {
+          float wd = wo_to_f32(wo_from_f32((float)w[n * K + k] * wscale[n], dtype, WO_CAST_RNE), dtype);
+          sub += wo_to_f32(x[m * K + k], dtype) * wd;
+        }
+      }
+      if (acc_out) acc_out[m * N + n] = acc;
+      float subT = wo_to_f32(wo_from_f32(sub, dtype, WO_CAST_RNE), dtype);
+      float dq = wo_to_f32(wo_from_f32((float)acc * range[m] * wscale[n] / 127.0f, dtype, WO_CAST_RNE), dtype);
+      uint16_t o = wo_from_f32(subT + dq, dtype, WO_CAST_RNE);
+      if (bias) o = wo_from_f32(wo_to_f32(o, dtype) + wo_to_f32(bias[n], dtype), dtype, WO_CAST_RNE);
+      out[m * N + n] = o;
+    }
+  if (qx_out) memcpy(qx_out, q, (size_t)M * K);
+  if (ranges_out) memcpy(ranges_out, range, (size_t)M * sizeof(float));
+  if (outlier_out) memcpy(outlier_out, outlier, (size_t)K);
+  free(outlier); free(range); free(q);
 }

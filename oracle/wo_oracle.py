@@ -57,6 +57,10 @@ def lib():
         L.wo_transpose_bytes.argtypes = [_i8p, _i64, _i64, _i8p]
         L.wo_apply_per_channel_scale.argtypes = [_u16p, _u16p, _i64, _i64, _int, _u16p]
         L.wo_apply_per_channel_scale.restype = None
+        L.wo_llm_int8_linear.argtypes = [_u16p, _i8p, ctypes.c_void_p, _f32p, ctypes.c_float, _i64, _i64, _i64,
+                                         _int, _u16p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                         ctypes.c_void_p]
+        L.wo_llm_int8_linear.restype = None
         L.wo_dequantize.argtypes = [_i8p, _u16p, _i64, _i64, _int, _int, _i64, _int, _int,
                                     ctypes.c_void_p, ctypes.c_void_p]
         L.wo_linear.argtypes = [_u16p, _i8p, ctypes.c_void_p, _u16p, _i64, _i64, _i64, _int, _int,
@@ -117,6 +121,30 @@ def apply_per_channel_scale(x_bits, scale_bits, dtype):
     out = np.empty((rows, cols), np.uint16)
     lib().wo_apply_per_channel_scale(x_bits, scale_bits, rows, cols, dtype, out)
     return out
+
+
+def llm_int8_linear(x_bits, w_nk, bias_bits, wscale, threshold, dtype):
+    """x_bits [M,K] uint16, w_nk [N,K] int8, wscale [N] float32.  Returns a dict:
+    out (T bits [M,N]), qx (int8 [M,K]), acc (int32 [M,N]), ranges (float32 [M]),
+    outlier (bool [K])."""
+    x_bits = np.ascontiguousarray(x_bits, dtype=np.uint16)
+    w_nk = np.ascontiguousarray(w_nk, dtype=np.int8)
+    wscale = np.ascontiguousarray(wscale, dtype=np.float32)
+    M, K = x_bits.shape
+    N = w_nk.shape[0]
+    assert w_nk.shape == (N, K) and wscale.shape == (N,)
+    out = np.empty((M, N), np.uint16)
+    qx = np.empty((M, K), np.int8)
+    acc = np.empty((M, N), np.int32)
+    ranges = np.empty(M, np.float32)
+    outlier = np.empty(K, np.uint8)
+    bias_ptr = None
+    if bias_bits is not None:
+        bias_bits = np.ascontiguousarray(bias_bits, dtype=np.uint16)
+        bias_ptr = bias_bits.ctypes.data
+    lib().wo_llm_int8_linear(x_bits, w_nk, bias_ptr, wscale, float(threshold), M, K, N, dtype, out,
+                             qx.ctypes.data, acc.ctypes.data, ranges.ctypes.data, outlier.ctypes.data)
+    return {"out": out, "qx": qx, "acc": acc, "ranges": ranges, "outlier": outlier.astype(bool)}
 
 
 def transpose_bytes(a):

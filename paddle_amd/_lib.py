@@ -30,6 +30,9 @@ SYMBOLS = (
     "wol_code_offset",
     "wol_apply_per_channel_scale",
     "wol_read_floor",
+    "wol_llm_int8_linear_workspace",
+    "wol_llm_int8_linear",
+    "wol_llm_int8_linear_stage_offsets",
 )
 
 
@@ -75,6 +78,12 @@ def _load():
     lib.wol_apply_per_channel_scale.restype = ci
     lib.wol_read_floor.argtypes = [vp, i64, i64, ci, vp, vp]
     lib.wol_read_floor.restype = ci
+    lib.wol_llm_int8_linear_workspace.argtypes = [i64, i64, i64]
+    lib.wol_llm_int8_linear_workspace.restype = sz
+    lib.wol_llm_int8_linear.argtypes = [vp, vp, vp, vp, ctypes.c_float, ci, i64, i64, i64, vp, vp, sz, vp]
+    lib.wol_llm_int8_linear.restype = ci
+    lib.wol_llm_int8_linear_stage_offsets.argtypes = [i64, i64, i64, ctypes.POINTER(i64)]
+    lib.wol_llm_int8_linear_stage_offsets.restype = ci
     return lib
 
 

@@ -231,6 +231,36 @@ int wol_apply_per_channel_scale(const void* x, const void* scales, int dtype, in
   return wol::launch_prescale(x, scales, dtype, rows, cols, out, static_cast<hipStream_t>(stream));
 }
 
+size_t wol_llm_int8_linear_workspace(int64_t M, int64_t K, int64_t N) {
+  if (check_problem(WOL_DTYPE_F16, K, N, 8, -1) != WOL_OK || M <= 0 || M > (int64_t{1} << 24)) return 0;
+  return wol::llm_int8_workspace(M, K, N);
+}
+
+int wol_llm_int8_linear_stage_offsets(int64_t M, int64_t K, int64_t N, int64_t* offsets) {
+  if (offsets == nullptr) return WOL_ERR_NULL_POINTER;
+  if (check_problem(WOL_DTYPE_F16, K, N, 8, -1) != WOL_OK || M <= 0 || M > (int64_t{1} << 24))
+    return WOL_ERR_BAD_SHAPE;
+  wol::llm_int8_workspace_offsets(M, K, N, offsets);
+  return WOL_OK;
+}
+
+int wol_llm_int8_linear(const void* x, const void* weight, const void* bias, const float* weight_scale,
+                        float threshold, int dtype, int64_t M, int64_t K, int64_t N, void* out,
+                        void* workspace, size_t workspace_bytes, void* stream) {
+  const int rc = check_problem(dtype, K, N, 8, -1);
+  if (rc != WOL_OK) return rc;
+  if (M < 0 || M > (int64_t{1} << 24)) return WOL_ERR_BAD_SHAPE;
+  if (M == 0) return WOL_OK;  // empty batch: nothing to write
+  if (x == nullptr || weight == nullptr || weight_scale == nullptr || out == nullptr)
+    return WOL_ERR_NULL_POINTER;
+  if (!aligned16(x) || !aligned16(weight) || !aligned16(weight_scale) || !aligned16(out))
+    return WOL_ERR_ALIGNMENT;
+  if (workspace == nullptr || workspace_bytes < wol::llm_int8_workspace(M, K, N)) return WOL_ERR_WORKSPACE;
+  if (!aligned16(workspace)) return WOL_ERR_ALIGNMENT;
+  return wol::launch_llm_int8_linear(x, weight, bias, weight_scale, threshold, dtype, M, K, N, out, workspace,
+                                     static_cast<hipStream_t>(stream));
+}
+
 int wol_read_floor(const void* codes, int64_t K, int64_t N, int bits, void* out, void* stream) {
   const int rc = check_problem(WOL_DTYPE_F16, K, N, bits, -1);
   if (rc != WOL_OK) return rc;

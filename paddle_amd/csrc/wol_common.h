@@ -218,6 +218,14 @@ int launch_read_floor(const void* codes, int64_t K, int64_t N, int bits, void* o
                       hipStream_t stream);
 int launch_prescale(const void* x, const void* scales, int dtype, int64_t rows, int64_t cols,
                     void* out, hipStream_t stream);
+int launch_llm_int8_linear(const void* x, const void* weight, const void* bias, const float* wscale,
+                           float threshold, int dtype, int64_t M, int64_t K, int64_t N, void* out,
+                           void* workspace, hipStream_t stream);
+// Scratch bytes launch_llm_int8_linear needs, and where its stages lie in them
+// (ranges, outlier mask, outlier count, outlier list, activation codes, int32
+// sums or -1 when the GEMM writes the output itself).
+size_t llm_int8_workspace(int64_t M, int64_t K, int64_t N);
+void llm_int8_workspace_offsets(int64_t M, int64_t K, int64_t N, int64_t* offsets);
 // Scratch bytes with which launch_linear_gemm splits K across workgroups (0: none needed).
 size_t linear_gemm_workspace(int64_t M, int64_t K, int64_t N, int bits, int group_size);
 

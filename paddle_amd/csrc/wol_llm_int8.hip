@@ -1,0 +1,608 @@
+// llm_int8_linear for gfx950: dynamic per-row int8 quantisation of the
+// activations, an int8 x int8 -> int32 MFMA GEMM against the plain [N,K] int8
+// weight that weight_quantize(algo="llm.int8") returns, the outlier columns in
+// T x dequantised-weight arithmetic, and the merge of the two.
+//
+// Stages (paddle/phi/kernels/impl/llm_int8_matmul_kernel_impl.h:560-690 runs
+// the same ones as separate kernels plus two library GEMMs and a device-to-host
+// copy of the outlier count; here nothing returns to the host):
+//   clear   : outlier bit mask and count to zero
+//   rowmax  : range[m] = max |x[m,k]| over the elements not above the
+//             threshold; bit k of the mask set where any |x[m,k]| > threshold
+//             (ReduceAbsMaxKernel, :221-268)
+//   quant   : qx = 0 in outlier columns, else clip(round(x * 127 * (1/range)))
+//             (QuantActKernel :270-303, QuantFunc :153-164); one extra
+//             workgroup turns the mask into an ascending list of columns
+//   gemm    : acc = qx . w^T in int32 on v_mfma_i32_32x32x32_i8, both operands
+//             through direct-to-LDS loads, three k tiles deep.  The epilogue is
+//             DequantMergeKernel (:415-447) with the outlier product folded in:
+//             out = T( T(sum_outliers x * T(w * wscale)) + T(acc * range *
+//             wscale / 127) ), then T(out + bias).
+//   merge   : only when K is cut into runs (few rows): the runs add their int32
+//             sums with integer atomics (exact, so order does not matter) and
+//             this kernel applies the same epilogue.
+#include <atomic>
+
+#include "wol_common.h"
+
+namespace wol {
+namespace {
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+constexpr int kTK = 64;      // k (bytes) per tile row
+constexpr int kStages = 3;
+
+// float -> T, round to nearest even, of exactly the fp32 value given: the
+// barrier keeps the compiler from merging the producing multiply or add with
+// the conversion into one instruction that rounds once.
+template <int DT>
+__device__ inline uint16_t cast_exact(float f) {
+  asm volatile("" : "+v"(f));
+  return from_f32_rne<DT>(f);
+}
+
+template <int DT>
+__device__ inline float round_to_t(float f) {
+  return to_f32<DT>(cast_exact<DT>(f));
+}
+
+template <int N_>
+__device__ inline void wait_vmcnt() {
+  // gfx9 encoding: vmcnt = [15:14][3:0], expcnt = [6:4], lgkmcnt = [11:8]
+  __builtin_amdgcn_s_waitcnt((N_ & 0xF) | ((N_ >> 4) << 14) | (0x7 << 4) | (0xF << 8));
+}
+
+// ---------------------------------------------------------------------------
+// activation side
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void llm_clear_kernel(int32_t* mask, int nwords, int32_t* count) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < nwords) mask[i] = 0;
+  if (i == 0) *count = 0;
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void llm_rowmax_kernel(const uint16_t* __restrict__ x, float threshold,
+                                                         int K, float* __restrict__ ranges,
+                                                         int32_t* __restrict__ mask) {
+  __shared__ float part[4];
+  const float thr = to_f32<DT>(from_f32_rne<DT>(threshold));  // the comparison is made in T
+  const uint16_t* row = x + static_cast<int64_t>(blockIdx.x) * K;
+  float mx = 0.0f;
+  for (int k0 = threadIdx.x * 8; k0 < K; k0 += 256 * 8) {
+    const u32x4 v = *reinterpret_cast<const u32x4*>(row + k0);
+    uint32_t bits = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float a = fabsf(to_f32<DT>(static_cast<uint16_t>(v[i >> 1] >> (16 * (i & 1)))));
+      if (a > thr) {
+        bits |= 1u << i;
+        a = 0.0f;
+      }
+      mx = a > mx ? a : mx;
+    }
+    if (bits != 0) atomicOr(&mask[k0 >> 5], static_cast<int32_t>(bits << (k0 & 31)));
+  }
+#pragma unroll
+  for (int d = 32; d > 0; d >>= 1) {
+    const float o = __shfl_xor(mx, d, 64);
+    mx = o > mx ? o : mx;
+  }
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float r = part[0];
+#pragma unroll
+    for (int i = 1; i < 4; ++i) r = part[i] > r ? part[i] : r;
+    ranges[blockIdx.x] = r;
+  }
+}
+
+// QuantFunc (:153-164).  NaN (0 * inf in a row whose range is 0) becomes 0.
+__device__ inline uint32_t quant_one(float xv, float inv) {
+  float t = xv * 127.0f * inv;
+  t = roundf(t);
+  t = t > 127.0f ? 127.0f : (t < -127.0f ? -127.0f : t);
+  if (t != t) t = 0.0f;
+  return static_cast<uint32_t>(static_cast<int>(t)) & 0xFFu;
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void llm_quant_kernel(const uint16_t* __restrict__ x,
+                                                        const float* __restrict__ ranges,
+                                                        const int32_t* __restrict__ mask, int M, int K,
+                                                        int8_t* __restrict__ qx, int32_t* __restrict__ count,
+                                                        int32_t* __restrict__ list, int32_t* __restrict__ acc,
+                                                        int64_t acc_vec) {
+  const int tid = threadIdx.x;
+  if (blockIdx.x == gridDim.x - 1) {
+    // the mask as an ascending list of outlier columns
+    __shared__ int scan[256];
+    __shared__ int base_s;
+    const int nwords = K / 32;
+    if (tid == 0) base_s = 0;
+    __syncthreads();
+    for (int w0 = 0; w0 < nwords; w0 += 256) {
+      uint32_t word = w0 + tid < nwords ? static_cast<uint32_t>(mask[w0 + tid]) : 0u;
+      const int c = __popc(word);
+      scan[tid] = c;
+      __syncthreads();
+      for (int d = 1; d < 256; d <<= 1) {
+        const int add = tid >= d ? scan[tid - d] : 0;
+        __syncthreads();
+        scan[tid] += add;
+        __syncthreads();
+      }
+      const int base = base_s;
+      int o = base + scan[tid] - c;
+      while (word != 0) {
+        const int b = __ffs(word) - 1;
+        list[o++] = (w0 + tid) * 32 + b;
+        word &= word - 1;
+      }
+      __syncthreads();
+      if (tid == 0) base_s = base + scan[255];
+      __syncthreads();
+    }
+    if (tid == 0) *count = base_s;
+    return;
+  }
+  const int64_t stride = static_cast<int64_t>(gridDim.x - 1) * 256;
+  const int64_t first = static_cast<int64_t>(blockIdx.x) * 256 + tid;
+  const int64_t nvec = static_cast<int64_t>(M) * K / 16;
+  for (int64_t v = first; v < nvec; v += stride) {
+    const int64_t e = v * 16;
+    const int m = static_cast<int>(e / K);
+    const int k = static_cast<int>(e - static_cast<int64_t>(m) * K);
+    const u32x4 lo = *reinterpret_cast<const u32x4*>(x + e);
+    const u32x4 hi = *reinterpret_cast<const u32x4*>(x + e + 8);
+    const uint32_t out_bits = static_cast<uint32_t>(mask[k >> 5]) >> (k & 31);
+    const float inv = 1.0f / ranges[m];
+    u32x4 q = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const uint32_t word = i < 8 ? lo[(i & 7) >> 1] : hi[(i & 7) >> 1];
+      const float xv = to_f32<DT>(static_cast<uint16_t>(word >> (16 * (i & 1))));
+      const uint32_t c = (out_bits >> i) & 1u ? 0u : quant_one(xv, inv);
+      q[i >> 2] |= c << (8 * (i & 3));
+    }
+    *reinterpret_cast<u32x4*>(qx + e) = q;
+  }
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  for (int64_t i = first; i < acc_vec; i += stride) reinterpret_cast<u32x4*>(acc)[i] = zero;
+}
+
+// ---------------------------------------------------------------------------
+// the epilogue arithmetic, shared by the GEMM and the merge kernel
+// ---------------------------------------------------------------------------
+struct Epi {
+  const uint16_t* x;      // [M,K] T
+  const int8_t* w;        // [N,K]
+  const float* wscale;    // [N]
+  const float* ranges;    // [M]
+  const uint16_t* bias;   // [N] T or null
+  const int32_t* count;
+  const int32_t* list;
+  uint16_t* out;          // [M,N] T
+  int M, K, N;
+};
+
+// DequantFunc (:172-176) and the two T additions that follow it.
+template <int DT>
+__device__ inline uint16_t merge_one(int acc, float sub, float range, float ws, bool has_bias, float bias) {
+  const float dq = round_to_t<DT>(static_cast<float>(acc) * range * ws / 127.0f);
+  const float o = round_to_t<DT>(round_to_t<DT>(sub) + dq);
+  return has_bias ? cast_exact<DT>(o + bias) : cast_exact<DT>(o);
+}
+
+// ---------------------------------------------------------------------------
+// int8 GEMM
+// ---------------------------------------------------------------------------
+struct GemmParams {
+  const int8_t* qx;  // [M,K]
+  Epi e;
+  int32_t* acc;      // [M,N] int32, zeroed; only with K runs
+  int nbx, nby;      // tiles along N and M
+  int tiles_per_run; // k tiles per K run
+};
+
+// XOR applied to the 16-byte piece index (four per 64-byte row) so that the
+// 16 rows a quarter of a wavefront reads hit distinct LDS banks, whether the
+// LDS serves 8 or 16 lanes of a 128-bit read per cycle.
+__device__ inline int row_swizzle(int row) {
+  return ((((row >> 1) ^ (row >> 3)) & 1) << 1) | ((row >> 2) & 1);
+}
+
+// WM x WN wavefronts, each TM x TN blocks of 32x32.  RUNS: K is cut into runs
+// across workgroups, which add into acc; otherwise the epilogue writes out.
+template <int DT, int WM, int WN, int TM, int TN, bool RUNS>
+__global__ __launch_bounds__(WM* WN * 64) __attribute__((amdgpu_waves_per_eu(2))) void llm_gemm_kernel(GemmParams p) {
+  constexpr int NW = WM * WN;
+  constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
+  constexpr int kABytes = BM * kTK, kBBytes = BN * kTK, kStage = kABytes + kBBytes;
+  constexpr int kABlocks = kABytes / 1024, kBBlocks = kBBytes / 1024;  // 1 KiB = one wavefront load
+  constexpr int kALoads = (kABlocks + NW - 1) / NW, kBLoads = (kBBlocks + NW - 1) / NW;
+  constexpr int kPerStage = kALoads + kBLoads;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+  const int M = p.e.M, K = p.e.K, N = p.e.N;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  const int r32 = lane & 31, b = lane >> 5;
+
+  // tile of this workgroup.  Consecutive workgroup ids go round the eight
+  // XCDs; each XCD gets a band of column tiles with every row tile, so that
+  // its L2 holds that band's weights once.
+  const int ntiles = p.nbx * p.nby;
+  const int run = blockIdx.x / ntiles;
+  const int t = blockIdx.x - run * ntiles;
+  int bx, by;
+  if (p.nbx % 8 == 0) {
+    const int xcd = t & 7, idx = t >> 3;
+    bx = xcd * (p.nbx / 8) + idx / p.nby;
+    by = idx % p.nby;
+  } else {
+    bx = t / p.nby;
+    by = t % p.nby;
+  }
+  const int m0 = by * BM, n0 = bx * BN;
+  const int ktiles = K / kTK;
+  const int t0 = run * p.tiles_per_run;
+  const int niter = (ktiles - t0) < p.tiles_per_run ? (ktiles - t0) : p.tiles_per_run;
+
+  // global sources of this lane's direct-to-LDS loads.  LDS piece q (16 bytes)
+  // of a tile region is row q / 4, slot q % 4, and holds the row's logical
+  // piece slot ^ swizzle(row).  Rows past M or N repeat the last valid row:
+  // computed on valid data, never stored.  Where a region has fewer 1 KiB
+  // blocks than there are wavefronts, some blocks are loaded twice.
+  // (the casts at the load builtin are needed: with the array element passed as
+  // it is, host compilation silently leaves out the kernel's stub and the
+  // library does not link)
+  const uint8_t* asrc[kALoads];
+  int ablk[kALoads];
+#pragma unroll
+  for (int c = 0; c < kALoads; ++c) {
+    ablk[c] = (c * NW + wave) % kABlocks;
+    const int q = ablk[c] * 64 + lane;
+    const int row = q >> 2, cc = (q & 3) ^ row_swizzle(row);
+    int m = m0 + row;
+    m = m < M ? m : M - 1;
+    asrc[c] = reinterpret_cast<const uint8_t*>(p.qx) + static_cast<int64_t>(m) * K + static_cast<int64_t>(t0) * kTK + cc * 16;
+  }
+  const uint8_t* bsrc[kBLoads];
+  int bblk[kBLoads];
+#pragma unroll
+  for (int c = 0; c < kBLoads; ++c) {
+    bblk[c] = (c * NW + wave) % kBBlocks;
+    const int q = bblk[c] * 64 + lane;
+    const int row = q >> 2, cc = (q & 3) ^ row_swizzle(row);
+    int n = n0 + row;
+    n = n < N ? n : N - 1;
+    bsrc[c] = reinterpret_cast<const uint8_t*>(p.e.w) + static_cast<int64_t>(n) * K + static_cast<int64_t>(t0) * kTK + cc * 16;
+  }
+  // tile `it` of this run into its stage; past the end of the run the last
+  // tile again, into a spare stage, so that every iteration issues the same
+  // number of loads
+#define WOL_LLM_ISSUE(it_)                                                                           \
+  do {                                                                                               \
+    const int koff_ = ((it_) < niter ? (it_) : niter - 1) * kTK;                                      \
+    unsigned char* stage_ = smem + ((it_) % kStages) * kStage;                                        \
+    _Pragma("unroll") for (int c = 0; c < kALoads; ++c) __builtin_amdgcn_global_load_lds(             \
+        reinterpret_cast<const uint8_t*>(asrc[c]) + koff_, (lds_ptr_t)(stage_ + ablk[c] * 1024), 16, 0, 0); \
+    _Pragma("unroll") for (int c = 0; c < kBLoads; ++c) __builtin_amdgcn_global_load_lds(             \
+        reinterpret_cast<const uint8_t*>(bsrc[c]) + koff_, (lds_ptr_t)(stage_ + kABytes + bblk[c] * 1024), \
+        16, 0, 0);                                                                                   \
+  } while (0)
+
+  i32x16 acc[TM][TN];
+#pragma unroll
+  for (int a = 0; a < TM; ++a)
+#pragma unroll
+    for (int c = 0; c < TN; ++c)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[a][c][v] = 0;
+
+  // byte offsets of this lane's fragments inside a stage, for k step 0; k step
+  // 1 is the same with the piece index XOR 2
+  const int swz = row_swizzle(r32);  // rows are 32 * block + r32: the swizzle has period 16
+  int aoff[TM], boff[TN];
+#pragma unroll
+  for (int a = 0; a < TM; ++a) aoff[a] = ((wm * TM + a) * 32 + r32) * kTK;
+#pragma unroll
+  for (int c = 0; c < TN; ++c) boff[c] = kABytes + ((wn * TN + c) * 32 + r32) * kTK;
+
+  WOL_LLM_ISSUE(0);
+  WOL_LLM_ISSUE(1);
+  for (int it = 0; it < niter; ++it) {
+    wait_vmcnt<kPerStage>();  // loads complete in order: all but the newest stage have landed
+    __syncthreads();
+    WOL_LLM_ISSUE(it + 2);  // into the stage every wavefront finished reading before the barrier
+    const unsigned char* stage = smem + (it % kStages) * kStage;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const int piece = ((ks * 2 + b) ^ swz) * 16;
+      i32x4 af[TM], bf[TN];
+#pragma unroll
+      for (int a = 0; a < TM; ++a) af[a] = *reinterpret_cast<const i32x4*>(stage + aoff[a] + piece);
+#pragma unroll
+      for (int c = 0; c < TN; ++c) bf[c] = *reinterpret_cast<const i32x4*>(stage + boff[c] + piece);
+#pragma unroll
+      for (int a = 0; a < TM; ++a)
+#pragma unroll
+        for (int c = 0; c < TN; ++c)
+          acc[a][c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bf[c], acc[a][c], 0, 0, 0);
+    }
+  }
+#undef WOL_LLM_ISSUE
+  wait_vmcnt<0>();  // the spare-stage loads must have landed before the LDS is reused (or the workgroup ends)
+
+  // accumulator v of a 32x32 block: row 8 * (v / 4) + 4 * (lane / 32) + v % 4, column lane % 32
+  const Epi& e = p.e;
+  // Each wavefront passes its blocks one at a time through a slab of LDS of its
+  // own (32 rows of kSlabRow ints: with that stride the two halves of the
+  // wavefront write to disjoint banks) and takes them back as rows: a lane
+  // owns eight neighbouring columns of one row, so the output leaves as
+  // 16-byte stores (with K runs: as eight integer atomics into the sums).  The
+  // loop over the rows is a real loop, which keeps the epilogue's registers few.
+  constexpr int kSlabRow = 40;
+  __syncthreads();  // every wavefront is done with the stages
+  int* slab = reinterpret_cast<int*>(smem) + wave * (32 * kSlabRow);
+  const int cnt = RUNS ? 0 : *e.count;
+  const int cgrp = (lane & 3) * 8;  // first of this lane's eight columns inside the block
+#pragma unroll
+  for (int c = 0; c < TN; ++c) {
+    const int n = n0 + (wn * TN + c) * 32 + cgrp;
+    const bool n_ok = n < N;  // N is a multiple of 16: eight columns are all inside or all outside
+    const int nn = n_ok ? n : 0;
+    float ws[8], bias[8];
+    if (!RUNS) {
+      const f32x4 w0 = *reinterpret_cast<const f32x4*>(e.wscale + nn);
+      const f32x4 w1 = *reinterpret_cast<const f32x4*>(e.wscale + nn + 4);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        ws[i] = w0[i];
+        ws[4 + i] = w1[i];
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) bias[i] = e.bias != nullptr ? to_f32<DT>(e.bias[nn + i]) : 0.0f;
+    }
+#pragma unroll
+    for (int a = 0; a < TM; ++a) {
+      __builtin_amdgcn_wave_barrier();  // the rows of the previous block have been read
+#pragma unroll
+      for (int v = 0; v < 16; ++v) slab[(8 * (v >> 2) + 4 * b + (v & 3)) * kSlabRow + r32] = acc[a][c][v];
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll 1
+      for (int h = 0; h < 2; ++h) {
+        const int row = h * 16 + (lane >> 2);
+        const int m = m0 + (wm * TM + a) * 32 + row;
+        if (m >= M || !n_ok) continue;
+        const i32x4 s0 = *reinterpret_cast<const i32x4*>(slab + row * kSlabRow + cgrp);
+        const i32x4 s1 = *reinterpret_cast<const i32x4*>(slab + row * kSlabRow + cgrp + 4);
+        if (RUNS) {
+          int32_t* dst = p.acc + static_cast<int64_t>(m) * N + nn;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            atomicAdd(dst + i, s0[i]);
+            atomicAdd(dst + 4 + i, s1[i]);
+          }
+          continue;
+        }
+        float sub[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sub[i] = 0.0f;
+#pragma unroll 1
+        for (int j = 0; j < cnt; ++j) {
+          const int kj = e.list[j];
+          const float xv = to_f32<DT>(e.x[static_cast<int64_t>(m) * K + kj]);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const float wd =
+                round_to_t<DT>(static_cast<float>(e.w[static_cast<int64_t>(nn + i) * K + kj]) * ws[i]);
+            sub[i] += xv * wd;
+          }
+        }
+        const float range = e.ranges[m];
+        u32x4 o;
+#pragma unroll
+        for (int i = 0; i < 8; i += 2) {
+          const uint32_t lo =
+              merge_one<DT>(i < 4 ? s0[i] : s1[i - 4], sub[i], range, ws[i], e.bias != nullptr, bias[i]);
+          const uint32_t hi = merge_one<DT>(i < 4 ? s0[i + 1] : s1[i - 3], sub[i + 1], range, ws[i + 1],
+                                            e.bias != nullptr, bias[i + 1]);
+          o[i >> 1] = lo | (hi << 16);
+        }
+        *reinterpret_cast<u32x4*>(e.out + static_cast<int64_t>(m) * N + nn) = o;
+      }
+    }
+  }
+}
+
+// One thread per output element (consecutive threads, consecutive columns).
+template <int DT>
+__global__ __launch_bounds__(256) void llm_merge_kernel(const int32_t* __restrict__ acc, Epi e) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= static_cast<int64_t>(e.M) * e.N) return;
+  const int m = static_cast<int>(i / e.N);
+  const int n = static_cast<int>(i - static_cast<int64_t>(m) * e.N);
+  const float ws = e.wscale[n];
+  const int cnt = *e.count;
+  float sub = 0.0f;
+  for (int j = 0; j < cnt; ++j) {
+    const int kj = e.list[j];
+    const float wd = round_to_t<DT>(static_cast<float>(e.w[static_cast<int64_t>(n) * e.K + kj]) * ws);
+    sub += to_f32<DT>(e.x[static_cast<int64_t>(m) * e.K + kj]) * wd;
+  }
+  const float bias = e.bias != nullptr ? to_f32<DT>(e.bias[n]) : 0.0f;
+  e.out[i] = merge_one<DT>(acc[i], sub, e.ranges[m], ws, e.bias != nullptr, bias);
+}
+
+inline void allow_lds(const void* kern, size_t lds, std::atomic<uint32_t>& done) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+  const uint32_t bit = 1u << (dev & 31);
+  if (done.load(std::memory_order_acquire) & bit) return;
+  (void)hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+  done.fetch_or(bit, std::memory_order_release);
+}
+
+inline int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
+
+struct Plan {
+  int bm, bn;     // tile
+  int runs;       // K runs (1: the GEMM writes the output itself)
+  int tiles_per_run;
+};
+
+// Rows per tile follow M; K is cut into runs while the tiles alone leave CUs
+// idle and every run keeps at least four k tiles.
+Plan make_plan(int64_t M, int64_t K, int64_t N) {
+  Plan pl;
+  if (M > 128) {
+    pl.bm = 256;
+    pl.bn = 128;
+  } else {
+    pl.bm = M > 64 ? 128 : (M > 32 ? 64 : 32);
+    pl.bn = 256;
+  }
+  const int64_t tiles = ((M + pl.bm - 1) / pl.bm) * ((N + pl.bn - 1) / pl.bn);
+  const int64_t ktiles = K / kTK;
+  int64_t runs = 1;
+  if (M <= 128 && tiles < 256) {
+    runs = (512 + tiles - 1) / tiles;
+    if (runs > ktiles / 4) runs = ktiles / 4;
+    if (runs < 1) runs = 1;
+  }
+  int64_t per = (ktiles + runs - 1) / runs;
+  runs = (ktiles + per - 1) / per;
+  pl.runs = static_cast<int>(runs);
+  pl.tiles_per_run = static_cast<int>(per);
+  return pl;
+}
+
+struct Workspace {
+  float* ranges;
+  int32_t* mask;
+  int32_t* count;
+  int32_t* list;
+  int8_t* qx;
+  int32_t* acc;
+  int64_t bytes;
+};
+
+Workspace carve(void* base, int64_t M, int64_t K, int64_t N, bool with_acc) {
+  unsigned char* p = static_cast<unsigned char*>(base);
+  int64_t off = 0;
+  Workspace w;
+  w.ranges = reinterpret_cast<float*>(p + off);
+  off += align256(M * 4);
+  w.mask = reinterpret_cast<int32_t*>(p + off);
+  off += align256(K / 32 * 4);
+  w.count = reinterpret_cast<int32_t*>(p + off);
+  off += 256;
+  w.list = reinterpret_cast<int32_t*>(p + off);
+  off += align256(K * 4);
+  w.qx = reinterpret_cast<int8_t*>(p + off);
+  off += align256(M * K);
+  w.acc = reinterpret_cast<int32_t*>(p + off);
+  if (with_acc) off += align256(M * N * 4);
+  w.bytes = off;
+  return w;
+}
+
+template <int DT, int WM, int WN, int TM, int TN, bool RUNS>
+int launch_gemm(const GemmParams& p, int runs, hipStream_t stream) {
+  constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
+  constexpr size_t lds = static_cast<size_t>(kStages) * (BM + BN) * kTK;
+  static std::atomic<uint32_t> done{0};
+  auto kern = llm_gemm_kernel<DT, WM, WN, TM, TN, RUNS>;
+  allow_lds(reinterpret_cast<const void*>(kern), lds, done);
+  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(p.nbx * p.nby * runs)), dim3(WM * WN * 64), lds, stream,
+                     p);
+  return check_launch();
+}
+
+template <int DT, bool RUNS>
+int launch_gemm_for(const GemmParams& p, const Plan& pl, hipStream_t stream) {
+  switch (pl.bm) {
+    case 256:
+      if (RUNS) return WOL_ERR_BAD_SHAPE;  // make_plan cuts K only for tiles of at most 128 rows
+      return launch_gemm<DT, 2, 2, 4, 2, false>(p, pl.runs, stream);
+    case 128: return launch_gemm<DT, 1, 4, 4, 2, RUNS>(p, pl.runs, stream);
+    case 64: return launch_gemm<DT, 1, 4, 2, 2, RUNS>(p, pl.runs, stream);
+    default: return launch_gemm<DT, 1, 4, 1, 2, RUNS>(p, pl.runs, stream);
+  }
+}
+
+template <int DT>
+int run_llm_int8(const void* x, const void* weight, const void* bias, const float* wscale, float threshold,
+                 int64_t M, int64_t K, int64_t N, void* out, void* workspace, hipStream_t stream) {
+  const Plan pl = make_plan(M, K, N);
+  const Workspace ws = carve(workspace, M, K, N, pl.runs > 1);
+  const uint16_t* xs = static_cast<const uint16_t*>(x);
+  const int nwords = static_cast<int>(K / 32);
+  hipLaunchKernelGGL(llm_clear_kernel, dim3((nwords + 255) / 256), dim3(256), 0, stream, ws.mask, nwords,
+                     ws.count);
+  hipLaunchKernelGGL(llm_rowmax_kernel<DT>, dim3(static_cast<unsigned>(M)), dim3(256), 0, stream, xs, threshold,
+                     static_cast<int>(K), ws.ranges, ws.mask);
+  const int64_t nvec = M * K / 16;
+  int64_t qblocks = (nvec + 255) / 256;
+  if (qblocks > 8192) qblocks = 8192;
+  const int64_t acc_vec = pl.runs > 1 ? align256(M * N * 4) / 16 : 0;
+  hipLaunchKernelGGL(llm_quant_kernel<DT>, dim3(static_cast<unsigned>(qblocks + 1)), dim3(256), 0, stream, xs,
+                     ws.ranges, ws.mask, static_cast<int>(M), static_cast<int>(K), ws.qx, ws.count, ws.list,
+                     ws.acc, acc_vec);
+  GemmParams p;
+  p.qx = ws.qx;
+  p.e = Epi{xs, static_cast<const int8_t*>(weight), wscale, ws.ranges, static_cast<const uint16_t*>(bias),
+            ws.count, ws.list, static_cast<uint16_t*>(out), static_cast<int>(M), static_cast<int>(K),
+            static_cast<int>(N)};
+  p.acc = ws.acc;
+  p.nbx = static_cast<int>((N + pl.bn - 1) / pl.bn);
+  p.nby = static_cast<int>((M + pl.bm - 1) / pl.bm);
+  p.tiles_per_run = pl.tiles_per_run;
+  if (check_launch() != WOL_OK) return WOL_ERR_HIP;
+  if (pl.runs == 1) return launch_gemm_for<DT, false>(p, pl, stream);
+  const int rc = launch_gemm_for<DT, true>(p, pl, stream);
+  if (rc != WOL_OK) return rc;
+  const int64_t total = M * N;
+  hipLaunchKernelGGL(llm_merge_kernel<DT>, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, stream,
+                     ws.acc, p.e);
+  return check_launch();
+}
+
+}  // namespace
+
+size_t llm_int8_workspace(int64_t M, int64_t K, int64_t N) {
+  const Plan pl = make_plan(M, K, N);
+  return static_cast<size_t>(carve(nullptr, M, K, N, pl.runs > 1).bytes);
+}
+
+void llm_int8_workspace_offsets(int64_t M, int64_t K, int64_t N, int64_t* offsets) {
+  const Plan pl = make_plan(M, K, N);
+  const Workspace w = carve(nullptr, M, K, N, pl.runs > 1);
+  offsets[0] = reinterpret_cast<intptr_t>(w.ranges);
+  offsets[1] = reinterpret_cast<intptr_t>(w.mask);
+  offsets[2] = reinterpret_cast<intptr_t>(w.count);
+  offsets[3] = reinterpret_cast<intptr_t>(w.list);
+  offsets[4] = reinterpret_cast<intptr_t>(w.qx);
+  offsets[5] = pl.runs > 1 ? reinterpret_cast<intptr_t>(w.acc) : -1;
+}
+
+int launch_llm_int8_linear(const void* x, const void* weight, const void* bias, const float* wscale,
+                           float threshold, int dtype, int64_t M, int64_t K, int64_t N, void* out,
+                           void* workspace, hipStream_t stream) {
+  if (dtype == WOL_DTYPE_BF16)
+    return run_llm_int8<WOL_DTYPE_BF16>(x, weight, bias, wscale, threshold, M, K, N, out, workspace, stream);
+  return run_llm_int8<WOL_DTYPE_F16>(x, weight, bias, wscale, threshold, M, K, N, out, workspace, stream);
+}
+
+}  // namespace wol

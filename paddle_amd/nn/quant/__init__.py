@@ -2,9 +2,11 @@
 (python/paddle/nn/quant/__init__.py:28-42 in the reference)."""
 from .quantized_linear import (  # noqa: F401
     apply_per_channel_scale,
+    llm_int8_linear,
     weight_dequantize,
     weight_only_linear,
     weight_quantize,
 )
 
-__all__ = ["weight_only_linear", "weight_quantize", "weight_dequantize", "apply_per_channel_scale"]
+__all__ = ["weight_only_linear", "weight_quantize", "weight_dequantize", "apply_per_channel_scale",
+           "llm_int8_linear"]

@@ -427,3 +427,73 @@ def apply_per_channel_scale(x, scales):
             )
         )
     return out
+
+
+def llm_int8_linear_infer_meta(x_shape, w_shape, bias_shape, scale_shape):
+    """LLMInt8LinearInferMeta (paddle/phi/infermeta/multiary.cc:3792-3837):
+    returns the output shape."""
+    if len(w_shape) != 2:
+        raise ValueError("(InvalidArgument) The input(weight) must be a 2D Tensor.")
+    if x_shape[-1] != w_shape[1]:
+        raise ValueError(
+            "(InvalidArgument) Input(X) dim[-1] and Input(Weight) dim[1] should be equal."
+            "But received Input(X) dim[-1](%s) != Input(Weight) dim[1](%s)" % (x_shape[-1], w_shape[1])
+        )
+    if w_shape[0] % 16 != 0:
+        raise ValueError(
+            "(InvalidArgument) The first dimension of input must be divisible by 16, but got[%d]" % w_shape[0]
+        )
+    if w_shape[1] % 16 != 0:
+        raise ValueError(
+            "(InvalidArgument) The second dimension of input must be divisible by 16, but got[%d]" % w_shape[1]
+        )
+    if scale_shape[0] != w_shape[0]:
+        raise ValueError(
+            "(InvalidArgument) Input(weight_scale) dim[0] and Input(Weight) dim[0] should be equal."
+            "But received Input(weight_scale) dim[0](%s) != Input(Weight) dim[0](%s)" % (scale_shape[0], w_shape[0])
+        )
+    return tuple(x_shape[:-1]) + (w_shape[0],)
+
+
+def llm_int8_linear(x, weight, bias=None, weight_scale=None, threshold=6.0):
+    """paddle.nn.quant.llm_int8_linear (python/paddle/nn/quant/quantized_linear.py:285-349
+    in the reference): x [..., K] float16/bfloat16, weight [N, K] int8 and
+    weight_scale [N] float32 as weight_quantize(algo="llm.int8") returns them,
+    bias [N] in x's dtype or None.  Columns of x holding an element above
+    threshold are multiplied in x's dtype with the dequantised weight, the
+    rest as int8 x int8 with a per-row dynamic scale.  The weight must have K
+    divisible by 64 (what weight_quantize accepts), not only by 16."""
+    out_shape = llm_int8_linear_infer_meta(
+        tuple(x.shape), tuple(weight.shape), None if bias is None else tuple(bias.shape),
+        tuple(weight_scale.shape),
+    )
+    dt = _dtype_id(x, "x")
+    _require_gpu(x, "x")
+    if weight.dtype != torch.int8:
+        raise ValueError("(InvalidArgument) weight must be int8, but got %s" % weight.dtype)
+    if weight_scale.dtype != torch.float32:
+        raise ValueError("(InvalidArgument) weight_scale must be float32, but got %s" % weight_scale.dtype)
+    if bias is not None and bias.dtype != x.dtype:
+        raise ValueError("(InvalidArgument) bias must have x's dtype")
+    N, K = int(weight.shape[0]), int(weight.shape[1])
+    if bias is not None and int(bias.shape[0]) != N:
+        raise ValueError("(InvalidArgument) bias must have %d elements" % N)
+    x = x.contiguous()
+    weight = weight.contiguous()
+    weight_scale = weight_scale.contiguous()
+    bias = None if bias is None else bias.contiguous()
+    M = x.numel() // K
+    out = torch.empty(out_shape, dtype=x.dtype, device=x.device)
+    if M == 0:
+        return out
+    ws_bytes = _lib.lib.wol_llm_int8_linear_workspace(M, K, N)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(
+            _lib.lib.wol_llm_int8_linear(
+                x.data_ptr(), weight.data_ptr(), None if bias is None else bias.data_ptr(),
+                weight_scale.data_ptr(), float(threshold), dt, M, K, N, out.data_ptr(), ws.data_ptr(),
+                ws_bytes, _stream_ptr(x),
+            )
+        )
+    return out

@@ -85,3 +85,40 @@ def linear(x_bits, codes_u8, bias_bits, scale_bits, dt, N, bits, g, f32=False, n
         _lib.check(_lib.lib.wol_linear_on(*args, 1 if f32 else 0, kernel, *tail))
     torch.cuda.synchronize()
     return out.cpu().numpy() if f32 else H.torch_to_bits(out)
+
+
+def llm_int8_linear(x_bits, w_nk, bias_bits, wscale, threshold, dt, stages=False):
+    """wol_llm_int8_linear through the C ABI.  w_nk [N,K] int8, wscale [N] float32.
+    Returns the output's T bits, and with stages=True also a dict of the
+    intermediate results left in the workspace."""
+    import ctypes
+
+    x = H.bits_to_torch(x_bits, dt, DEV)
+    M, K = x.shape
+    w = torch.from_numpy(np.ascontiguousarray(w_nk, dtype=np.int8)).to(DEV)
+    N = w.shape[0]
+    s = torch.from_numpy(np.ascontiguousarray(wscale, dtype=np.float32)).to(DEV)
+    b = None if bias_bits is None else H.bits_to_torch(bias_bits, dt, DEV)
+    out = torch.full((M, N), float("nan"), dtype=x.dtype, device=DEV)
+    wsb = _lib.lib.wol_llm_int8_linear_workspace(M, K, N)
+    ws = torch.full((wsb,), 0xA5, dtype=torch.uint8, device=DEV)  # dirty on purpose
+    _lib.check(_lib.lib.wol_llm_int8_linear(x.data_ptr(), w.data_ptr(), None if b is None else b.data_ptr(),
+                                            s.data_ptr(), float(threshold), dt, M, K, N, out.data_ptr(),
+                                            ws.data_ptr(), wsb, None))
+    torch.cuda.synchronize()
+    if not stages:
+        return H.torch_to_bits(out)
+    offs = (ctypes.c_int64 * 6)()
+    _lib.check(_lib.lib.wol_llm_int8_linear_stage_offsets(M, K, N, offs))
+    raw = ws.cpu().numpy()
+    count = int(raw[offs[2]:offs[2] + 4].view(np.int32)[0])
+    mask_words = raw[offs[1]:offs[1] + K // 32 * 4].view(np.uint32)
+    st = {
+        "ranges": raw[offs[0]:offs[0] + 4 * M].view(np.float32).copy(),
+        "outlier": ((mask_words[:, None] >> np.arange(32, dtype=np.uint32)[None, :]) & 1).astype(bool).reshape(-1),
+        "count": count,
+        "list": raw[offs[3]:offs[3] + 4 * count].view(np.int32).copy(),
+        "qx": raw[offs[4]:offs[4] + M * K].view(np.int8).reshape(M, K).copy(),
+        "acc": None if offs[5] < 0 else raw[offs[5]:offs[5] + 4 * M * N].view(np.int32).reshape(M, N).copy(),
+    }
+    return H.torch_to_bits(out), st
