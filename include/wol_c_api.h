@@ -242,8 +242,8 @@ int wol_apply_per_channel_scale(const void* x, const void* scales, int dtype,
  * Requires K % 64 == 0 and N % 16 == 0 (what weight_quantize accepts); x,
  * weight, weight_scale, out and workspace 16-byte aligned.  The workspace is
  * required (wol_llm_int8_linear_workspace bytes); it holds the row ranges,
- * the outlier mask and list, the activation codes and, for few rows, int32
- * sums.  Nothing returns to the host: the reference's device-to-host copy of
+ * the outlier mask and list, the activation codes and, for few rows, the int32
+ * sums of the runs K is cut into.  Nothing returns to the host: the reference's device-to-host copy of
  * the outlier count has no counterpart here.
  */
 size_t wol_llm_int8_linear_workspace(int64_t M, int64_t K, int64_t N);
@@ -256,8 +256,10 @@ int wol_llm_int8_linear(const void* x, const void* weight, const void* bias,
  * after a call, as byte offsets: [0] range (float [M]), [1] outlier mask
  * (bit k % 32 of int32 word k / 32), [2] outlier count (int32), [3] outlier
  * columns (int32, ascending), [4] activation codes (int8 [M,K]), [5] int32
- * sums [M,N] or -1 when the GEMM writes the output itself.  For tests that
- * compare the stages with the reference's; no counterpart there. */
+ * sums, one [M,N] slab per K run, or -1 when the GEMM writes the output
+ * itself; [6] is the number of K runs (not an offset).  offsets has room for
+ * seven values.  For tests that compare the stages with the reference's; no
+ * counterpart there. */
 int wol_llm_int8_linear_stage_offsets(int64_t M, int64_t K, int64_t N,
                                       int64_t* offsets);
 

@@ -223,7 +223,8 @@ int launch_llm_int8_linear(const void* x, const void* weight, const void* bias, 
                            void* workspace, hipStream_t stream);
 // Scratch bytes launch_llm_int8_linear needs, and where its stages lie in them
 // (ranges, outlier mask, outlier count, outlier list, activation codes, int32
-// sums or -1 when the GEMM writes the output itself).
+// sums of the K runs or -1 when the GEMM writes the output itself, number of
+// K runs: seven values).
 size_t llm_int8_workspace(int64_t M, int64_t K, int64_t N);
 void llm_int8_workspace_offsets(int64_t M, int64_t K, int64_t N, int64_t* offsets);
 // Scratch bytes with which launch_linear_gemm splits K across workgroups (0: none needed).

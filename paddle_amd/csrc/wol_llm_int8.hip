@@ -13,14 +13,16 @@
 //   quant   : qx = 0 in outlier columns, else clip(round(x * 127 * (1/range)))
 //             (QuantActKernel :270-303, QuantFunc :153-164); one extra
 //             workgroup turns the mask into an ascending list of columns
+//   outlier : sub = T(sum over the outlier columns of x * T(w * wscale)), fp32
+//             sum in ascending column order; leaves at once without outliers
 //   gemm    : acc = qx . w^T in int32 on v_mfma_i32_32x32x32_i8, both operands
-//             through direct-to-LDS loads, three k tiles deep.  The epilogue is
-//             DequantMergeKernel (:415-447) with the outlier product folded in:
-//             out = T( T(sum_outliers x * T(w * wscale)) + T(acc * range *
-//             wscale / 127) ), then T(out + bias).
-//   merge   : only when K is cut into runs (few rows): the runs add their int32
-//             sums with integer atomics (exact, so order does not matter) and
-//             this kernel applies the same epilogue.
+//             through direct-to-LDS loads, two or three k tiles deep.  The
+//             epilogue is DequantMergeKernel (:415-447): out = T( sub + T(acc *
+//             range * wscale / 127) ), then T(out + bias).
+//   merge   : only when K is cut into runs (few rows): every run leaves its
+//             int32 sums in a slab of its own and this kernel adds them (exact,
+//             so the result does not depend on the cut) and applies the same
+//             epilogue.
 #include <atomic>
 
 #include "wol_common.h"
@@ -34,22 +36,6 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
-constexpr int kTK = 64;      // k (bytes) per tile row
-constexpr int kStages = 3;
-
-// float -> T, round to nearest even, of exactly the fp32 value given: the
-// barrier keeps the compiler from merging the producing multiply or add with
-// the conversion into one instruction that rounds once.
-template <int DT>
-__device__ inline uint16_t cast_exact(float f) {
-  asm volatile("" : "+v"(f));
-  return from_f32_rne<DT>(f);
-}
-
-template <int DT>
-__device__ inline float round_to_t(float f) {
-  return to_f32<DT>(cast_exact<DT>(f));
-}
 
 template <int N_>
 __device__ inline void wait_vmcnt() {
@@ -66,40 +52,63 @@ __global__ __launch_bounds__(256) void llm_clear_kernel(int32_t* mask, int nword
   if (i == 0) *count = 0;
 }
 
+// A workgroup takes kRowsPerGroup rows and a thread the same columns of each,
+// so that a column's outlier bits are ORed over the rows in registers and
+// reach the mask as one atomic per workgroup (outlier columns tend to be the
+// same in every row).
+constexpr int kRowsPerGroup = 8;
+
 template <int DT>
-__global__ __launch_bounds__(256) void llm_rowmax_kernel(const uint16_t* __restrict__ x, float threshold,
+__global__ __launch_bounds__(256) void llm_rowmax_kernel(const uint16_t* __restrict__ x, float threshold, int M,
                                                          int K, float* __restrict__ ranges,
-                                                         int32_t* __restrict__ mask) {
-  __shared__ float part[4];
+                                                         int32_t* mask) {
+  __shared__ float part[4][kRowsPerGroup];
   const float thr = to_f32<DT>(from_f32_rne<DT>(threshold));  // the comparison is made in T
-  const uint16_t* row = x + static_cast<int64_t>(blockIdx.x) * K;
-  float mx = 0.0f;
+  const int m0 = blockIdx.x * kRowsPerGroup;
+  float mx[kRowsPerGroup];
+#pragma unroll
+  for (int r = 0; r < kRowsPerGroup; ++r) mx[r] = 0.0f;
   for (int k0 = threadIdx.x * 8; k0 < K; k0 += 256 * 8) {
-    const u32x4 v = *reinterpret_cast<const u32x4*>(row + k0);
+    u32x4 v[kRowsPerGroup];
+#pragma unroll
+    for (int r = 0; r < kRowsPerGroup; ++r) {
+      const int m = m0 + r < M ? m0 + r : M - 1;  // past the end: the last row again
+      v[r] = *reinterpret_cast<const u32x4*>(x + static_cast<int64_t>(m) * K + k0);
+    }
     uint32_t bits = 0;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      float a = fabsf(to_f32<DT>(static_cast<uint16_t>(v[i >> 1] >> (16 * (i & 1)))));
-      if (a > thr) {
-        bits |= 1u << i;
-        a = 0.0f;
+    for (int r = 0; r < kRowsPerGroup; ++r) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        float a = fabsf(to_f32<DT>(static_cast<uint16_t>(v[r][i >> 1] >> (16 * (i & 1)))));
+        if (a > thr) {
+          bits |= 1u << i;
+          a = 0.0f;
+        }
+        mx[r] = a > mx[r] ? a : mx[r];
       }
-      mx = a > mx ? a : mx;
     }
-    if (bits != 0) atomicOr(&mask[k0 >> 5], static_cast<int32_t>(bits << (k0 & 31)));
+    if (bits != 0) {
+      // skip the atomic where the bits are already set (a stale read only costs an atomic)
+      const int32_t want = static_cast<int32_t>(bits << (k0 & 31));
+      if ((__builtin_nontemporal_load(&mask[k0 >> 5]) & want) != want) atomicOr(&mask[k0 >> 5], want);
+    }
   }
 #pragma unroll
-  for (int d = 32; d > 0; d >>= 1) {
-    const float o = __shfl_xor(mx, d, 64);
-    mx = o > mx ? o : mx;
+  for (int r = 0; r < kRowsPerGroup; ++r) {
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) {
+      const float o = __shfl_xor(mx[r], d, 64);
+      mx[r] = o > mx[r] ? o : mx[r];
+    }
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6][r] = mx[r];
   }
-  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = mx;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    float r = part[0];
+  if (threadIdx.x < kRowsPerGroup && m0 + threadIdx.x < M) {
+    float r = part[0][threadIdx.x];
 #pragma unroll
-    for (int i = 1; i < 4; ++i) r = part[i] > r ? part[i] : r;
-    ranges[blockIdx.x] = r;
+    for (int i = 1; i < 4; ++i) r = part[i][threadIdx.x] > r ? part[i][threadIdx.x] : r;
+    ranges[m0 + threadIdx.x] = r;
   }
 }
 
@@ -117,8 +126,7 @@ __global__ __launch_bounds__(256) void llm_quant_kernel(const uint16_t* __restri
                                                         const float* __restrict__ ranges,
                                                         const int32_t* __restrict__ mask, int M, int K,
                                                         int8_t* __restrict__ qx, int32_t* __restrict__ count,
-                                                        int32_t* __restrict__ list, int32_t* __restrict__ acc,
-                                                        int64_t acc_vec) {
+                                                        int32_t* __restrict__ list) {
   const int tid = threadIdx.x;
   if (blockIdx.x == gridDim.x - 1) {
     // the mask as an ascending list of outlier columns
@@ -173,8 +181,6 @@ __global__ __launch_bounds__(256) void llm_quant_kernel(const uint16_t* __restri
     }
     *reinterpret_cast<u32x4*>(qx + e) = q;
   }
-  const u32x4 zero = {0u, 0u, 0u, 0u};
-  for (int64_t i = first; i < acc_vec; i += stride) reinterpret_cast<u32x4*>(acc)[i] = zero;
 }
 
 // ---------------------------------------------------------------------------
@@ -188,16 +194,157 @@ struct Epi {
   const uint16_t* bias;   // [N] T or null
   const int32_t* count;
   const int32_t* list;
+  const uint16_t* sub;    // [M,N] T: the outlier columns' product, valid when *count > 0
   uint16_t* out;          // [M,N] T
   int M, K, N;
 };
 
-// DequantFunc (:172-176) and the two T additions that follow it.
+// v / 127, correctly rounded, in four instructions instead of the dozen of the
+// IEEE division sequence: q = v * RN(1/127), r = v - 127 q (exact in an FMA),
+// q + r * RN(1/127).  Equal to the division for every one of the 2^32 float
+// inputs (checked exhaustively on a CPU with hardware FMA); q itself is the
+// answer where r is zero or NaN (v = -0, infinities).
+__device__ inline float div127(float v) {
+  const float y = 1.0f / 127.0f;
+  const float q = v * y;
+  const float r = __builtin_fmaf(-q, 127.0f, v);
+  const float q2 = __builtin_fmaf(r, y, q);
+  return (r != 0.0f && r == r) ? q2 : q;
+}
+
+// DequantFunc (:172-176) and the two T additions that follow it.  The casts
+// are the hardware's round-to-nearest-even conversions (the payload of a NaN
+// result is unspecified).
 template <int DT>
 __device__ inline uint16_t merge_one(int acc, float sub, float range, float ws, bool has_bias, float bias) {
-  const float dq = round_to_t<DT>(static_cast<float>(acc) * range * ws / 127.0f);
-  const float o = round_to_t<DT>(round_to_t<DT>(sub) + dq);
-  return has_bias ? cast_exact<DT>(o + bias) : cast_exact<DT>(o);
+  const float dq = to_f32<DT>(cast_out<DT>(div127(static_cast<float>(acc) * range * ws)));
+  const float o = to_f32<DT>(cast_out<DT>(sub + dq));  // sub is a T value
+  return has_bias ? cast_out<DT>(o + bias) : cast_out<DT>(o);
+}
+
+// The same without outlier columns (sub = +0): T(0 + dq) is dq, -0 becoming +0.
+template <int DT>
+__device__ inline uint16_t merge_plain(int acc, float range, float ws, bool has_bias, float bias) {
+  const uint16_t dq = cast_out<DT>(div127(static_cast<float>(acc) * range * ws));
+  if (!has_bias) return dq == 0x8000u ? static_cast<uint16_t>(0) : dq;
+  return cast_out<DT>(to_f32<DT>(dq) + 0.0f + bias);
+}
+
+// Eight neighbouring columns nn .. nn+7 of row m: the merge with the outlier
+// columns' product (when there are any: out of LDS if xs is given, else as
+// the outlier kernel left it in e.sub) and one 16-byte store.  ws and bias hold the eight columns' values.
+template <int DT>
+__device__ inline void finish8(const Epi& e, int cnt, int m, int nn, i32x4 s0, i32x4 s1, const float* ws,
+                               const float* bias, const float* xs, int xs_stride, const float* wd,
+                               int wd_stride) {
+  const float range = e.ranges[m];
+  u32x4 o;
+  if (cnt == 0) {  // uniform: the count is one value for the whole launch
+#pragma unroll
+    for (int i = 0; i < 8; i += 2) {
+      const uint32_t lo = merge_plain<DT>(i < 4 ? s0[i] : s1[i - 4], range, ws[i], e.bias != nullptr, bias[i]);
+      const uint32_t hi =
+          merge_plain<DT>(i < 4 ? s0[i + 1] : s1[i - 3], range, ws[i + 1], e.bias != nullptr, bias[i + 1]);
+      o[i >> 1] = lo | (hi << 16);
+    }
+    *reinterpret_cast<u32x4*>(e.out + static_cast<int64_t>(m) * e.N + nn) = o;
+    return;
+  }
+  float sub[8];
+  if (xs != nullptr) {
+    // the workgroup holds this row's activations and these columns' dequantised
+    // weights of every outlier column in LDS (xs[j * xs_stride], wd[j * wd_stride + i])
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sub[i] = 0.0f;
+#pragma unroll 1
+    for (int j = 0; j < cnt; ++j) {
+      const float xv = xs[j * xs_stride];
+      const f32x4 w0 = *reinterpret_cast<const f32x4*>(wd + j * wd_stride);
+      const f32x4 w1 = *reinterpret_cast<const f32x4*>(wd + j * wd_stride + 4);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        sub[i] += xv * w0[i];
+        sub[4 + i] += xv * w1[i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sub[i] = to_f32<DT>(cast_out<DT>(sub[i]));
+  } else {
+    const u32x4 sv = *reinterpret_cast<const u32x4*>(e.sub + static_cast<int64_t>(m) * e.N + nn);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sub[i] = to_f32<DT>(static_cast<uint16_t>(sv[i >> 1] >> (16 * (i & 1))));
+  }
+#pragma unroll
+  for (int i = 0; i < 8; i += 2) {
+    const uint32_t lo = merge_one<DT>(i < 4 ? s0[i] : s1[i - 4], sub[i], range, ws[i], e.bias != nullptr, bias[i]);
+    const uint32_t hi =
+        merge_one<DT>(i < 4 ? s0[i + 1] : s1[i - 3], sub[i + 1], range, ws[i + 1], e.bias != nullptr, bias[i + 1]);
+    o[i >> 1] = lo | (hi << 16);
+  }
+  *reinterpret_cast<u32x4*>(e.out + static_cast<int64_t>(m) * e.N + nn) = o;
+}
+
+// The eight columns' scales and biases.
+template <int DT>
+__device__ inline void load_ws_bias8(const Epi& e, int nn, float* ws, float* bias) {
+  const f32x4 w0 = *reinterpret_cast<const f32x4*>(e.wscale + nn);
+  const f32x4 w1 = *reinterpret_cast<const f32x4*>(e.wscale + nn + 4);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    ws[i] = w0[i];
+    ws[4 + i] = w1[i];
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) bias[i] = e.bias != nullptr ? to_f32<DT>(e.bias[nn + i]) : 0.0f;
+}
+
+// sub[m,n] = T( sum over the outlier columns k, ascending, of x[m,k] * T(w[n,k] *
+// wscale[n]) ), fp32 sum: what the reference computes with SplitKernel and a
+// library GEMM (:305-362, :593-640).  A workgroup takes 64 rows x 256 columns,
+// a thread one column of them; the rows' activations of 32 outlier columns at
+// a time wait in LDS.  Workgroups leave at once when there is no outlier or
+// the GEMM's epilogue computes the product itself (up to fused_cap columns).
+template <int DT>
+__global__ __launch_bounds__(256) void llm_outlier_kernel(Epi e, uint16_t* __restrict__ sub, int fused_cap) {
+  const int cnt = *e.count;
+  if (cnt <= fused_cap) return;  // none, or few enough for the GEMM's epilogue to take them
+  __shared__ __attribute__((aligned(16))) float xs[32][64];
+  const int tid = threadIdx.x;
+  const int nbx = (e.N + 255) / 256;
+  const int m0 = static_cast<int>(blockIdx.x / nbx) * 64;
+  const int n = static_cast<int>(blockIdx.x % nbx) * 256 + tid;
+  const int nn = n < e.N ? n : e.N - 1;
+  const float ws = e.wscale[nn];
+  const int8_t* wrow = e.w + static_cast<int64_t>(nn) * e.K;
+  float acc[64];
+#pragma unroll
+  for (int r = 0; r < 64; ++r) acc[r] = 0.0f;
+  for (int j0 = 0; j0 < cnt; j0 += 32) {
+    __syncthreads();
+    for (int i = tid; i < 64 * 32; i += 256) {
+      const int r = i & 63, c = i >> 6;
+      int m = m0 + r;
+      m = m < e.M ? m : e.M - 1;
+      xs[c][r] = j0 + c < cnt ? to_f32<DT>(e.x[static_cast<int64_t>(m) * e.K + e.list[j0 + c]]) : 0.0f;
+    }
+    __syncthreads();
+    const int cn = cnt - j0 < 32 ? cnt - j0 : 32;
+#pragma unroll 1
+    for (int c = 0; c < cn; ++c) {
+      const float wd = to_f32<DT>(cast_out<DT>(static_cast<float>(wrow[e.list[j0 + c]]) * ws));
+#pragma unroll
+      for (int r = 0; r < 64; r += 4) {
+        const f32x4 xv = *reinterpret_cast<const f32x4*>(&xs[c][r]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[r + i] += xv[i] * wd;
+      }
+    }
+  }
+  if (n < e.N) {
+#pragma unroll
+    for (int r = 0; r < 64; ++r)
+      if (m0 + r < e.M) sub[static_cast<int64_t>(m0 + r) * e.N + n] = cast_out<DT>(acc[r]);
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -206,24 +353,30 @@ __device__ inline uint16_t merge_one(int acc, float sub, float range, float ws, 
 struct GemmParams {
   const int8_t* qx;  // [M,K]
   Epi e;
-  int32_t* acc;      // [M,N] int32, zeroed; only with K runs
+  int32_t* acc;      // [runs][M,N] int32, one slab per K run; only with K runs
   int nbx, nby;      // tiles along N and M
   int tiles_per_run; // k tiles per K run
+  int cap;  // outlier columns the epilogue takes through LDS itself; more come from e.sub
 };
 
-// XOR applied to the 16-byte piece index (four per 64-byte row) so that the
-// 16 rows a quarter of a wavefront reads hit distinct LDS banks, whether the
-// LDS serves 8 or 16 lanes of a 128-bit read per cycle.
+// XOR applied to the 16-byte piece index of a row in LDS (C pieces per row) so
+// that the 16 rows a quarter of a wavefront reads hit distinct LDS banks,
+// whether the LDS serves 8 or 16 lanes of a 128-bit read per cycle.
+template <int C>
 __device__ inline int row_swizzle(int row) {
-  return ((((row >> 1) ^ (row >> 3)) & 1) << 1) | ((row >> 2) & 1);
+  if (C == 8) return (row & 7) ^ ((row >> 3) & 1);                             // 128-byte rows
+  return ((((row >> 1) ^ (row >> 3)) & 1) << 1) | ((row >> 2) & 1);            // 64-byte rows
 }
 
-// WM x WN wavefronts, each TM x TN blocks of 32x32.  RUNS: K is cut into runs
-// across workgroups, which add into acc; otherwise the epilogue writes out.
-template <int DT, int WM, int WN, int TM, int TN, bool RUNS>
+// WM x WN wavefronts, each TM x TN blocks of 32x32; k tiles of TK bytes per row
+// (128: whole cache lines per row and load; 64 for a K that is not a multiple
+// of 128), STAGES of them in LDS.  RUNS: K is cut into runs across workgroups,
+// each leaving its sums in its slab of acc; otherwise the epilogue writes out.
+template <int DT, int WM, int WN, int TM, int TN, int TK, int STAGES, bool RUNS>
 __global__ __launch_bounds__(WM* WN * 64) __attribute__((amdgpu_waves_per_eu(2))) void llm_gemm_kernel(GemmParams p) {
   constexpr int NW = WM * WN;
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
+  constexpr int kTK = TK, kStages = STAGES, C = TK / 16;  // C: 16-byte pieces per row
   constexpr int kABytes = BM * kTK, kBBytes = BN * kTK, kStage = kABytes + kBBytes;
   constexpr int kABlocks = kABytes / 1024, kBBlocks = kBBytes / 1024;  // 1 KiB = one wavefront load
   constexpr int kALoads = (kABlocks + NW - 1) / NW, kBLoads = (kBBlocks + NW - 1) / NW;
@@ -257,7 +410,7 @@ __global__ __launch_bounds__(WM* WN * 64) __attribute__((amdgpu_waves_per_eu(2))
   const int niter = (ktiles - t0) < p.tiles_per_run ? (ktiles - t0) : p.tiles_per_run;
 
   // global sources of this lane's direct-to-LDS loads.  LDS piece q (16 bytes)
-  // of a tile region is row q / 4, slot q % 4, and holds the row's logical
+  // of a tile region is row q / C, slot q % C, and holds the row's logical
   // piece slot ^ swizzle(row).  Rows past M or N repeat the last valid row:
   // computed on valid data, never stored.  Where a region has fewer 1 KiB
   // blocks than there are wavefronts, some blocks are loaded twice.
@@ -270,7 +423,7 @@ __global__ __launch_bounds__(WM* WN * 64) __attribute__((amdgpu_waves_per_eu(2))
   for (int c = 0; c < kALoads; ++c) {
     ablk[c] = (c * NW + wave) % kABlocks;
     const int q = ablk[c] * 64 + lane;
-    const int row = q >> 2, cc = (q & 3) ^ row_swizzle(row);
+    const int row = q / C, cc = (q % C) ^ row_swizzle<C>(row);
     int m = m0 + row;
     m = m < M ? m : M - 1;
     asrc[c] = reinterpret_cast<const uint8_t*>(p.qx) + static_cast<int64_t>(m) * K + static_cast<int64_t>(t0) * kTK + cc * 16;
@@ -281,7 +434,7 @@ __global__ __launch_bounds__(WM* WN * 64) __attribute__((amdgpu_waves_per_eu(2))
   for (int c = 0; c < kBLoads; ++c) {
     bblk[c] = (c * NW + wave) % kBBlocks;
     const int q = bblk[c] * 64 + lane;
-    const int row = q >> 2, cc = (q & 3) ^ row_swizzle(row);
+    const int row = q / C, cc = (q % C) ^ row_swizzle<C>(row);
     int n = n0 + row;
     n = n < N ? n : N - 1;
     bsrc[c] = reinterpret_cast<const uint8_t*>(p.e.w) + static_cast<int64_t>(n) * K + static_cast<int64_t>(t0) * kTK + cc * 16;
@@ -310,7 +463,7 @@ __global__ __launch_bounds__(WM* WN * 64) __attribute__((amdgpu_waves_per_eu(2))
 
   // byte offsets of this lane's fragments inside a stage, for k step 0; k step
   // 1 is the same with the piece index XOR 2
-  const int swz = row_swizzle(r32);  // rows are 32 * block + r32: the swizzle has period 16
+  const int swz = row_swizzle<C>(r32);  // rows are 32 * block + r32: the swizzle has period 16
   int aoff[TM], boff[TN];
 #pragma unroll
   for (int a = 0; a < TM; ++a) aoff[a] = ((wm * TM + a) * 32 + r32) * kTK;
@@ -318,14 +471,17 @@ __global__ __launch_bounds__(WM* WN * 64) __attribute__((amdgpu_waves_per_eu(2))
   for (int c = 0; c < TN; ++c) boff[c] = kABytes + ((wn * TN + c) * 32 + r32) * kTK;
 
   WOL_LLM_ISSUE(0);
-  WOL_LLM_ISSUE(1);
+  if (kStages == 3) WOL_LLM_ISSUE(1);
   for (int it = 0; it < niter; ++it) {
-    wait_vmcnt<kPerStage>();  // loads complete in order: all but the newest stage have landed
-    __syncthreads();
-    WOL_LLM_ISSUE(it + 2);  // into the stage every wavefront finished reading before the barrier
+    // loads complete in order: all but the newest stage have landed.  A bare
+    // s_barrier, not __syncthreads(): the fence of the latter makes the
+    // compiler wait for every load in flight, the prefetched tile included.
+    wait_vmcnt<(kStages - 2) * kPerStage>();
+    __builtin_amdgcn_s_barrier();
+    WOL_LLM_ISSUE(it + kStages - 1);  // into the stage every wavefront finished reading before the barrier
     const unsigned char* stage = smem + (it % kStages) * kStage;
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
+    for (int ks = 0; ks < C / 2; ++ks) {
       const int piece = ((ks * 2 + b) ^ swz) * 16;
       i32x4 af[TM], bf[TN];
 #pragma unroll
@@ -355,23 +511,33 @@ __global__ __launch_bounds__(WM* WN * 64) __attribute__((amdgpu_waves_per_eu(2))
   int* slab = reinterpret_cast<int*>(smem) + wave * (32 * kSlabRow);
   const int cnt = RUNS ? 0 : *e.count;
   const int cgrp = (lane & 3) * 8;  // first of this lane's eight columns inside the block
+  // few outlier columns: their activations (this tile's rows) and dequantised
+  // weights (this tile's columns) go to LDS behind the slabs, as floats
+  float* xs = reinterpret_cast<float*>(smem + NW * 32 * kSlabRow * 4);  // [cnt][BM]
+  float* wdl = xs + p.cap * BM;                                         // [cnt][BN]
+  const bool fused = !RUNS && cnt > 0 && cnt <= p.cap;
+  if (fused) {
+    for (int i = tid; i < cnt * BM; i += NW * 64) {
+      const int j = i / BM;
+      int m = m0 + i % BM;
+      m = m < M ? m : M - 1;
+      xs[i] = to_f32<DT>(e.x[static_cast<int64_t>(m) * K + e.list[j]]);
+    }
+    for (int i = tid; i < cnt * BN; i += NW * 64) {
+      const int j = i / BN;
+      int n = n0 + i % BN;
+      n = n < N ? n : N - 1;
+      wdl[i] = to_f32<DT>(cast_out<DT>(static_cast<float>(e.w[static_cast<int64_t>(n) * K + e.list[j]]) * e.wscale[n]));
+    }
+    __syncthreads();
+  }
 #pragma unroll
   for (int c = 0; c < TN; ++c) {
     const int n = n0 + (wn * TN + c) * 32 + cgrp;
     const bool n_ok = n < N;  // N is a multiple of 16: eight columns are all inside or all outside
     const int nn = n_ok ? n : 0;
     float ws[8], bias[8];
-    if (!RUNS) {
-      const f32x4 w0 = *reinterpret_cast<const f32x4*>(e.wscale + nn);
-      const f32x4 w1 = *reinterpret_cast<const f32x4*>(e.wscale + nn + 4);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        ws[i] = w0[i];
-        ws[4 + i] = w1[i];
-      }
-#pragma unroll
-      for (int i = 0; i < 8; ++i) bias[i] = e.bias != nullptr ? to_f32<DT>(e.bias[nn + i]) : 0.0f;
-    }
+    if (!RUNS) load_ws_bias8<DT>(e, nn, ws, bias);
 #pragma unroll
     for (int a = 0; a < TM; ++a) {
       __builtin_amdgcn_wave_barrier();  // the rows of the previous block have been read
@@ -387,62 +553,37 @@ __global__ __launch_bounds__(WM* WN * 64) __attribute__((amdgpu_waves_per_eu(2))
         if (m >= M || !n_ok) continue;
         const i32x4 s0 = *reinterpret_cast<const i32x4*>(slab + row * kSlabRow + cgrp);
         const i32x4 s1 = *reinterpret_cast<const i32x4*>(slab + row * kSlabRow + cgrp + 4);
-        if (RUNS) {
-          int32_t* dst = p.acc + static_cast<int64_t>(m) * N + nn;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            atomicAdd(dst + i, s0[i]);
-            atomicAdd(dst + 4 + i, s1[i]);
-          }
+        if (RUNS) {  // this run's sums, to be added by the merge kernel
+          int32_t* dst = p.acc + (static_cast<int64_t>(run) * M + m) * N + nn;
+          *reinterpret_cast<i32x4*>(dst) = s0;
+          *reinterpret_cast<i32x4*>(dst + 4) = s1;
           continue;
         }
-        float sub[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) sub[i] = 0.0f;
-#pragma unroll 1
-        for (int j = 0; j < cnt; ++j) {
-          const int kj = e.list[j];
-          const float xv = to_f32<DT>(e.x[static_cast<int64_t>(m) * K + kj]);
-#pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            const float wd =
-                round_to_t<DT>(static_cast<float>(e.w[static_cast<int64_t>(nn + i) * K + kj]) * ws[i]);
-            sub[i] += xv * wd;
-          }
-        }
-        const float range = e.ranges[m];
-        u32x4 o;
-#pragma unroll
-        for (int i = 0; i < 8; i += 2) {
-          const uint32_t lo =
-              merge_one<DT>(i < 4 ? s0[i] : s1[i - 4], sub[i], range, ws[i], e.bias != nullptr, bias[i]);
-          const uint32_t hi = merge_one<DT>(i < 4 ? s0[i + 1] : s1[i - 3], sub[i + 1], range, ws[i + 1],
-                                            e.bias != nullptr, bias[i + 1]);
-          o[i >> 1] = lo | (hi << 16);
-        }
-        *reinterpret_cast<u32x4*>(e.out + static_cast<int64_t>(m) * N + nn) = o;
+        finish8<DT>(e, cnt, m, nn, s0, s1, ws, bias, fused ? xs + (wm * TM + a) * 32 + row : nullptr, BM,
+                    wdl + (wn * TN + c) * 32 + cgrp, BN);
       }
     }
   }
 }
 
-// One thread per output element (consecutive threads, consecutive columns).
+// Adds the K runs' int32 sums and finishes; one thread per eight columns.
 template <int DT>
-__global__ __launch_bounds__(256) void llm_merge_kernel(const int32_t* __restrict__ acc, Epi e) {
+__global__ __launch_bounds__(256) void llm_merge_kernel(const int32_t* __restrict__ acc, int runs, Epi e) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  if (i >= static_cast<int64_t>(e.M) * e.N) return;
-  const int m = static_cast<int>(i / e.N);
-  const int n = static_cast<int>(i - static_cast<int64_t>(m) * e.N);
-  const float ws = e.wscale[n];
-  const int cnt = *e.count;
-  float sub = 0.0f;
-  for (int j = 0; j < cnt; ++j) {
-    const int kj = e.list[j];
-    const float wd = round_to_t<DT>(static_cast<float>(e.w[static_cast<int64_t>(n) * e.K + kj]) * ws);
-    sub += to_f32<DT>(e.x[static_cast<int64_t>(m) * e.K + kj]) * wd;
+  const int groups = e.N / 8;
+  if (i >= static_cast<int64_t>(e.M) * groups) return;
+  const int m = static_cast<int>(i / groups);
+  const int nn = static_cast<int>(i - static_cast<int64_t>(m) * groups) * 8;
+  const int64_t slab = static_cast<int64_t>(e.M) * e.N;
+  const int32_t* src = acc + static_cast<int64_t>(m) * e.N + nn;
+  i32x4 s0 = {0, 0, 0, 0}, s1 = {0, 0, 0, 0};
+  for (int r = 0; r < runs; ++r) {
+    s0 += *reinterpret_cast<const i32x4*>(src + r * slab);
+    s1 += *reinterpret_cast<const i32x4*>(src + r * slab + 4);
   }
-  const float bias = e.bias != nullptr ? to_f32<DT>(e.bias[n]) : 0.0f;
-  e.out[i] = merge_one<DT>(acc[i], sub, e.ranges[m], ws, e.bias != nullptr, bias);
+  float ws[8], bias[8];
+  load_ws_bias8<DT>(e, nn, ws, bias);
+  finish8<DT>(e, *e.count, m, nn, s0, s1, ws, bias, nullptr, 0, nullptr, 0);
 }
 
 inline void allow_lds(const void* kern, size_t lds, std::atomic<uint32_t>& done) {
@@ -458,31 +599,49 @@ inline int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
 
 struct Plan {
   int bm, bn;     // tile
+  int tk;         // k bytes per tile row
   int runs;       // K runs (1: the GEMM writes the output itself)
   int tiles_per_run;
 };
 
-// Rows per tile follow M; K is cut into runs while the tiles alone leave CUs
-// idle and every run keeps at least four k tiles.
+inline int num_cus() {
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    return n;
+  }();
+  return cus;
+}
+
+// Up to 128 rows: one row tile of 32, 64 or 128 rows, 128 columns wide so that
+// the column tiles spread over the CUs, and K cut into runs while CUs are
+// still idle, every run keeps 256 k and the runs' int32 sums (written and read
+// once each) stay below the weight bytes.
 Plan make_plan(int64_t M, int64_t K, int64_t N) {
   Plan pl;
+  const int tk = K % 128 == 0 ? 128 : 64;
+  const int64_t ktiles = K / tk;
+  int64_t runs = 1;
   if (M > 128) {
+    // 128-deep tiles: 256x256, two stages, eight wavefronts, one workgroup per
+    // CU.  64-deep tiles (K not a multiple of 128): 256x128, three stages, two
+    // workgroups of four wavefronts per CU.
     pl.bm = 256;
-    pl.bn = 128;
+    pl.bn = tk == 128 ? 256 : 128;
   } else {
     pl.bm = M > 64 ? 128 : (M > 32 ? 64 : 32);
-    pl.bn = 256;
-  }
-  const int64_t tiles = ((M + pl.bm - 1) / pl.bm) * ((N + pl.bn - 1) / pl.bn);
-  const int64_t ktiles = K / kTK;
-  int64_t runs = 1;
-  if (M <= 128 && tiles < 256) {
-    runs = (512 + tiles - 1) / tiles;
-    if (runs > ktiles / 4) runs = ktiles / 4;
+    pl.bn = 128;
+    const int64_t tiles = (N + pl.bn - 1) / pl.bn;
+    runs = (2 * num_cus() + tiles - 1) / tiles;
+    if (runs > ktiles * tk / 256) runs = ktiles * tk / 256;  // at least 256 k per run
+    if (runs > K / (8 * M)) runs = K / (8 * M);
     if (runs < 1) runs = 1;
   }
   int64_t per = (ktiles + runs - 1) / runs;
   runs = (ktiles + per - 1) / per;
+  pl.tk = tk;
   pl.runs = static_cast<int>(runs);
   pl.tiles_per_run = static_cast<int>(per);
   return pl;
@@ -494,11 +653,13 @@ struct Workspace {
   int32_t* count;
   int32_t* list;
   int8_t* qx;
+  uint16_t* sub;
   int32_t* acc;
   int64_t bytes;
 };
 
-Workspace carve(void* base, int64_t M, int64_t K, int64_t N, bool with_acc) {
+Workspace carve(void* base, int64_t M, int64_t K, int64_t N, int runs) {
+  if (runs <= 1) runs = 0;
   unsigned char* p = static_cast<unsigned char*>(base);
   int64_t off = 0;
   Workspace w;
@@ -512,70 +673,92 @@ Workspace carve(void* base, int64_t M, int64_t K, int64_t N, bool with_acc) {
   off += align256(K * 4);
   w.qx = reinterpret_cast<int8_t*>(p + off);
   off += align256(M * K);
+  w.sub = reinterpret_cast<uint16_t*>(p + off);
+  off += align256(M * N * 2);
   w.acc = reinterpret_cast<int32_t*>(p + off);
-  if (with_acc) off += align256(M * N * 4);
+  off += align256(M * N * 4 * runs);
   w.bytes = off;
   return w;
 }
 
-template <int DT, int WM, int WN, int TM, int TN, bool RUNS>
+template <int DT, int WM, int WN, int TM, int TN, int TK, int STAGES, bool RUNS>
 int launch_gemm(const GemmParams& p, int runs, hipStream_t stream) {
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-  constexpr size_t lds = static_cast<size_t>(kStages) * (BM + BN) * kTK;
+  constexpr size_t lds = static_cast<size_t>(STAGES) * (BM + BN) * TK;
+  static_assert(lds >= static_cast<size_t>(WM * WN) * 32 * 40 * 4, "the epilogue's slabs must fit the stages");
   static std::atomic<uint32_t> done{0};
-  auto kern = llm_gemm_kernel<DT, WM, WN, TM, TN, RUNS>;
+  auto kern = llm_gemm_kernel<DT, WM, WN, TM, TN, TK, STAGES, RUNS>;
   allow_lds(reinterpret_cast<const void*>(kern), lds, done);
   hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(p.nbx * p.nby * runs)), dim3(WM * WN * 64), lds, stream,
                      p);
   return check_launch();
 }
 
-template <int DT, bool RUNS>
+template <int DT, int TK, bool RUNS>
 int launch_gemm_for(const GemmParams& p, const Plan& pl, hipStream_t stream) {
   switch (pl.bm) {
     case 256:
       if (RUNS) return WOL_ERR_BAD_SHAPE;  // make_plan cuts K only for tiles of at most 128 rows
-      return launch_gemm<DT, 2, 2, 4, 2, false>(p, pl.runs, stream);
-    case 128: return launch_gemm<DT, 1, 4, 4, 2, RUNS>(p, pl.runs, stream);
-    case 64: return launch_gemm<DT, 1, 4, 2, 2, RUNS>(p, pl.runs, stream);
-    default: return launch_gemm<DT, 1, 4, 1, 2, RUNS>(p, pl.runs, stream);
+      if (pl.bn == 256) return launch_gemm<DT, 2, 4, 4, 2, 128, 2, false>(p, pl.runs, stream);
+      return launch_gemm<DT, 2, 2, 4, 2, 64, 3, false>(p, pl.runs, stream);
+    case 128: return launch_gemm<DT, 1, 4, 4, 1, TK, 3, RUNS>(p, pl.runs, stream);
+    case 64: return launch_gemm<DT, 1, 4, 2, 1, TK, 3, RUNS>(p, pl.runs, stream);
+    default: return launch_gemm<DT, 1, 4, 1, 1, TK, 3, RUNS>(p, pl.runs, stream);
   }
+}
+
+template <int DT, bool RUNS>
+int launch_gemm_tk(const GemmParams& p, const Plan& pl, hipStream_t stream) {
+  return pl.tk == 128 ? launch_gemm_for<DT, 128, RUNS>(p, pl, stream) : launch_gemm_for<DT, 64, RUNS>(p, pl, stream);
+}
+
+// Outlier columns the GEMM's epilogue can hold in LDS behind its slabs (at most
+// 32): (rows + columns of the tile) floats each.
+int fused_cap(const Plan& pl) {
+  if (pl.runs > 1) return 0;  // the merge kernel reads the outlier kernel's product
+  const bool big = pl.bm == 256 && pl.bn == 256;
+  const int64_t lds = static_cast<int64_t>(big ? 2 : 3) * (pl.bm + pl.bn) * pl.tk;
+  const int64_t room = lds - (big ? 8 : 4) * 32 * 40 * 4;
+  const int64_t cap = room / ((pl.bm + pl.bn) * 4);
+  return static_cast<int>(cap > 32 ? 32 : (cap < 0 ? 0 : cap));
 }
 
 template <int DT>
 int run_llm_int8(const void* x, const void* weight, const void* bias, const float* wscale, float threshold,
                  int64_t M, int64_t K, int64_t N, void* out, void* workspace, hipStream_t stream) {
   const Plan pl = make_plan(M, K, N);
-  const Workspace ws = carve(workspace, M, K, N, pl.runs > 1);
+  const Workspace ws = carve(workspace, M, K, N, pl.runs);
   const uint16_t* xs = static_cast<const uint16_t*>(x);
   const int nwords = static_cast<int>(K / 32);
   hipLaunchKernelGGL(llm_clear_kernel, dim3((nwords + 255) / 256), dim3(256), 0, stream, ws.mask, nwords,
                      ws.count);
-  hipLaunchKernelGGL(llm_rowmax_kernel<DT>, dim3(static_cast<unsigned>(M)), dim3(256), 0, stream, xs, threshold,
-                     static_cast<int>(K), ws.ranges, ws.mask);
+  hipLaunchKernelGGL(llm_rowmax_kernel<DT>, dim3(static_cast<unsigned>((M + kRowsPerGroup - 1) / kRowsPerGroup)),
+                     dim3(256), 0, stream, xs, threshold, static_cast<int>(M), static_cast<int>(K), ws.ranges,
+                     ws.mask);
   const int64_t nvec = M * K / 16;
   int64_t qblocks = (nvec + 255) / 256;
   if (qblocks > 8192) qblocks = 8192;
-  const int64_t acc_vec = pl.runs > 1 ? align256(M * N * 4) / 16 : 0;
   hipLaunchKernelGGL(llm_quant_kernel<DT>, dim3(static_cast<unsigned>(qblocks + 1)), dim3(256), 0, stream, xs,
-                     ws.ranges, ws.mask, static_cast<int>(M), static_cast<int>(K), ws.qx, ws.count, ws.list,
-                     ws.acc, acc_vec);
+                     ws.ranges, ws.mask, static_cast<int>(M), static_cast<int>(K), ws.qx, ws.count, ws.list);
   GemmParams p;
   p.qx = ws.qx;
   p.e = Epi{xs, static_cast<const int8_t*>(weight), wscale, ws.ranges, static_cast<const uint16_t*>(bias),
-            ws.count, ws.list, static_cast<uint16_t*>(out), static_cast<int>(M), static_cast<int>(K),
+            ws.count, ws.list, ws.sub, static_cast<uint16_t*>(out), static_cast<int>(M), static_cast<int>(K),
             static_cast<int>(N)};
   p.acc = ws.acc;
   p.nbx = static_cast<int>((N + pl.bn - 1) / pl.bn);
   p.nby = static_cast<int>((M + pl.bm - 1) / pl.bm);
   p.tiles_per_run = pl.tiles_per_run;
+  p.cap = fused_cap(pl);
+  hipLaunchKernelGGL(llm_outlier_kernel<DT>, dim3(static_cast<unsigned>(((N + 255) / 256) * ((M + 63) / 64))),
+                     dim3(256), 0, stream, p.e, ws.sub, p.cap);
   if (check_launch() != WOL_OK) return WOL_ERR_HIP;
-  if (pl.runs == 1) return launch_gemm_for<DT, false>(p, pl, stream);
-  const int rc = launch_gemm_for<DT, true>(p, pl, stream);
+  if (pl.runs == 1) return launch_gemm_tk<DT, false>(p, pl, stream);
+  const int rc = launch_gemm_tk<DT, true>(p, pl, stream);
   if (rc != WOL_OK) return rc;
-  const int64_t total = M * N;
+  const int64_t total = M * (N / 8);
   hipLaunchKernelGGL(llm_merge_kernel<DT>, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, stream,
-                     ws.acc, p.e);
+                     ws.acc, pl.runs, p.e);
   return check_launch();
 }
 
@@ -583,18 +766,19 @@ int run_llm_int8(const void* x, const void* weight, const void* bias, const floa
 
 size_t llm_int8_workspace(int64_t M, int64_t K, int64_t N) {
   const Plan pl = make_plan(M, K, N);
-  return static_cast<size_t>(carve(nullptr, M, K, N, pl.runs > 1).bytes);
+  return static_cast<size_t>(carve(nullptr, M, K, N, pl.runs).bytes);
 }
 
 void llm_int8_workspace_offsets(int64_t M, int64_t K, int64_t N, int64_t* offsets) {
   const Plan pl = make_plan(M, K, N);
-  const Workspace w = carve(nullptr, M, K, N, pl.runs > 1);
+  const Workspace w = carve(nullptr, M, K, N, pl.runs);
   offsets[0] = reinterpret_cast<intptr_t>(w.ranges);
   offsets[1] = reinterpret_cast<intptr_t>(w.mask);
   offsets[2] = reinterpret_cast<intptr_t>(w.count);
   offsets[3] = reinterpret_cast<intptr_t>(w.list);
   offsets[4] = reinterpret_cast<intptr_t>(w.qx);
   offsets[5] = pl.runs > 1 ? reinterpret_cast<intptr_t>(w.acc) : -1;
+  offsets[6] = pl.runs;
 }
 
 int launch_llm_int8_linear(const void* x, const void* weight, const void* bias, const float* wscale,

@@ -108,7 +108,7 @@ def llm_int8_linear(x_bits, w_nk, bias_bits, wscale, threshold, dt, stages=False
     torch.cuda.synchronize()
     if not stages:
         return H.torch_to_bits(out)
-    offs = (ctypes.c_int64 * 6)()
+    offs = (ctypes.c_int64 * 7)()
     _lib.check(_lib.lib.wol_llm_int8_linear_stage_offsets(M, K, N, offs))
     raw = ws.cpu().numpy()
     count = int(raw[offs[2]:offs[2] + 4].view(np.int32)[0])
@@ -119,6 +119,8 @@ def llm_int8_linear(x_bits, w_nk, bias_bits, wscale, threshold, dt, stages=False
         "count": count,
         "list": raw[offs[3]:offs[3] + 4 * count].view(np.int32).copy(),
         "qx": raw[offs[4]:offs[4] + M * K].view(np.int8).reshape(M, K).copy(),
-        "acc": None if offs[5] < 0 else raw[offs[5]:offs[5] + 4 * M * N].view(np.int32).reshape(M, N).copy(),
+        "acc": None if offs[5] < 0 else
+        raw[offs[5]:offs[5] + 4 * M * N * offs[6]].view(np.int32).reshape(offs[6], M, N).sum(axis=0, dtype=np.int32),
+        "runs": int(offs[6]),
     }
     return H.torch_to_bits(out), st

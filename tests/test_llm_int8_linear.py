@@ -170,12 +170,14 @@ GPU_CASES = [  # M, K, N, kind, threshold, bias
     (1, 256, 272, "spiky", 6.0, True),        # one row; N past one 256-column tile by 16
     (5, 128, 48, "normal", 2.0, True),        # many outlier columns
     (33, 192, 80, "spiky", 6.0, False),       # 64-row tile
-    (100, 320, 400, "spiky", 6.0, True),      # 128-row tile
+    (100, 320, 400, "spiky", 6.0, True),      # 128-row tile, one run
     (130, 1024, 144, "spiky", 6.0, True),     # 256-row tile, fused epilogue, ragged in M and N
     (300, 512, 1040, "normal", 3.0, False),   # several row tiles, column tiles not a multiple of 8
     (257, 64, 2048, "spiky", 6.0, True),      # one k tile; column tiles spread over the XCD bands
     (3, 64, 16, "normal", 0.0, True),         # every column an outlier
-    (16, 4096, 512, "spiky", 6.0, True),      # K cut into runs, integer atomics
+    (16, 4096, 512, "spiky", 6.0, True),      # K cut into runs
+    (128, 2048, 272, "spiky", 6.0, True),     # 128-row tile, two runs
+    (700, 512, 8192, "spiky", 6.0, True),     # 256x256 tiles
 ]
 
 
