@@ -25,6 +25,7 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TF = 2500.0   # MI355X dense bf16 MFMA, published
+MFMA_INT8_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA, published
 
 DECODE = dict(M=1, K=4096, N=11008, bits=4, group_size=128, dtype="bfloat16")
 PREFILL = dict(M=2048, K=4096, N=12288, bits=8, group_size=-1, dtype="bfloat16")
@@ -133,6 +134,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--prefill-steps", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-llm-int8", action="store_true", help="skip the llm_int8_linear timing")
     ap.add_argument("--eager", action="store_true", help="time eager launches instead of a graph")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 256 MiB device copies (a known-size kernel to scale "
@@ -217,6 +219,33 @@ def main():
     flops = 2.0 * p["M"] * p["K"] * p["N"]
     pre_tf = flops / pre_s / 1e12
 
+    # ---------------- llm_int8_linear on the prefill shape ----------------
+    # the sibling op on the same weight (algo="llm.int8"): activations N(0,1)
+    # with eight columns scaled x12, so that the outlier branch runs
+    llm = None
+    if not args.no_llm_int8:
+        lw, lscale = Q.weight_quantize(H.bits_to_torch(pw_bits, dt, dev), algo="llm.int8")
+        lx = px.clone()
+        lx[:, 100:3700:450] *= 12.0
+
+        def llm_step(i):
+            return Q.llm_int8_linear(lx, lw, None, lscale, 6.0)
+
+        llm_s = timer(torch, llm_step, args.prefill_steps, args.warmup) / args.prefill_steps
+        llm_tops = flops / llm_s / 1e12
+        llm = {
+            "workload": "llm_int8_linear M=2048, K=4096 N=12288, bf16 x with 8 outlier columns, threshold 6.0; "
+                        "all stages of one call (row ranges, activation codes, int8 GEMM with the merge)",
+            "value": round(llm_tops, 2),
+            "unit": "TOP/s",
+            "ms_per_step": round(llm_s * 1e3, 4),
+            "steps": args.prefill_steps,
+            "roofline": {"bound": "mfma", "achieved": round(llm_tops, 2), "peak": MFMA_INT8_PEAK_TOPS,
+                         "unit": "TOP/s", "frac": round(llm_tops / MFMA_INT8_PEAK_TOPS, 4), "traffic": None,
+                         "kernel": "wol::llm_gemm_kernel<1, 2, 4, 4, 2, 128, 2, false> (256x256 tiles, "
+                                   "v_mfma_i32_32x32x32_i8)"},
+        }
+
     # ---------------- CPU baseline + parity of the decode output ----------------
     cpu = None
     parity = {}
@@ -281,6 +310,7 @@ def main():
                 "kernel": "wol::gemm_dma_kernel<1, 8, 0, false, 2, 4, 4, 2, 3> (256x256 tiles on the columns that fill whole rounds of the 256 CUs) + <1, 8, 0, false, 2, 4, 4, 1, 3> (256x128 tiles on the rest)",
             },
         },
+        "llm_int8": llm,
         "cpu_baseline": cpu,
         "parity": parity,
     }

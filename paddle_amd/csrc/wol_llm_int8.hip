@@ -57,6 +57,11 @@ __global__ __launch_bounds__(256) void llm_clear_kernel(int32_t* mask, int nword
 // reach the mask as one atomic per workgroup (outlier columns tend to be the
 // same in every row).
 constexpr int kRowsPerGroup = 8;
+// The mask is kept in kMaskCopies copies, workgroup g of the row kernel ORing
+// into copy g % kMaskCopies: atomics on one word serialise (about 50 ns each
+// across the XCDs), and this many fewer meet on a hot column's word.  Readers
+// OR the copies; the list kernel leaves the combined mask in copy 0.
+constexpr int kMaskCopies = 8;
 
 template <int DT>
 __global__ __launch_bounds__(256) void llm_rowmax_kernel(const uint16_t* __restrict__ x, float threshold, int M,
@@ -65,6 +70,7 @@ __global__ __launch_bounds__(256) void llm_rowmax_kernel(const uint16_t* __restr
   __shared__ float part[4][kRowsPerGroup];
   const float thr = to_f32<DT>(from_f32_rne<DT>(threshold));  // the comparison is made in T
   const int m0 = blockIdx.x * kRowsPerGroup;
+  mask += static_cast<int64_t>(blockIdx.x % kMaskCopies) * (K / 32);
   float mx[kRowsPerGroup];
 #pragma unroll
   for (int r = 0; r < kRowsPerGroup; ++r) mx[r] = 0.0f;
@@ -124,7 +130,7 @@ __device__ inline uint32_t quant_one(float xv, float inv) {
 template <int DT>
 __global__ __launch_bounds__(256) void llm_quant_kernel(const uint16_t* __restrict__ x,
                                                         const float* __restrict__ ranges,
-                                                        const int32_t* __restrict__ mask, int M, int K,
+                                                        int32_t* mask, int M, int K,
                                                         int8_t* __restrict__ qx, int32_t* __restrict__ count,
                                                         int32_t* __restrict__ list) {
   const int tid = threadIdx.x;
@@ -136,7 +142,12 @@ __global__ __launch_bounds__(256) void llm_quant_kernel(const uint16_t* __restri
     if (tid == 0) base_s = 0;
     __syncthreads();
     for (int w0 = 0; w0 < nwords; w0 += 256) {
-      uint32_t word = w0 + tid < nwords ? static_cast<uint32_t>(mask[w0 + tid]) : 0u;
+      uint32_t word = 0u;
+      if (w0 + tid < nwords) {
+#pragma unroll
+        for (int r = 0; r < kMaskCopies; ++r) word |= static_cast<uint32_t>(mask[r * nwords + w0 + tid]);
+        mask[w0 + tid] = static_cast<int32_t>(word);  // the combined mask, for whoever inspects the stages
+      }
       const int c = __popc(word);
       scan[tid] = c;
       __syncthreads();
@@ -169,7 +180,10 @@ __global__ __launch_bounds__(256) void llm_quant_kernel(const uint16_t* __restri
     const int k = static_cast<int>(e - static_cast<int64_t>(m) * K);
     const u32x4 lo = *reinterpret_cast<const u32x4*>(x + e);
     const u32x4 hi = *reinterpret_cast<const u32x4*>(x + e + 8);
-    const uint32_t out_bits = static_cast<uint32_t>(mask[k >> 5]) >> (k & 31);
+    uint32_t mword = 0u;
+#pragma unroll
+    for (int r = 0; r < kMaskCopies; ++r) mword |= static_cast<uint32_t>(mask[r * (K / 32) + (k >> 5)]);
+    const uint32_t out_bits = mword >> (k & 31);
     const float inv = 1.0f / ranges[m];
     u32x4 q = {0u, 0u, 0u, 0u};
 #pragma unroll
@@ -194,7 +208,6 @@ struct Epi {
   const uint16_t* bias;   // [N] T or null
   const int32_t* count;
   const int32_t* list;
-  const uint16_t* sub;    // [M,N] T: the outlier columns' product, valid when *count > 0
   uint16_t* out;          // [M,N] T
   int M, K, N;
 };
@@ -232,7 +245,7 @@ __device__ inline uint16_t merge_plain(int acc, float range, float ws, bool has_
 
 // Eight neighbouring columns nn .. nn+7 of row m: the merge with the outlier
 // columns' product (when there are any: out of LDS if xs is given, else as
-// the outlier kernel left it in e.sub) and one 16-byte store.  ws and bias hold the eight columns' values.
+// the outlier kernel left it in the output's own place) and one 16-byte store.  ws and bias hold the eight columns' values.
 template <int DT>
 __device__ inline void finish8(const Epi& e, int cnt, int m, int nn, i32x4 s0, i32x4 s1, const float* ws,
                                const float* bias, const float* xs, int xs_stride, const float* wd,
@@ -270,7 +283,7 @@ __device__ inline void finish8(const Epi& e, int cnt, int m, int nn, i32x4 s0, i
 #pragma unroll
     for (int i = 0; i < 8; ++i) sub[i] = to_f32<DT>(cast_out<DT>(sub[i]));
   } else {
-    const u32x4 sv = *reinterpret_cast<const u32x4*>(e.sub + static_cast<int64_t>(m) * e.N + nn);
+    const u32x4 sv = *reinterpret_cast<const u32x4*>(e.out + static_cast<int64_t>(m) * e.N + nn);
 #pragma unroll
     for (int i = 0; i < 8; ++i) sub[i] = to_f32<DT>(static_cast<uint16_t>(sv[i >> 1] >> (16 * (i & 1))));
   }
@@ -305,7 +318,8 @@ __device__ inline void load_ws_bias8(const Epi& e, int nn, float* ws, float* bia
 // a time wait in LDS.  Workgroups leave at once when there is no outlier or
 // the GEMM's epilogue computes the product itself (up to fused_cap columns).
 template <int DT>
-__global__ __launch_bounds__(256) void llm_outlier_kernel(Epi e, uint16_t* __restrict__ sub, int fused_cap) {
+__global__ __launch_bounds__(256) void llm_outlier_kernel(Epi e, int fused_cap) {
+  uint16_t* sub = e.out;  // the product waits where the output will go: whoever merges element (m, n) reads it first
   const int cnt = *e.count;
   if (cnt <= fused_cap) return;  // none, or few enough for the GEMM's epilogue to take them
   __shared__ __attribute__((aligned(16))) float xs[32][64];
@@ -356,7 +370,7 @@ struct GemmParams {
   int32_t* acc;      // [runs][M,N] int32, one slab per K run; only with K runs
   int nbx, nby;      // tiles along N and M
   int tiles_per_run; // k tiles per K run
-  int cap;  // outlier columns the epilogue takes through LDS itself; more come from e.sub
+  int cap;  // outlier columns the epilogue takes through LDS itself; more come from the outlier kernel
 };
 
 // XOR applied to the 16-byte piece index of a row in LDS (C pieces per row) so
@@ -625,11 +639,19 @@ Plan make_plan(int64_t M, int64_t K, int64_t N) {
   const int64_t ktiles = K / tk;
   int64_t runs = 1;
   if (M > 128) {
-    // 128-deep tiles: 256x256, two stages, eight wavefronts, one workgroup per
-    // CU.  64-deep tiles (K not a multiple of 128): 256x128, three stages, two
-    // workgroups of four wavefronts per CU.
+    // 128-deep tiles, eight wavefronts, one workgroup per CU: 256x256 with two
+    // stages, or 128x256 with three where their rounds over the CUs come out
+    // shorter (a half tile takes 0.55 of a whole one; 384 whole tiles on 256
+    // CUs are two rounds, 768 half tiles three).  64-deep tiles (K not a
+    // multiple of 128): 256x128, three stages, two workgroups of four per CU.
     pl.bm = 256;
     pl.bn = tk == 128 ? 256 : 128;
+    if (tk == 128) {
+      const int64_t cus = num_cus();
+      const int64_t cols = (N + 255) / 256;
+      const int64_t whole = ((M + 255) / 256) * cols, half = ((M + 127) / 128) * cols;
+      if (11 * ((half + cus - 1) / cus) < 20 * ((whole + cus - 1) / cus)) pl.bm = 128;
+    }
   } else {
     pl.bm = M > 64 ? 128 : (M > 32 ? 64 : 32);
     pl.bn = 128;
@@ -653,7 +675,6 @@ struct Workspace {
   int32_t* count;
   int32_t* list;
   int8_t* qx;
-  uint16_t* sub;
   int32_t* acc;
   int64_t bytes;
 };
@@ -666,15 +687,13 @@ Workspace carve(void* base, int64_t M, int64_t K, int64_t N, int runs) {
   w.ranges = reinterpret_cast<float*>(p + off);
   off += align256(M * 4);
   w.mask = reinterpret_cast<int32_t*>(p + off);
-  off += align256(K / 32 * 4);
+  off += align256(K / 32 * 4 * kMaskCopies);
   w.count = reinterpret_cast<int32_t*>(p + off);
   off += 256;
   w.list = reinterpret_cast<int32_t*>(p + off);
   off += align256(K * 4);
   w.qx = reinterpret_cast<int8_t*>(p + off);
   off += align256(M * K);
-  w.sub = reinterpret_cast<uint16_t*>(p + off);
-  off += align256(M * N * 2);
   w.acc = reinterpret_cast<int32_t*>(p + off);
   off += align256(M * N * 4 * runs);
   w.bytes = off;
@@ -701,7 +720,12 @@ int launch_gemm_for(const GemmParams& p, const Plan& pl, hipStream_t stream) {
       if (RUNS) return WOL_ERR_BAD_SHAPE;  // make_plan cuts K only for tiles of at most 128 rows
       if (pl.bn == 256) return launch_gemm<DT, 2, 4, 4, 2, 128, 2, false>(p, pl.runs, stream);
       return launch_gemm<DT, 2, 2, 4, 2, 64, 3, false>(p, pl.runs, stream);
-    case 128: return launch_gemm<DT, 1, 4, 4, 1, TK, 3, RUNS>(p, pl.runs, stream);
+    case 128:
+      if (pl.bn == 256) {
+        if (RUNS || TK != 128) return WOL_ERR_BAD_SHAPE;  // make_plan: many rows, 128-deep tiles
+        return launch_gemm<DT, 2, 4, 2, 2, 128, 3, false>(p, pl.runs, stream);
+      }
+      return launch_gemm<DT, 1, 4, 4, 1, TK, 3, RUNS>(p, pl.runs, stream);
     case 64: return launch_gemm<DT, 1, 4, 2, 1, TK, 3, RUNS>(p, pl.runs, stream);
     default: return launch_gemm<DT, 1, 4, 1, 1, TK, 3, RUNS>(p, pl.runs, stream);
   }
@@ -716,9 +740,9 @@ int launch_gemm_tk(const GemmParams& p, const Plan& pl, hipStream_t stream) {
 // 32): (rows + columns of the tile) floats each.
 int fused_cap(const Plan& pl) {
   if (pl.runs > 1) return 0;  // the merge kernel reads the outlier kernel's product
-  const bool big = pl.bm == 256 && pl.bn == 256;
-  const int64_t lds = static_cast<int64_t>(big ? 2 : 3) * (pl.bm + pl.bn) * pl.tk;
-  const int64_t room = lds - (big ? 8 : 4) * 32 * 40 * 4;
+  const bool eight = pl.bn == 256;  // the configurations of eight wavefronts
+  const int64_t lds = static_cast<int64_t>(pl.bm == 256 && eight ? 2 : 3) * (pl.bm + pl.bn) * pl.tk;
+  const int64_t room = lds - (eight ? 8 : 4) * 32 * 40 * 4;
   const int64_t cap = room / ((pl.bm + pl.bn) * 4);
   return static_cast<int>(cap > 32 ? 32 : (cap < 0 ? 0 : cap));
 }
@@ -729,7 +753,7 @@ int run_llm_int8(const void* x, const void* weight, const void* bias, const floa
   const Plan pl = make_plan(M, K, N);
   const Workspace ws = carve(workspace, M, K, N, pl.runs);
   const uint16_t* xs = static_cast<const uint16_t*>(x);
-  const int nwords = static_cast<int>(K / 32);
+  const int nwords = static_cast<int>(K / 32) * kMaskCopies;
   hipLaunchKernelGGL(llm_clear_kernel, dim3((nwords + 255) / 256), dim3(256), 0, stream, ws.mask, nwords,
                      ws.count);
   hipLaunchKernelGGL(llm_rowmax_kernel<DT>, dim3(static_cast<unsigned>((M + kRowsPerGroup - 1) / kRowsPerGroup)),
@@ -743,7 +767,7 @@ int run_llm_int8(const void* x, const void* weight, const void* bias, const floa
   GemmParams p;
   p.qx = ws.qx;
   p.e = Epi{xs, static_cast<const int8_t*>(weight), wscale, ws.ranges, static_cast<const uint16_t*>(bias),
-            ws.count, ws.list, ws.sub, static_cast<uint16_t*>(out), static_cast<int>(M), static_cast<int>(K),
+            ws.count, ws.list, static_cast<uint16_t*>(out), static_cast<int>(M), static_cast<int>(K),
             static_cast<int>(N)};
   p.acc = ws.acc;
   p.nbx = static_cast<int>((N + pl.bn - 1) / pl.bn);
@@ -751,7 +775,7 @@ int run_llm_int8(const void* x, const void* weight, const void* bias, const floa
   p.tiles_per_run = pl.tiles_per_run;
   p.cap = fused_cap(pl);
   hipLaunchKernelGGL(llm_outlier_kernel<DT>, dim3(static_cast<unsigned>(((N + 255) / 256) * ((M + 63) / 64))),
-                     dim3(256), 0, stream, p.e, ws.sub, p.cap);
+                     dim3(256), 0, stream, p.e, p.cap);
   if (check_launch() != WOL_OK) return WOL_ERR_HIP;
   if (pl.runs == 1) return launch_gemm_tk<DT, false>(p, pl, stream);
   const int rc = launch_gemm_tk<DT, true>(p, pl, stream);

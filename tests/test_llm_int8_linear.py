@@ -207,13 +207,14 @@ def test_gpu_llm_int8_linear_bit_exact(device, oracle, dt, case):
 
 
 @pytest.mark.gpu
-def test_gpu_llm_int8_linear_large_properties(device, oracle):
-    """M = 2048, K = 4096, N = 12288 (too large for the scalar oracle): rows
+@pytest.mark.parametrize("N", [12288, 8192])  # 128x256 tiles (three rounds of the CUs), 256x256 tiles (one round)
+def test_gpu_llm_int8_linear_large_properties(device, oracle, N):
+    """M = 2048, K = 4096, N = 12288 | 8192 (too large for the scalar oracle): rows
     checked against the oracle on a slice of the columns, and the whole result
     against a float64 statement of the no-outlier formula."""
     import gpu_calls as G
 
-    dt, M, K, N = H.BF16, 2048, 4096, 12288
+    dt, M, K = H.BF16, 2048, 4096
     rng = np.random.default_rng(5)
     w_nk = rng.integers(-127, 128, (N, K), dtype=np.int8)
     ws = (rng.random(N, dtype=np.float32) * np.float32(1e-3) + np.float32(1e-4)).astype(np.float32)
