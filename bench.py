@@ -242,7 +242,7 @@ def main():
             "steps": args.prefill_steps,
             "roofline": {"bound": "mfma", "achieved": round(llm_tops, 2), "peak": MFMA_INT8_PEAK_TOPS,
                          "unit": "TOP/s", "frac": round(llm_tops / MFMA_INT8_PEAK_TOPS, 4), "traffic": None,
-                         "kernel": "wol::llm_gemm_kernel<1, 2, 4, 4, 2, 128, 2, false> (256x256 tiles, "
+                         "kernel": "wol::llm_gemm_kernel<1, 2, 4, 2, 2, 128, 3, false> (128x256 tiles, "
                                    "v_mfma_i32_32x32x32_i8)"},
         }
 

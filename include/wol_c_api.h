@@ -240,7 +240,9 @@ int wol_apply_per_channel_scale(const void* x, const void* scales, int dtype,
  * as the operator's description and the reference's own test
  * (test/quantization/test_llm_int8_linear.py:84-111) have it.
  * Requires K % 64 == 0 and N % 16 == 0 (what weight_quantize accepts); x,
- * weight, weight_scale, out and workspace 16-byte aligned.  The workspace is
+ * weight, weight_scale, out and workspace 16-byte aligned; out must not
+ * overlap an input (with many outlier columns their product waits in out
+ * until it is merged).  The workspace is
  * required (wol_llm_int8_linear_workspace bytes); it holds the row ranges,
  * the outlier mask and list, the activation codes and, for few rows, the int32
  * sums of the runs K is cut into.  Nothing returns to the host: the reference's device-to-host copy of

@@ -497,3 +497,29 @@ void wo_llm_int8_linear(const uint16_t* x, const int8_t* w, const uint16_t* bias
   if (outlier_out) memcpy(outlier_out, outlier, (size_t)K);
   free(outlier); free(range); free(q);
 }
+
+/* The division by 127 of DequantFunc as the HIP epilogue performs it: a
+ * reciprocal multiply corrected by two FMAs.  Counts the inputs first,
+ * first + stride, ... (count of them, as float bit patterns) for which it
+ * differs from the IEEE division the reference uses
+ * (impl/llm_int8_matmul_kernel_impl.h:172-176).  The full sweep (first 0,
+ * stride 1, count 2^32) returns 0; the tests run a strided sample. */
+int64_t wo_div127_fma_mismatches(uint32_t first, uint32_t stride, int64_t count) {
+  const float y = 1.0f / 127.0f;
+  int64_t bad = 0;
+  uint32_t u = first;
+  for (int64_t i = 0; i < count; ++i, u += stride) {
+    float v, ref, q, r, q2;
+    uint32_t a, b;
+    memcpy(&v, &u, 4);
+    ref = v / 127.0f;
+    q = v * y;
+    r = fmaf(-q, 127.0f, v);
+    q2 = fmaf(r, y, q);
+    if (!(r != 0.0f && r == r)) q2 = q;
+    memcpy(&a, &ref, 4);
+    memcpy(&b, &q2, 4);
+    if (a != b && !(ref != ref && q2 != q2)) ++bad;
+  }
+  return bad;
+}

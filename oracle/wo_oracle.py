@@ -61,6 +61,8 @@ def lib():
                                          _int, _u16p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                          ctypes.c_void_p]
         L.wo_llm_int8_linear.restype = None
+        L.wo_div127_fma_mismatches.argtypes = [ctypes.c_uint32, ctypes.c_uint32, _i64]
+        L.wo_div127_fma_mismatches.restype = _i64
         L.wo_dequantize.argtypes = [_i8p, _u16p, _i64, _i64, _int, _int, _i64, _int, _int,
                                     ctypes.c_void_p, ctypes.c_void_p]
         L.wo_linear.argtypes = [_u16p, _i8p, ctypes.c_void_p, _u16p, _i64, _i64, _i64, _int, _int,
@@ -145,6 +147,12 @@ def llm_int8_linear(x_bits, w_nk, bias_bits, wscale, threshold, dtype):
     lib().wo_llm_int8_linear(x_bits, w_nk, bias_ptr, wscale, float(threshold), M, K, N, dtype, out,
                              qx.ctypes.data, acc.ctypes.data, ranges.ctypes.data, outlier.ctypes.data)
     return {"out": out, "qx": qx, "acc": acc, "ranges": ranges, "outlier": outlier.astype(bool)}
+
+
+def div127_fma_mismatches(first, stride, count):
+    """Inputs (float bit patterns first, first + stride, ...) on which the FMA-corrected
+    reciprocal multiply of the HIP epilogue differs from the IEEE division by 127."""
+    return int(lib().wo_div127_fma_mismatches(first, stride, count))
 
 
 def transpose_bytes(a):

@@ -137,6 +137,15 @@ def test_oracle_invariants_and_reference_expectation(oracle, dt):
     assert H.rel_l2(H.bits_to_f32(o2["out"], dt), want) < (2e-3 if dt == H.F16 else 1e-2)
 
 
+def test_division_by_127_as_the_kernel_does_it(oracle):
+    # q = v * RN(1/127); r = fma(-q, 127, v); q + r * RN(1/127): equal to v / 127.0f on all 2^32 floats (the full
+    # sweep takes half a minute on eight cores and was run once); here every 1021st pattern, the values around
+    # zero, the subnormal boundary, infinity and the int32 range the accumulators come from
+    assert oracle.div127_fma_mismatches(0, 1021, (1 << 32) // 1021) == 0
+    for first in (0x00000000, 0x80000000, 0x007FFF00, 0x7F7FFF00, 0xFF7FFF00, 0x4B000000, 0x4EFFFF00):
+        assert oracle.div127_fma_mismatches(first, 1, 1 << 12) == 0
+
+
 def test_infer_meta_checks():
     from paddle_amd.nn.quant import quantized_linear as QL
 
