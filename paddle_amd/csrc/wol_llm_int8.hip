@@ -56,7 +56,7 @@ __global__ __launch_bounds__(256) void llm_clear_kernel(int32_t* mask, int nword
 // so that a column's outlier bits are ORed over the rows in registers and
 // reach the mask as one atomic per workgroup (outlier columns tend to be the
 // same in every row).
-constexpr int kRowsPerGroup = 8;
+constexpr int kRowsPerGroup = 4;
 // The mask is kept in kMaskCopies copies, workgroup g of the row kernel ORing
 // into copy g % kMaskCopies: atomics on one word serialise (about 50 ns each
 // across the XCDs), and this many fewer meet on a hot column's word.  Readers
@@ -127,6 +127,127 @@ __device__ inline uint32_t quant_one(float xv, float inv) {
   return static_cast<uint32_t>(static_cast<int>(t)) & 0xFFu;
 }
 
+// The mask (nwords words, word w from word_at(w)) as an ascending list of
+// outlier columns and their count.  Called by every thread of a workgroup (of
+// at least 256 threads; the first 256 do the work); scan (256 ints) and base_s
+// are LDS.
+template <class F>
+__device__ inline void build_list(int nwords, F word_at, int32_t* list, int32_t* count, int* scan, int* base_s) {
+  const int tid = threadIdx.x;
+  const bool worker = tid < 256;
+  if (tid == 0) *base_s = 0;
+  __syncthreads();
+  for (int w0 = 0; w0 < nwords; w0 += 256) {
+    uint32_t word = worker && w0 + tid < nwords ? word_at(w0 + tid) : 0u;
+    const int c = __popc(word);
+    if (worker) scan[tid] = c;
+    __syncthreads();
+    for (int d = 1; d < 256; d <<= 1) {
+      const int add = worker && tid >= d ? scan[tid - d] : 0;
+      __syncthreads();
+      if (worker) scan[tid] += add;
+      __syncthreads();
+    }
+    const int base = *base_s;
+    int o = worker ? base + scan[tid] - c : 0;
+    while (word != 0) {
+      const int b = __ffs(word) - 1;
+      list[o++] = (w0 + tid) * 32 + b;
+      word &= word - 1;
+    }
+    __syncthreads();
+    if (tid == 0) *base_s = base + scan[255];
+    __syncthreads();
+  }
+  if (tid == 0) *count = *base_s;
+}
+
+// Row ranges, outlier mask and list, activation codes of up to kSmallRows rows
+// in one workgroup: the decode-sized case, where three launches cost more
+// than the work.  The mask lives in LDS (K / 32 words, dynamic).
+constexpr int kSmallRows = 2;  // beyond two rows the single workgroup takes longer than the three launches
+constexpr int kSmallThreads = 1024;
+constexpr int kSmallMaxK = 65536;
+
+template <int DT>
+__global__ __launch_bounds__(kSmallThreads) void llm_act_small_kernel(const uint16_t* __restrict__ x, float threshold,
+                                                                      int M, int K, float* __restrict__ ranges,
+                                                                      int32_t* __restrict__ mask,
+                                                                      int8_t* __restrict__ qx,
+                                                                      int32_t* __restrict__ count,
+                                                                      int32_t* __restrict__ list) {
+  extern __shared__ uint32_t smask[];
+  __shared__ float part[kSmallThreads / 64][kSmallRows];
+  __shared__ float srange[kSmallRows];
+  __shared__ int scan[256];
+  __shared__ int base_s;
+  const int tid = threadIdx.x;
+  const int nwords = K / 32;
+  const float thr = to_f32<DT>(from_f32_rne<DT>(threshold));
+  for (int w = tid; w < nwords; w += kSmallThreads) smask[w] = 0u;
+  __syncthreads();
+  float mx[kSmallRows];
+#pragma unroll
+  for (int r = 0; r < kSmallRows; ++r) mx[r] = 0.0f;
+  for (int k0 = tid * 8; k0 < K; k0 += kSmallThreads * 8) {
+    uint32_t bits = 0;
+#pragma unroll
+    for (int r = 0; r < kSmallRows; ++r) {
+      if (r < M) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(x + static_cast<int64_t>(r) * K + k0);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          float a = fabsf(to_f32<DT>(static_cast<uint16_t>(v[i >> 1] >> (16 * (i & 1)))));
+          if (a > thr) {
+            bits |= 1u << i;
+            a = 0.0f;
+          }
+          mx[r] = a > mx[r] ? a : mx[r];
+        }
+      }
+    }
+    if (bits != 0) atomicOr(&smask[k0 >> 5], bits << (k0 & 31));
+  }
+#pragma unroll
+  for (int r = 0; r < kSmallRows; ++r) {
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) {
+      const float o = __shfl_xor(mx[r], d, 64);
+      mx[r] = o > mx[r] ? o : mx[r];
+    }
+    if ((tid & 63) == 0) part[tid >> 6][r] = mx[r];
+  }
+  __syncthreads();
+  if (tid < M) {
+    float r = part[0][tid];
+#pragma unroll
+    for (int i = 1; i < kSmallThreads / 64; ++i) r = part[i][tid] > r ? part[i][tid] : r;
+    ranges[tid] = r;
+    srange[tid] = r;
+  }
+  for (int w = tid; w < nwords; w += kSmallThreads) mask[w] = static_cast<int32_t>(smask[w]);  // for whoever inspects the stages
+  build_list(nwords, [&](int w) { return smask[w]; }, list, count, scan, &base_s);  // its barriers also publish srange
+  const int64_t nvec = static_cast<int64_t>(M) * K / 16;
+  for (int64_t v = tid; v < nvec; v += kSmallThreads) {
+    const int64_t e = v * 16;
+    const int m = static_cast<int>(e / K);
+    const int k = static_cast<int>(e - static_cast<int64_t>(m) * K);
+    const u32x4 lo = *reinterpret_cast<const u32x4*>(x + e);
+    const u32x4 hi = *reinterpret_cast<const u32x4*>(x + e + 8);
+    const uint32_t out_bits = smask[k >> 5] >> (k & 31);
+    const float inv = 1.0f / srange[m];
+    u32x4 q = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const uint32_t word = i < 8 ? lo[(i & 7) >> 1] : hi[(i & 7) >> 1];
+      const float xv = to_f32<DT>(static_cast<uint16_t>(word >> (16 * (i & 1))));
+      const uint32_t c = (out_bits >> i) & 1u ? 0u : quant_one(xv, inv);
+      q[i >> 2] |= c << (8 * (i & 3));
+    }
+    *reinterpret_cast<u32x4*>(qx + e) = q;
+  }
+}
+
 template <int DT>
 __global__ __launch_bounds__(256) void llm_quant_kernel(const uint16_t* __restrict__ x,
                                                         const float* __restrict__ ranges,
@@ -135,40 +256,16 @@ __global__ __launch_bounds__(256) void llm_quant_kernel(const uint16_t* __restri
                                                         int32_t* __restrict__ list) {
   const int tid = threadIdx.x;
   if (blockIdx.x == gridDim.x - 1) {
-    // the mask as an ascending list of outlier columns
     __shared__ int scan[256];
     __shared__ int base_s;
     const int nwords = K / 32;
-    if (tid == 0) base_s = 0;
-    __syncthreads();
-    for (int w0 = 0; w0 < nwords; w0 += 256) {
+    build_list(nwords, [&](int w) {
       uint32_t word = 0u;
-      if (w0 + tid < nwords) {
 #pragma unroll
-        for (int r = 0; r < kMaskCopies; ++r) word |= static_cast<uint32_t>(mask[r * nwords + w0 + tid]);
-        mask[w0 + tid] = static_cast<int32_t>(word);  // the combined mask, for whoever inspects the stages
-      }
-      const int c = __popc(word);
-      scan[tid] = c;
-      __syncthreads();
-      for (int d = 1; d < 256; d <<= 1) {
-        const int add = tid >= d ? scan[tid - d] : 0;
-        __syncthreads();
-        scan[tid] += add;
-        __syncthreads();
-      }
-      const int base = base_s;
-      int o = base + scan[tid] - c;
-      while (word != 0) {
-        const int b = __ffs(word) - 1;
-        list[o++] = (w0 + tid) * 32 + b;
-        word &= word - 1;
-      }
-      __syncthreads();
-      if (tid == 0) base_s = base + scan[255];
-      __syncthreads();
-    }
-    if (tid == 0) *count = base_s;
+      for (int r = 0; r < kMaskCopies; ++r) word |= static_cast<uint32_t>(mask[r * nwords + w]);
+      mask[w] = static_cast<int32_t>(word);  // the combined mask, for whoever inspects the stages
+      return word;
+    }, list, count, scan, &base_s);
     return;
   }
   const int64_t stride = static_cast<int64_t>(gridDim.x - 1) * 256;
@@ -656,7 +753,7 @@ Plan make_plan(int64_t M, int64_t K, int64_t N) {
     pl.bm = M > 64 ? 128 : (M > 32 ? 64 : 32);
     pl.bn = 128;
     const int64_t tiles = (N + pl.bn - 1) / pl.bn;
-    runs = (2 * num_cus() + tiles - 1) / tiles;
+    runs = 2 * num_cus() / tiles;  // two workgroups fit a CU: no second, nearly empty round
     if (runs > ktiles * tk / 256) runs = ktiles * tk / 256;  // at least 256 k per run
     if (runs > K / (8 * M)) runs = K / (8 * M);
     if (runs < 1) runs = 1;
@@ -753,16 +850,22 @@ int run_llm_int8(const void* x, const void* weight, const void* bias, const floa
   const Plan pl = make_plan(M, K, N);
   const Workspace ws = carve(workspace, M, K, N, pl.runs);
   const uint16_t* xs = static_cast<const uint16_t*>(x);
+  const bool small = M <= kSmallRows && K <= kSmallMaxK;
+  if (small) {
+    hipLaunchKernelGGL(llm_act_small_kernel<DT>, dim3(1), dim3(kSmallThreads), static_cast<size_t>(K / 32 * 4), stream,
+                       xs, threshold, static_cast<int>(M), static_cast<int>(K), ws.ranges, ws.mask, ws.qx, ws.count,
+                       ws.list);
+  }
   const int nwords = static_cast<int>(K / 32) * kMaskCopies;
-  hipLaunchKernelGGL(llm_clear_kernel, dim3((nwords + 255) / 256), dim3(256), 0, stream, ws.mask, nwords,
+  if (!small) hipLaunchKernelGGL(llm_clear_kernel, dim3((nwords + 255) / 256), dim3(256), 0, stream, ws.mask, nwords,
                      ws.count);
-  hipLaunchKernelGGL(llm_rowmax_kernel<DT>, dim3(static_cast<unsigned>((M + kRowsPerGroup - 1) / kRowsPerGroup)),
+  if (!small) hipLaunchKernelGGL(llm_rowmax_kernel<DT>, dim3(static_cast<unsigned>((M + kRowsPerGroup - 1) / kRowsPerGroup)),
                      dim3(256), 0, stream, xs, threshold, static_cast<int>(M), static_cast<int>(K), ws.ranges,
                      ws.mask);
   const int64_t nvec = M * K / 16;
   int64_t qblocks = (nvec + 255) / 256;
   if (qblocks > 8192) qblocks = 8192;
-  hipLaunchKernelGGL(llm_quant_kernel<DT>, dim3(static_cast<unsigned>(qblocks + 1)), dim3(256), 0, stream, xs,
+  if (!small) hipLaunchKernelGGL(llm_quant_kernel<DT>, dim3(static_cast<unsigned>(qblocks + 1)), dim3(256), 0, stream, xs,
                      ws.ranges, ws.mask, static_cast<int>(M), static_cast<int>(K), ws.qx, ws.count, ws.list);
   GemmParams p;
   p.qx = ws.qx;
