@@ -591,19 +591,44 @@ __global__ __launch_bounds__(WM* WN * 64) __attribute__((amdgpu_waves_per_eu(2))
     __builtin_amdgcn_s_barrier();
     WOL_LLM_ISSUE(it + kStages - 1);  // into the stage every wavefront finished reading before the barrier
     const unsigned char* stage = smem + (it % kStages) * kStage;
+    // the fragments of k step ks + 1 are read while the MFMAs of step ks run
+    constexpr int KS = C / 2;
+    i32x4 af[2][TM], bf[2][TN];
+    {
+      const int piece = (b ^ swz) * 16;
 #pragma unroll
-    for (int ks = 0; ks < C / 2; ++ks) {
-      const int piece = ((ks * 2 + b) ^ swz) * 16;
-      i32x4 af[TM], bf[TN];
+      for (int a = 0; a < TM; ++a) af[0][a] = *reinterpret_cast<const i32x4*>(stage + aoff[a] + piece);
 #pragma unroll
-      for (int a = 0; a < TM; ++a) af[a] = *reinterpret_cast<const i32x4*>(stage + aoff[a] + piece);
+      for (int c = 0; c < TN; ++c) bf[0][c] = *reinterpret_cast<const i32x4*>(stage + boff[c] + piece);
+    }
 #pragma unroll
-      for (int c = 0; c < TN; ++c) bf[c] = *reinterpret_cast<const i32x4*>(stage + boff[c] + piece);
+    for (int ks = 0; ks < KS; ++ks) {
+      if (ks + 1 < KS) {
+        const int piece = (((ks + 1) * 2 + b) ^ swz) * 16;
+#pragma unroll
+        for (int a = 0; a < TM; ++a)
+          af[(ks + 1) & 1][a] = *reinterpret_cast<const i32x4*>(stage + aoff[a] + piece);
+#pragma unroll
+        for (int c = 0; c < TN; ++c)
+          bf[(ks + 1) & 1][c] = *reinterpret_cast<const i32x4*>(stage + boff[c] + piece);
+      }
 #pragma unroll
       for (int a = 0; a < TM; ++a)
 #pragma unroll
         for (int c = 0; c < TN; ++c)
-          acc[a][c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bf[c], acc[a][c], 0, 0, 0);
+          acc[a][c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][a], bf[ks & 1][c], acc[a][c], 0, 0, 0);
+      // issue order: the LDS reads of the next step spread between this step's
+      // MFMAs (left alone the scheduler reads one fragment, waits, and issues
+      // the two MFMAs that use it)
+      constexpr int kMfma = TM * TN, kRead = TM + TN;
+#pragma unroll
+      for (int i = 0; i < kMfma; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        const int reads = ks + 1 < KS ? kRead * (i + 1) / kMfma - kRead * i / kMfma : 0;
+#pragma unroll
+        for (int r = 0; r < reads; ++r) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // nothing moves between k steps
     }
   }
 #undef WOL_LLM_ISSUE
