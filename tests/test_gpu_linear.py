@@ -304,7 +304,7 @@ def test_calls_replay_correctly_from_a_hip_graph(device):
     # Every entry point is stream-ordered and allocation-free, so a captured
     # sequence must replay to the eager results: quantise (per-channel, with its
     # scratch), decode, the small-M GEMM with its K runs and reduction, the
-    # prefill GEMM.  Replayed three times with eager work in between.
+    # prefill GEMM, llm_int8_linear.  Replayed three times with eager work in between.
     import torch
     from paddle_amd.nn import quant as Q
 
@@ -319,7 +319,11 @@ def test_calls_replay_correctly_from_a_hip_graph(device):
         c4, s4 = Q.weight_quantize(w, algo="weight_only_int4", group_size=128)
         outs = [Q.weight_only_linear(x, codes, None, scale, "int8", None, -1) for x in xs.values()]
         outs += [Q.weight_only_linear(x, c4, None, s4, "int4", None, 128) for x in xs.values()]
-        return [codes, scale, c4, s4] + outs
+        # llm_int8_linear: one row (single-workgroup activation stages, K runs), 40 rows (K runs, with
+        # threshold 3 more outlier columns than the epilogue takes: the outlier kernel), 300 rows (fused)
+        lw, ls = Q.weight_quantize(w, algo="llm.int8")
+        outs += [Q.llm_int8_linear(x, lw, None, ls, 3.0) for x in xs.values()]
+        return [codes, scale, c4, s4, lw, ls] + outs
 
     eager = [t.clone() for t in work()]
     torch.cuda.synchronize()
