@@ -344,10 +344,9 @@ __device__ inline uint16_t merge_plain(int acc, float range, float ws, bool has_
 // columns' product (when there are any: out of LDS if xs is given, else as
 // the outlier kernel left it in the output's own place) and one 16-byte store.  ws and bias hold the eight columns' values.
 template <int DT>
-__device__ inline void finish8(const Epi& e, int cnt, int m, int nn, i32x4 s0, i32x4 s1, const float* ws,
-                               const float* bias, const float* xs, int xs_stride, const float* wd,
-                               int wd_stride) {
-  const float range = e.ranges[m];
+__device__ inline void finish8(const Epi& e, int cnt, int m, int nn, float range, i32x4 s0, i32x4 s1,
+                               const float* ws, const float* bias, const float* xs, int xs_stride,
+                               const float* wd, int wd_stride) {
   u32x4 o;
   if (cnt == 0) {  // uniform: the count is one value for the whole launch
 #pragma unroll
@@ -649,9 +648,16 @@ __global__ __launch_bounds__(WM* WN * 64) __attribute__((amdgpu_waves_per_eu(2))
   const int cgrp = (lane & 3) * 8;  // first of this lane's eight columns inside the block
   // few outlier columns: their activations (this tile's rows) and dequantised
   // weights (this tile's columns) go to LDS behind the slabs, as floats
-  float* xs = reinterpret_cast<float*>(smem + NW * 32 * kSlabRow * 4);  // [cnt][BM]
-  float* wdl = xs + p.cap * BM;                                         // [cnt][BN]
+  float* rng = reinterpret_cast<float*>(smem + NW * 32 * kSlabRow * 4);  // [BM]: the tile's row ranges
+  float* xs = rng + BM;                                                  // [cnt][BM]
+  float* wdl = xs + p.cap * BM;                                          // [cnt][BN]
   const bool fused = !RUNS && cnt > 0 && cnt <= p.cap;
+  if (!RUNS) {
+    // (read per row out of global memory inside the row loop they cost a
+    // memory latency per row, sixteen in a row per wavefront)
+    for (int i = tid; i < BM; i += NW * 64) rng[i] = e.ranges[m0 + i < M ? m0 + i : M - 1];
+    if (!fused) __syncthreads();
+  }
   if (fused) {
     for (int i = tid; i < cnt * BM; i += NW * 64) {
       const int j = i / BM;
@@ -695,7 +701,7 @@ __global__ __launch_bounds__(WM* WN * 64) __attribute__((amdgpu_waves_per_eu(2))
           *reinterpret_cast<i32x4*>(dst + 4) = s1;
           continue;
         }
-        finish8<DT>(e, cnt, m, nn, s0, s1, ws, bias, fused ? xs + (wm * TM + a) * 32 + row : nullptr, BM,
+        finish8<DT>(e, cnt, m, nn, rng[(wm * TM + a) * 32 + row], s0, s1, ws, bias, fused ? xs + (wm * TM + a) * 32 + row : nullptr, BM,
                     wdl + (wn * TN + c) * 32 + cgrp, BN);
       }
     }
@@ -719,7 +725,7 @@ __global__ __launch_bounds__(256) void llm_merge_kernel(const int32_t* __restric
   }
   float ws[8], bias[8];
   load_ws_bias8<DT>(e, nn, ws, bias);
-  finish8<DT>(e, *e.count, m, nn, s0, s1, ws, bias, nullptr, 0, nullptr, 0);
+  finish8<DT>(e, *e.count, m, nn, e.ranges[m], s0, s1, ws, bias, nullptr, 0, nullptr, 0);
 }
 
 inline void allow_lds(const void* kern, size_t lds, std::atomic<uint32_t>& done) {
@@ -826,7 +832,8 @@ template <int DT, int WM, int WN, int TM, int TN, int TK, int STAGES, bool RUNS>
 int launch_gemm(const GemmParams& p, int runs, hipStream_t stream) {
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
   constexpr size_t lds = static_cast<size_t>(STAGES) * (BM + BN) * TK;
-  static_assert(lds >= static_cast<size_t>(WM * WN) * 32 * 40 * 4, "the epilogue's slabs must fit the stages");
+  static_assert(lds >= static_cast<size_t>(WM * WN) * 32 * 40 * 4 + BM * 4,
+                "the epilogue's slabs and row ranges must fit the stages");
   static std::atomic<uint32_t> done{0};
   auto kern = llm_gemm_kernel<DT, WM, WN, TM, TN, TK, STAGES, RUNS>;
   allow_lds(reinterpret_cast<const void*>(kern), lds, done);
@@ -864,7 +871,7 @@ int fused_cap(const Plan& pl) {
   if (pl.runs > 1) return 0;  // the merge kernel reads the outlier kernel's product
   const bool eight = pl.bn == 256;  // the configurations of eight wavefronts
   const int64_t lds = static_cast<int64_t>(pl.bm == 256 && eight ? 2 : 3) * (pl.bm + pl.bn) * pl.tk;
-  const int64_t room = lds - (eight ? 8 : 4) * 32 * 40 * 4;
+  const int64_t room = lds - (eight ? 8 : 4) * 32 * 40 * 4 - pl.bm * 4;  // slabs, row ranges
   const int64_t cap = room / ((pl.bm + pl.bn) * 4);
   return static_cast<int>(cap > 32 ? 32 : (cap < 0 ? 0 : cap));
 }
