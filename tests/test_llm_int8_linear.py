@@ -37,6 +37,23 @@ def _act(M, K, dt, seed, kind):
     return H.f32_to_bits(x, dt)
 
 
+def _adversarial_act(M, K, dt, seed):
+    """Rows of zeros, negative zeros, one huge element, values on the threshold and on quantisation ties, tiny and
+    subnormal rows: the corners of the activation quantiser."""
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((M, K), dtype=np.float32)
+    x[0] = 0.0                                     # range 0: 0 * inf, codes 0
+    x[1 % M] = -0.0
+    x[2 % M, 5] = 6.0                              # exactly the threshold: not an outlier (compare is >)
+    x[3 % M, 9] = 60000.0 if dt == H.F16 else 3.0e38
+    x[4 % M] = np.float32(2.0 ** -20) * rng.standard_normal(K).astype(np.float32)   # tiny row
+    x[5 % M] = np.float32(6.0e-8 if dt == H.F16 else 1.0e-39) * rng.integers(-3, 4, K).astype(np.float32)  # subnormal T
+    x[6 % M] = np.float32(1.0)                     # every element the row maximum: codes 127
+    x[6 % M, ::2] = np.float32(-0.5)               # x * 127 / range = -63.5: the only exact tie a power-of-two range has
+    x[7 % M, :] = np.float32(-5.5)
+    return H.f32_to_bits(x, dt)
+
+
 def _round_half_away(a64):
     return np.sign(a64) * np.floor(np.abs(a64) + 0.5)
 
@@ -107,6 +124,40 @@ def test_oracle_matches_numpy_statement(oracle, dt, case):
     assert np.array_equal(o["out"], r["out"])
     if kind != "uniform" and thr < 100:
         assert r["outlier"].any()
+
+
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+def test_oracle_matches_numpy_statement_on_corner_cases(oracle, dt):
+    M, K, N = 8, 128, 32
+    _, w_nk, ws = _weights(K, N, dt, seed=21)
+    xb = _adversarial_act(M, K, dt, seed=22)
+    bb = H.make_bias(N, dt, seed=3, std=1.0)
+    o = oracle.llm_int8_linear(xb, w_nk, bb, ws, 6.0, dt)
+    r = np_llm_int8(xb, w_nk, bb, ws, 6.0, dt)
+    for key in ("outlier", "ranges", "qx", "acc", "out"):
+        assert np.array_equal(o[key], r[key]), key
+    assert not o["qx"][0].any() and not o["qx"][1].any()
+    assert not o["outlier"][5] and o["outlier"][9]
+    assert set(np.unique(o["qx"][6][~o["outlier"]]).tolist()) <= {-64, 127}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+@pytest.mark.parametrize("M", [8, 40, 200])
+def test_gpu_llm_int8_linear_corner_cases_bit_exact(device, oracle, dt, M):
+    import gpu_calls as G
+
+    K, N = 128, 48
+    print("llm_int8 corner cases M", M, "dtype", dt, flush=True)
+    _, w_nk, ws = _weights(K, N, dt, seed=21)
+    xb = _adversarial_act(M, K, dt, seed=22)
+    bb = H.make_bias(N, dt, seed=3, std=1.0)
+    o = oracle.llm_int8_linear(xb, w_nk, bb, ws, 6.0, dt)
+    got, st = G.llm_int8_linear(xb, w_nk, bb, ws, 6.0, dt, stages=True)
+    assert np.array_equal(st["ranges"], o["ranges"])
+    assert np.array_equal(st["outlier"], o["outlier"])
+    assert np.array_equal(st["qx"], o["qx"])
+    assert np.array_equal(got, o["out"])
 
 
 @pytest.mark.parametrize("dt", [H.F16, H.BF16])
