@@ -241,7 +241,8 @@ def main():
             "ms_per_step": round(llm_s * 1e3, 4),
             "steps": args.prefill_steps,
             "roofline": {"bound": "mfma", "achieved": round(llm_tops, 2), "peak": MFMA_INT8_PEAK_TOPS,
-                         "unit": "TOP/s", "frac": round(llm_tops / MFMA_INT8_PEAK_TOPS, 4), "traffic": None,
+                         "unit": "TOP/s", "frac": round(llm_tops / MFMA_INT8_PEAK_TOPS, 4),
+                         "traffic": _load_traffic().get("llm_int8_gemm_bytes_per_launch"),
                          "kernel": "wol::llm_gemm_kernel<1, 2, 4, 2, 2, 128, 3, false> (128x256 tiles, "
                                    "v_mfma_i32_32x32x32_i8)"},
         }
