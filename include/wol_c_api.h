@@ -239,7 +239,8 @@ int wol_apply_per_channel_scale(const void* x, const void* scales, int dtype,
  * than the one its quantiser writes; this library indexes weight[n,k] plainly,
  * as the operator's description and the reference's own test
  * (test/quantization/test_llm_int8_linear.py:84-111) have it.
- * Requires K % 64 == 0 and N % 16 == 0 (what weight_quantize accepts); x,
+ * Requires K % 64 == 0, K <= 262144 and N % 16 == 0 (what weight_quantize
+ * accepts, and an outlier mask that fits the LDS); x,
  * weight, weight_scale, out and workspace 16-byte aligned; out must not
  * overlap an input (with many outlier columns their product waits in out
  * until it is merged).  The workspace is

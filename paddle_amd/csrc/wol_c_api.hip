@@ -231,14 +231,18 @@ int wol_apply_per_channel_scale(const void* x, const void* scales, int dtype, in
   return wol::launch_prescale(x, scales, dtype, rows, cols, out, static_cast<hipStream_t>(stream));
 }
 
+// the outlier mask of a call (K / 32 words) is kept in LDS by two of its kernels
+constexpr int64_t kLlmInt8MaxK = 262144;
+
 size_t wol_llm_int8_linear_workspace(int64_t M, int64_t K, int64_t N) {
   if (check_problem(WOL_DTYPE_F16, K, N, 8, -1) != WOL_OK || M <= 0 || M > (int64_t{1} << 24)) return 0;
+  if (K > kLlmInt8MaxK) return 0;
   return wol::llm_int8_workspace(M, K, N);
 }
 
 int wol_llm_int8_linear_stage_offsets(int64_t M, int64_t K, int64_t N, int64_t* offsets) {
   if (offsets == nullptr) return WOL_ERR_NULL_POINTER;
-  if (check_problem(WOL_DTYPE_F16, K, N, 8, -1) != WOL_OK || M <= 0 || M > (int64_t{1} << 24))
+  if (check_problem(WOL_DTYPE_F16, K, N, 8, -1) != WOL_OK || M <= 0 || M > (int64_t{1} << 24) || K > kLlmInt8MaxK)
     return WOL_ERR_BAD_SHAPE;
   wol::llm_int8_workspace_offsets(M, K, N, offsets);
   return WOL_OK;
@@ -250,6 +254,7 @@ int wol_llm_int8_linear(const void* x, const void* weight, const void* bias, con
   const int rc = check_problem(dtype, K, N, 8, -1);
   if (rc != WOL_OK) return rc;
   if (M < 0 || M > (int64_t{1} << 24)) return WOL_ERR_BAD_SHAPE;
+  if (M * N > (int64_t{1} << 40) || K > kLlmInt8MaxK) return WOL_ERR_BAD_SHAPE;  // tile counts in int32; mask in LDS
   if (M == 0) return WOL_OK;  // empty batch: nothing to write
   if (x == nullptr || weight == nullptr || weight_scale == nullptr || out == nullptr)
     return WOL_ERR_NULL_POINTER;

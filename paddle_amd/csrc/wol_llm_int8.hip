@@ -6,13 +6,14 @@
 // Stages (paddle/phi/kernels/impl/llm_int8_matmul_kernel_impl.h:560-690 runs
 // the same ones as separate kernels plus two library GEMMs and a device-to-host
 // copy of the outlier count; here nothing returns to the host):
-//   clear   : outlier bit mask and count to zero
 //   rowmax  : range[m] = max |x[m,k]| over the elements not above the
-//             threshold; bit k of the mask set where any |x[m,k]| > threshold
-//             (ReduceAbsMaxKernel, :221-268)
+//             threshold; bit k set where any |x[m,k]| > threshold
+//             (ReduceAbsMaxKernel, :221-268), per workgroup in LDS
+//   mask    : ORs the workgroups' bits into the mask
 //   quant   : qx = 0 in outlier columns, else clip(round(x * 127 * (1/range)))
 //             (QuantActKernel :270-303, QuantFunc :153-164); one extra
 //             workgroup turns the mask into an ascending list of columns
+//             (one or two rows: these three as one single-workgroup kernel)
 //   outlier : sub = T(sum over the outlier columns of x * T(w * wscale)), fp32
 //             sum in ascending column order; leaves at once without outliers
 //   gemm    : acc = qx . w^T in int32 on v_mfma_i32_32x32x32_i8, both operands
@@ -46,76 +47,73 @@ __device__ inline void wait_vmcnt() {
 // ---------------------------------------------------------------------------
 // activation side
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void llm_clear_kernel(int32_t* mask, int nwords, int32_t* count) {
-  const int i = blockIdx.x * 256 + threadIdx.x;
-  if (i < nwords) mask[i] = 0;
-  if (i == 0) *count = 0;
-}
-
-// A workgroup takes kRowsPerGroup rows and a thread the same columns of each,
-// so that a column's outlier bits are ORed over the rows in registers and
-// reach the mask as one atomic per workgroup (outlier columns tend to be the
-// same in every row).
-constexpr int kRowsPerGroup = 4;
-// The mask is kept in kMaskCopies copies, workgroup g of the row kernel ORing
-// into copy g % kMaskCopies: atomics on one word serialise (about 50 ns each
-// across the XCDs), and this many fewer meet on a hot column's word.  Readers
-// OR the copies; the list kernel leaves the combined mask in copy 0.
-constexpr int kMaskCopies = 8;
+// Row ranges and outlier bits.  A workgroup takes a run of rows, four at a time,
+// and a thread the same columns of each (16-byte loads); the outlier bits of
+// the run are ORed in an LDS mask and leave as the workgroup's own row of
+// `part` -- no global atomics: device-wide atomics on one word serialise at
+// 100-150 ns each across the XCDs, and outlier columns are the same in most
+// rows (with them this kernel took 15 us for 2048 rows x 4096).  The mask
+// kernel below ORs the rows of `part`.
+constexpr int kRowChunk = 4;
+constexpr int kMaxRowGroups = 512;
 
 template <int DT>
 __global__ __launch_bounds__(256) void llm_rowmax_kernel(const uint16_t* __restrict__ x, float threshold, int M,
-                                                         int K, float* __restrict__ ranges,
-                                                         int32_t* mask) {
-  __shared__ float part[4][kRowsPerGroup];
+                                                         int K, int rows_per_group, float* __restrict__ ranges,
+                                                         uint32_t* __restrict__ part) {
+  extern __shared__ uint32_t smask[];  // K / 32 words
+  __shared__ float red[4][kRowChunk];
   const float thr = to_f32<DT>(from_f32_rne<DT>(threshold));  // the comparison is made in T
-  const int m0 = blockIdx.x * kRowsPerGroup;
-  mask += static_cast<int64_t>(blockIdx.x % kMaskCopies) * (K / 32);
-  float mx[kRowsPerGroup];
-#pragma unroll
-  for (int r = 0; r < kRowsPerGroup; ++r) mx[r] = 0.0f;
-  for (int k0 = threadIdx.x * 8; k0 < K; k0 += 256 * 8) {
-    u32x4 v[kRowsPerGroup];
-#pragma unroll
-    for (int r = 0; r < kRowsPerGroup; ++r) {
-      const int m = m0 + r < M ? m0 + r : M - 1;  // past the end: the last row again
-      v[r] = *reinterpret_cast<const u32x4*>(x + static_cast<int64_t>(m) * K + k0);
-    }
-    uint32_t bits = 0;
-#pragma unroll
-    for (int r = 0; r < kRowsPerGroup; ++r) {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        float a = fabsf(to_f32<DT>(static_cast<uint16_t>(v[r][i >> 1] >> (16 * (i & 1)))));
-        if (a > thr) {
-          bits |= 1u << i;
-          a = 0.0f;
-        }
-        mx[r] = a > mx[r] ? a : mx[r];
-      }
-    }
-    if (bits != 0) {
-      // skip the atomic where the bits are already set (a stale read only costs an atomic)
-      const int32_t want = static_cast<int32_t>(bits << (k0 & 31));
-      if ((__builtin_nontemporal_load(&mask[k0 >> 5]) & want) != want) atomicOr(&mask[k0 >> 5], want);
-    }
-  }
-#pragma unroll
-  for (int r = 0; r < kRowsPerGroup; ++r) {
-#pragma unroll
-    for (int d = 32; d > 0; d >>= 1) {
-      const float o = __shfl_xor(mx[r], d, 64);
-      mx[r] = o > mx[r] ? o : mx[r];
-    }
-    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6][r] = mx[r];
-  }
+  const int nwords = K / 32;
+  for (int w = threadIdx.x; w < nwords; w += 256) smask[w] = 0u;
   __syncthreads();
-  if (threadIdx.x < kRowsPerGroup && m0 + threadIdx.x < M) {
-    float r = part[0][threadIdx.x];
+  const int m_begin = blockIdx.x * rows_per_group;
+  const int m_end = m_begin + rows_per_group < M ? m_begin + rows_per_group : M;
+  for (int m0 = m_begin; m0 < m_end; m0 += kRowChunk) {
+    float mx[kRowChunk];
 #pragma unroll
-    for (int i = 1; i < 4; ++i) r = part[i][threadIdx.x] > r ? part[i][threadIdx.x] : r;
-    ranges[m0 + threadIdx.x] = r;
+    for (int r = 0; r < kRowChunk; ++r) mx[r] = 0.0f;
+    for (int k0 = threadIdx.x * 8; k0 < K; k0 += 256 * 8) {
+      u32x4 v[kRowChunk];
+#pragma unroll
+      for (int r = 0; r < kRowChunk; ++r) {
+        const int m = m0 + r < m_end ? m0 + r : m_end - 1;  // past the end: the last row again
+        v[r] = *reinterpret_cast<const u32x4*>(x + static_cast<int64_t>(m) * K + k0);
+      }
+      uint32_t bits = 0;
+#pragma unroll
+      for (int r = 0; r < kRowChunk; ++r) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          float a = fabsf(to_f32<DT>(static_cast<uint16_t>(v[r][i >> 1] >> (16 * (i & 1)))));
+          if (a > thr) {
+            bits |= 1u << i;
+            a = 0.0f;
+          }
+          mx[r] = a > mx[r] ? a : mx[r];
+        }
+      }
+      if (bits != 0) atomicOr(&smask[k0 >> 5], bits << (k0 & 31));
+    }
+#pragma unroll
+    for (int r = 0; r < kRowChunk; ++r) {
+#pragma unroll
+      for (int d = 32; d > 0; d >>= 1) {
+        const float o = __shfl_xor(mx[r], d, 64);
+        mx[r] = o > mx[r] ? o : mx[r];
+      }
+      if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6][r] = mx[r];
+    }
+    __syncthreads();
+    if (threadIdx.x < kRowChunk && m0 + threadIdx.x < m_end) {
+      float r = red[0][threadIdx.x];
+#pragma unroll
+      for (int i = 1; i < 4; ++i) r = red[i][threadIdx.x] > r ? red[i][threadIdx.x] : r;
+      ranges[m0 + threadIdx.x] = r;
+    }
+    __syncthreads();  // red is reused by the next four rows
   }
+  for (int w = threadIdx.x; w < nwords; w += 256) part[static_cast<int64_t>(blockIdx.x) * nwords + w] = smask[w];
 }
 
 // QuantFunc (:153-164).  NaN (0 * inf in a row whose range is 0) becomes 0.
@@ -248,24 +246,42 @@ __global__ __launch_bounds__(kSmallThreads) void llm_act_small_kernel(const uint
   }
 }
 
+// ORs the row kernel's partial masks (groups rows of K / 32 words) into the
+// mask.  A workgroup takes four words; 64 threads per word each take every
+// 64th group and meet in LDS.
+__global__ __launch_bounds__(256) void llm_mask_kernel(const uint32_t* __restrict__ part, int groups, int K,
+                                                       int32_t* __restrict__ mask) {
+  __shared__ uint32_t red[64][4];
+  const int tid = threadIdx.x;
+  const int nwords = K / 32;
+  const int wl = tid & 3, sub = tid >> 2;
+  const int w = blockIdx.x * 4 + wl;
+  uint32_t v = 0u;
+  if (w < nwords)
+    for (int g = sub; g < groups; g += 64) v |= part[static_cast<int64_t>(g) * nwords + w];
+  red[sub][wl] = v;
+  __syncthreads();
+  if (tid < 4 && w < nwords) {
+    uint32_t o = 0u;
+#pragma unroll
+    for (int i = 0; i < 64; ++i) o |= red[i][tid];
+    mask[w] = static_cast<int32_t>(o);
+  }
+}
+
+// Activation codes; the last workgroup instead turns the mask into the
+// ascending list of outlier columns.
 template <int DT>
 __global__ __launch_bounds__(256) void llm_quant_kernel(const uint16_t* __restrict__ x,
                                                         const float* __restrict__ ranges,
-                                                        int32_t* mask, int M, int K,
+                                                        const int32_t* __restrict__ mask, int M, int K,
                                                         int8_t* __restrict__ qx, int32_t* __restrict__ count,
                                                         int32_t* __restrict__ list) {
   const int tid = threadIdx.x;
   if (blockIdx.x == gridDim.x - 1) {
     __shared__ int scan[256];
     __shared__ int base_s;
-    const int nwords = K / 32;
-    build_list(nwords, [&](int w) {
-      uint32_t word = 0u;
-#pragma unroll
-      for (int r = 0; r < kMaskCopies; ++r) word |= static_cast<uint32_t>(mask[r * nwords + w]);
-      mask[w] = static_cast<int32_t>(word);  // the combined mask, for whoever inspects the stages
-      return word;
-    }, list, count, scan, &base_s);
+    build_list(K / 32, [&](int w) { return static_cast<uint32_t>(mask[w]); }, list, count, scan, &base_s);
     return;
   }
   const int64_t stride = static_cast<int64_t>(gridDim.x - 1) * 256;
@@ -277,10 +293,7 @@ __global__ __launch_bounds__(256) void llm_quant_kernel(const uint16_t* __restri
     const int k = static_cast<int>(e - static_cast<int64_t>(m) * K);
     const u32x4 lo = *reinterpret_cast<const u32x4*>(x + e);
     const u32x4 hi = *reinterpret_cast<const u32x4*>(x + e + 8);
-    uint32_t mword = 0u;
-#pragma unroll
-    for (int r = 0; r < kMaskCopies; ++r) mword |= static_cast<uint32_t>(mask[r * (K / 32) + (k >> 5)]);
-    const uint32_t out_bits = mword >> (k & 31);
+    const uint32_t out_bits = static_cast<uint32_t>(mask[k >> 5]) >> (k & 31);
     const float inv = 1.0f / ranges[m];
     u32x4 q = {0u, 0u, 0u, 0u};
 #pragma unroll
@@ -800,6 +813,7 @@ Plan make_plan(int64_t M, int64_t K, int64_t N) {
 struct Workspace {
   float* ranges;
   int32_t* mask;
+  uint32_t* part;
   int32_t* count;
   int32_t* list;
   int8_t* qx;
@@ -815,7 +829,9 @@ Workspace carve(void* base, int64_t M, int64_t K, int64_t N, int runs) {
   w.ranges = reinterpret_cast<float*>(p + off);
   off += align256(M * 4);
   w.mask = reinterpret_cast<int32_t*>(p + off);
-  off += align256(K / 32 * 4 * kMaskCopies);
+  off += align256(K / 32 * 4);
+  w.part = reinterpret_cast<uint32_t*>(p + off);
+  off += align256(static_cast<int64_t>(kMaxRowGroups) * (K / 32) * 4);
   w.count = reinterpret_cast<int32_t*>(p + off);
   off += 256;
   w.list = reinterpret_cast<int32_t*>(p + off);
@@ -888,17 +904,23 @@ int run_llm_int8(const void* x, const void* weight, const void* bias, const floa
                        xs, threshold, static_cast<int>(M), static_cast<int>(K), ws.ranges, ws.mask, ws.qx, ws.count,
                        ws.list);
   }
-  const int nwords = static_cast<int>(K / 32) * kMaskCopies;
-  if (!small) hipLaunchKernelGGL(llm_clear_kernel, dim3((nwords + 255) / 256), dim3(256), 0, stream, ws.mask, nwords,
-                     ws.count);
-  if (!small) hipLaunchKernelGGL(llm_rowmax_kernel<DT>, dim3(static_cast<unsigned>((M + kRowsPerGroup - 1) / kRowsPerGroup)),
-                     dim3(256), 0, stream, xs, threshold, static_cast<int>(M), static_cast<int>(K), ws.ranges,
-                     ws.mask);
-  const int64_t nvec = M * K / 16;
-  int64_t qblocks = (nvec + 255) / 256;
-  if (qblocks > 8192) qblocks = 8192;
-  if (!small) hipLaunchKernelGGL(llm_quant_kernel<DT>, dim3(static_cast<unsigned>(qblocks + 1)), dim3(256), 0, stream, xs,
-                     ws.ranges, ws.mask, static_cast<int>(M), static_cast<int>(K), ws.qx, ws.count, ws.list);
+  if (!small) {
+    // at most kMaxRowGroups workgroups, each a whole number of four-row chunks
+    int64_t rows_per_group = (M + kMaxRowGroups - 1) / kMaxRowGroups;
+    rows_per_group = (rows_per_group + kRowChunk - 1) / kRowChunk * kRowChunk;
+    const int groups = static_cast<int>((M + rows_per_group - 1) / rows_per_group);
+    const size_t mask_lds = static_cast<size_t>(K / 32) * 4;
+    hipLaunchKernelGGL(llm_rowmax_kernel<DT>, dim3(static_cast<unsigned>(groups)), dim3(256), mask_lds, stream, xs,
+                       threshold, static_cast<int>(M), static_cast<int>(K), static_cast<int>(rows_per_group),
+                       ws.ranges, ws.part);
+    hipLaunchKernelGGL(llm_mask_kernel, dim3(static_cast<unsigned>((K / 32 + 3) / 4)), dim3(256), 0, stream, ws.part,
+                       groups, static_cast<int>(K), ws.mask);
+    const int64_t nvec = M * K / 16;
+    int64_t qblocks = (nvec + 255) / 256;
+    if (qblocks > 8192) qblocks = 8192;
+    hipLaunchKernelGGL(llm_quant_kernel<DT>, dim3(static_cast<unsigned>(qblocks + 1)), dim3(256), 0, stream, xs,
+                       ws.ranges, ws.mask, static_cast<int>(M), static_cast<int>(K), ws.qx, ws.count, ws.list);
+  }
   GemmParams p;
   p.qx = ws.qx;
   p.e = Epi{xs, static_cast<const int8_t*>(weight), wscale, ws.ranges, static_cast<const uint16_t*>(bias),
