@@ -478,6 +478,7 @@ struct GemmParams {
   Epi e;
   int32_t* acc;      // [runs][M,N] int32, one slab per K run; only with K runs
   int nbx, nby;      // tiles along N and M
+  int n_lo, n_hi;    // columns [n_lo, n_hi) of the output belong to this launch
   int tiles_per_run; // k tiles per K run
   int cap;  // outlier columns the epilogue takes through LDS itself; more come from the outlier kernel
 };
@@ -527,7 +528,7 @@ __global__ __launch_bounds__(WM* WN * 64) __attribute__((amdgpu_waves_per_eu(2))
     bx = t / p.nby;
     by = t % p.nby;
   }
-  const int m0 = by * BM, n0 = bx * BN;
+  const int m0 = by * BM, n0 = p.n_lo + bx * BN;
   const int ktiles = K / kTK;
   const int t0 = run * p.tiles_per_run;
   const int niter = (ktiles - t0) < p.tiles_per_run ? (ktiles - t0) : p.tiles_per_run;
@@ -689,7 +690,7 @@ __global__ __launch_bounds__(WM* WN * 64) __attribute__((amdgpu_waves_per_eu(2))
 #pragma unroll
   for (int c = 0; c < TN; ++c) {
     const int n = n0 + (wn * TN + c) * 32 + cgrp;
-    const bool n_ok = n < N;  // N is a multiple of 16: eight columns are all inside or all outside
+    const bool n_ok = n < p.n_hi;  // a multiple of 16: eight columns are all inside or all outside
     const int nn = n_ok ? n : 0;
     float ws[8], bias[8];
     if (!RUNS) load_ws_bias8<DT>(e, nn, ws, bias);
@@ -755,6 +756,7 @@ inline int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
 struct Plan {
   int bm, bn;     // tile
   int tk;         // k bytes per tile row
+  int whole_cols; // many rows: the first whole_cols columns get 256x256 tiles, the rest 128x256
   int runs;       // K runs (1: the GEMM writes the output itself)
   int tiles_per_run;
 };
@@ -776,6 +778,7 @@ inline int num_cus() {
 // once each) stay below the weight bytes.
 Plan make_plan(int64_t M, int64_t K, int64_t N) {
   Plan pl;
+  pl.whole_cols = 0;
   const int tk = K % 128 == 0 ? 128 : 64;
   const int64_t ktiles = K / tk;
   int64_t runs = 1;
@@ -788,10 +791,20 @@ Plan make_plan(int64_t M, int64_t K, int64_t N) {
     pl.bm = 256;
     pl.bn = tk == 128 ? 256 : 128;
     if (tk == 128) {
+      // a launch takes ceil(tiles / CUs) tile times: the columns are shared
+      // out so that whole tiles fill whole rounds of the CUs
       const int64_t cus = num_cus();
-      const int64_t cols = (N + 255) / 256;
-      const int64_t whole = ((M + 255) / 256) * cols, half = ((M + 127) / 128) * cols;
-      if (11 * ((half + cus - 1) / cus) < 20 * ((whole + cus - 1) / cus)) pl.bm = 128;
+      const int64_t cols = (N + 255) / 256, rows256 = (M + 255) / 256, rows128 = (M + 127) / 128;
+      int64_t best_c = cols, best_t = INT64_MAX;
+      for (int64_t c = cols; c >= 0; --c) {
+        const int64_t t = 20 * ((c * rows256 + cus - 1) / cus) + 11 * (((cols - c) * rows128 + cus - 1) / cus);
+        if (t < best_t) {
+          best_t = t;
+          best_c = c;
+        }
+      }
+      pl.whole_cols = static_cast<int>(best_c * 256 < N ? best_c * 256 : N);
+      if (best_c == 0) pl.bm = 128;
     }
   } else {
     pl.bm = M > 64 ? 128 : (M > 32 ? 64 : 32);
@@ -927,13 +940,35 @@ int run_llm_int8(const void* x, const void* weight, const void* bias, const floa
             ws.count, ws.list, static_cast<uint16_t*>(out), static_cast<int>(M), static_cast<int>(K),
             static_cast<int>(N)};
   p.acc = ws.acc;
+  p.n_lo = 0;
+  p.n_hi = static_cast<int>(N);
   p.nbx = static_cast<int>((N + pl.bn - 1) / pl.bn);
   p.nby = static_cast<int>((M + pl.bm - 1) / pl.bm);
   p.tiles_per_run = pl.tiles_per_run;
   p.cap = fused_cap(pl);
+  if (pl.runs == 1 && pl.bm == 256 && pl.bn == 256 && pl.whole_cols < N) {
+    Plan half = pl;
+    half.bm = 128;
+    const int c = fused_cap(half);  // both launches and the outlier kernel go by one limit
+    p.cap = c < p.cap ? c : p.cap;
+  }
   hipLaunchKernelGGL(llm_outlier_kernel<DT>, dim3(static_cast<unsigned>(((N + 255) / 256) * ((M + 63) / 64))),
                      dim3(256), 0, stream, p.e, p.cap);
   if (check_launch() != WOL_OK) return WOL_ERR_HIP;
+  if (pl.runs == 1 && pl.bm == 256 && pl.bn == 256 && pl.whole_cols < N) {
+    // 256x256 tiles on the first columns, 128x256 tiles on the rest
+    p.n_hi = pl.whole_cols;
+    p.nbx = pl.whole_cols / 256;
+    const int rc = launch_gemm_tk<DT, false>(p, pl, stream);
+    if (rc != WOL_OK) return rc;
+    Plan half = pl;
+    half.bm = 128;
+    p.n_lo = pl.whole_cols;
+    p.n_hi = static_cast<int>(N);
+    p.nbx = static_cast<int>((N - pl.whole_cols + 255) / 256);
+    p.nby = static_cast<int>((M + 127) / 128);
+    return launch_gemm_tk<DT, false>(p, half, stream);
+  }
   if (pl.runs == 1) return launch_gemm_tk<DT, false>(p, pl, stream);
   const int rc = launch_gemm_tk<DT, true>(p, pl, stream);
   if (rc != WOL_OK) return rc;
