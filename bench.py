@@ -243,8 +243,9 @@ def main():
             "roofline": {"bound": "mfma", "achieved": round(llm_tops, 2), "peak": MFMA_INT8_PEAK_TOPS,
                          "unit": "TOP/s", "frac": round(llm_tops / MFMA_INT8_PEAK_TOPS, 4),
                          "traffic": _load_traffic().get("llm_int8_gemm_bytes_per_launch"),
-                         "kernel": "wol::llm_gemm_kernel<1, 2, 4, 2, 2, 128, 3, false> (128x256 tiles, "
-                                   "v_mfma_i32_32x32x32_i8)"},
+                         "kernel": "wol::llm_gemm_kernel<1, 2, 4, 4, 2, 128, 2, false> (256x256 tiles on 8192 columns) "
+                                   "+ <1, 2, 4, 2, 2, 128, 3, false> (128x256 tiles on the rest), "
+                                   "v_mfma_i32_32x32x32_i8"},
         }
 
     # ---------------- CPU baseline + parity of the decode output ----------------

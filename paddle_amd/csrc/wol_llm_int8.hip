@@ -354,8 +354,9 @@ __device__ inline uint16_t merge_plain(int acc, float range, float ws, bool has_
 }
 
 // Eight neighbouring columns nn .. nn+7 of row m: the merge with the outlier
-// columns' product (when there are any: out of LDS if xs is given, else as
-// the outlier kernel left it in the output's own place) and one 16-byte store.  ws and bias hold the eight columns' values.
+// columns' product (when there are any: out of LDS if xs is given, computed on
+// the spot if wd_stride is negative, else as the outlier kernel left it in the
+// output's own place) and one 16-byte store.  ws and bias hold the eight columns' values.
 template <int DT>
 __device__ inline void finish8(const Epi& e, int cnt, int m, int nn, float range, i32x4 s0, i32x4 s1,
                                const float* ws, const float* bias, const float* xs, int xs_stride,
@@ -387,6 +388,22 @@ __device__ inline void finish8(const Epi& e, int cnt, int m, int nn, float range
       for (int i = 0; i < 4; ++i) {
         sub[i] += xv * w0[i];
         sub[4 + i] += xv * w1[i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sub[i] = to_f32<DT>(cast_out<DT>(sub[i]));
+  } else if (wd_stride < 0) {
+    // very few rows: straight from x and the weight, no outlier kernel ran
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sub[i] = 0.0f;
+#pragma unroll 1
+    for (int j = 0; j < cnt; ++j) {
+      const int kj = e.list[j];
+      const float xv = to_f32<DT>(e.x[static_cast<int64_t>(m) * e.K + kj]);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float w = static_cast<float>(e.w[static_cast<int64_t>(nn + i) * e.K + kj]);
+        sub[i] += xv * to_f32<DT>(cast_out<DT>(w * ws[i]));
       }
     }
 #pragma unroll
@@ -724,7 +741,8 @@ __global__ __launch_bounds__(WM* WN * 64) __attribute__((amdgpu_waves_per_eu(2))
 
 // Adds the K runs' int32 sums and finishes; one thread per eight columns.
 template <int DT>
-__global__ __launch_bounds__(256) void llm_merge_kernel(const int32_t* __restrict__ acc, int runs, Epi e) {
+__global__ __launch_bounds__(256) void llm_merge_kernel(const int32_t* __restrict__ acc, int runs, Epi e,
+                                                        int direct_outliers) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
   const int groups = e.N / 8;
   if (i >= static_cast<int64_t>(e.M) * groups) return;
@@ -739,7 +757,7 @@ __global__ __launch_bounds__(256) void llm_merge_kernel(const int32_t* __restric
   }
   float ws[8], bias[8];
   load_ws_bias8<DT>(e, nn, ws, bias);
-  finish8<DT>(e, *e.count, m, nn, e.ranges[m], s0, s1, ws, bias, nullptr, 0, nullptr, 0);
+  finish8<DT>(e, *e.count, m, nn, e.ranges[m], s0, s1, ws, bias, nullptr, 0, nullptr, direct_outliers ? -1 : 0);
 }
 
 inline void allow_lds(const void* kern, size_t lds, std::atomic<uint32_t>& done) {
@@ -952,8 +970,12 @@ int run_llm_int8(const void* x, const void* weight, const void* bias, const floa
     const int c = fused_cap(half);  // both launches and the outlier kernel go by one limit
     p.cap = c < p.cap ? c : p.cap;
   }
-  hipLaunchKernelGGL(llm_outlier_kernel<DT>, dim3(static_cast<unsigned>(((N + 255) / 256) * ((M + 63) / 64))),
-                     dim3(256), 0, stream, p.e, p.cap);
+  // up to four rows with K runs the merge kernel multiplies the outlier columns
+  // itself (a launch costs more than that work)
+  const bool direct = pl.runs > 1 && M <= 4;
+  if (!direct)
+    hipLaunchKernelGGL(llm_outlier_kernel<DT>, dim3(static_cast<unsigned>(((N + 255) / 256) * ((M + 63) / 64))),
+                       dim3(256), 0, stream, p.e, p.cap);
   if (check_launch() != WOL_OK) return WOL_ERR_HIP;
   if (pl.runs == 1 && pl.bm == 256 && pl.bn == 256 && pl.whole_cols < N) {
     // 256x256 tiles on the first columns, 128x256 tiles on the rest
@@ -974,7 +996,7 @@ int run_llm_int8(const void* x, const void* weight, const void* bias, const floa
   if (rc != WOL_OK) return rc;
   const int64_t total = M * (N / 8);
   hipLaunchKernelGGL(llm_merge_kernel<DT>, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, stream,
-                     ws.acc, pl.runs, p.e);
+                     ws.acc, pl.runs, p.e, direct ? 1 : 0);
   return check_launch();
 }
 

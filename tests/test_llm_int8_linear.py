@@ -236,6 +236,8 @@ GPU_CASES = [  # M, K, N, kind, threshold, bias
     (257, 64, 2048, "spiky", 6.0, True),      # one k tile; column tiles spread over the XCD bands
     (3, 64, 16, "normal", 0.0, True),         # every column an outlier
     (16, 4096, 512, "spiky", 6.0, True),      # K cut into runs
+    (1, 4096, 512, "spiky", 6.0, True),       # one row, K runs: the merge kernel multiplies the outlier columns itself
+    (4, 2048, 256, "normal", 2.0, False),     # four rows, K runs, most columns outliers
     (128, 2048, 272, "spiky", 6.0, True),     # 128-row tile, two runs
     (700, 512, 8192, "spiky", 6.0, True),     # 256x256 tiles
 ]
