@@ -619,9 +619,9 @@ __global__ __launch_bounds__(WM* WN * 64) __attribute__((amdgpu_waves_per_eu(2))
     // compiler wait for every load in flight, the prefetched tile included.
     wait_vmcnt<(kStages - 2) * kPerStage>();
     __builtin_amdgcn_s_barrier();
-    WOL_LLM_ISSUE(it + kStages - 1);  // into the stage every wavefront finished reading before the barrier
     const unsigned char* stage = smem + (it % kStages) * kStage;
-    // the fragments of k step ks + 1 are read while the MFMAs of step ks run
+    // the fragments of k step ks + 1 are read while the MFMAs of step ks run;
+    // those of step 0 while the next tile's loads are issued
     constexpr int KS = C / 2;
     i32x4 af[2][TM], bf[2][TN];
     {
@@ -631,6 +631,9 @@ __global__ __launch_bounds__(WM* WN * 64) __attribute__((amdgpu_waves_per_eu(2))
 #pragma unroll
       for (int c = 0; c < TN; ++c) bf[0][c] = *reinterpret_cast<const i32x4*>(stage + boff[c] + piece);
     }
+    __builtin_amdgcn_sched_barrier(0);
+    WOL_LLM_ISSUE(it + kStages - 1);  // into the stage every wavefront finished reading before the barrier
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       if (ks + 1 < KS) {
