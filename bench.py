@@ -3,19 +3,33 @@
 
 One "step" is one weight_only_linear call at M=1 on the headline shape
 (int4, group 128, K=4096, N=11008, bf16 activations): the bandwidth-bound
-decode GEMV.  The timed region holds exactly --steps such calls, captured into
-one HIP graph so the host's launch rate does not enter, rotating over enough
-distinct copies of the packed weight that neither L2 nor the 256 MB Infinity
-Cache can serve a repeat.  A second region times the compute-bound prefill
-GEMM (M=2048, int8 per-channel, K=4096, N=12288) and is reported under
-"prefill".  The CPU baseline (oracle quantize + dequantize + fp32 matmul on the
-host cores) is timed on rank 0 on the same arrays.
+decode GEMV.  --steps such calls are captured into one HIP graph, so the
+host's launch rate does not enter, rotating over enough distinct copies of the
+packed weight that neither L2 nor the 256 MB Infinity Cache can serve a
+repeat.  Whatever --steps/--warmup say, the graph is replayed untimed until at
+least 400 launches and 50 ms of load have run (the clocks need that to
+settle), then replayed REPLAYS times, each replay between its own pair of
+events on the launching stream; ms_per_step is the MEDIAN replay divided by
+--steps (the minimum is reported beside it).
+
+Beside the headline the line carries
+  prefill    the compute-bound GEMM (M=2048, int8 per-channel, K=4096,
+             N=12288) with an in-run ceiling: a register-only MFMA loop;
+  configs    one entry per configuration of BASELINE.json and row count, the
+             last one the 32-layer decoder stack as a sequence (decode steps
+             at M=8, one prefill chunk at M=1024);
+  llm_int8   the sibling op on the prefill shape;
+  cpu_baseline  the CPU oracle (quantize, dequantize) + fp32 BLAS matmul on
+             the host cores, on a bounded sample;
+  parity     the measured outputs against the oracle.  A parity failure makes
+             the run exit non-zero: no throughput is published for wrong results.
 
 Prints ONE JSON line.
 """
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -26,9 +40,11 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TF = 2500.0   # MI355X dense bf16 MFMA, published
 MFMA_INT8_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA, published
+REPLAYS = 7                  # timed replays of every graph (median and minimum are reported)
 
 DECODE = dict(M=1, K=4096, N=11008, bits=4, group_size=128, dtype="bfloat16")
 PREFILL = dict(M=2048, K=4096, N=12288, bits=8, group_size=-1, dtype="bfloat16")
+REL_L2_BAR = 1e-3
 
 
 def _load_traffic():
@@ -40,53 +56,182 @@ def _load_traffic():
     return {}
 
 
-def _quantize(torch, Q, w, bits, group_size):
+def _quantize(Q, w, bits, group_size):
     algo = "weight_only_int8" if bits == 8 else "weight_only_int4"
     return Q.weight_quantize(w, algo=algo, group_size=group_size)
 
 
-def _time_graph(torch, fn, steps, warmup):
-    """Run fn(i) warmup times eagerly, then capture steps calls into one graph
-    and time its replay with events on the launching stream.  The graph is
-    replayed untimed first (graph upload), as often as it takes to cover the
-    warm-up count in graph form too: the clocks need a few milliseconds of
-    load to settle, and eager launches of a 6 us kernel do not load the GPU."""
-    for i in range(warmup):
+def time_graph(torch, fn, launches, warm_launches=400, warm_ms=50.0, replays=REPLAYS, eager=False):
+    """fn(i) enqueues launch i on the current stream.  Captures `launches`
+    calls into one HIP graph, replays it untimed until both warm-up thresholds
+    are met, then times `replays` replays one by one (events on the current
+    stream).  Returns (median, minimum) seconds per replay."""
+    for i in range(3):
         fn(i)
     torch.cuda.synchronize()
-    g = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(g):
-        for i in range(steps):
-            fn(warmup + i)
+    if eager:
+        def run():
+            for i in range(launches):
+                fn(i)
+    else:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for i in range(launches):
+                fn(i)
+        run = g.replay
     torch.cuda.synchronize()
-    for _ in range(max(1, -(-warmup // steps))):
-        g.replay()
+    done, batch = 0, 1
+    t0 = time.perf_counter()
+    while True:
+        tb = time.perf_counter()
+        for _ in range(batch):
+            run()
+        torch.cuda.synchronize()
+        done += launches * batch
+        now = time.perf_counter()
+        if done >= warm_launches and (now - t0) * 1e3 >= warm_ms:
+            break
+        # replays go out in batches of about 5 ms so that the GPU stays loaded between host synchronisations
+        batch = int(min(256, max(1, 5e-3 / max((now - tb) / batch, 1e-6))))
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(replays)]
     torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
+    for e0, e1 in ev:
+        e0.record()
+        run()
+        e1.record()
     torch.cuda.synchronize()
-    e0.record()
-    g.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / 1e3  # seconds for `steps` launches
+    ts = [e0.elapsed_time(e1) / 1e3 for e0, e1 in ev]
+    return statistics.median(ts), min(ts)
 
 
-def _time_eager(torch, fn, steps, warmup):
-    for i in range(warmup):
-        fn(i)
-    torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for i in range(steps):
-        fn(warmup + i)
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / 1e3
+def _plan(_lib, M, K, N, bits, g):
+    """The kernel path wol_linear takes for a problem, as the library describes it."""
+    import ctypes
+
+    if not hasattr(_lib.lib, "wol_linear_plan"):
+        return None
+    buf = ctypes.create_string_buffer(256)
+    ws = _lib.lib.wol_linear_workspace(M, K, N, bits, g)
+    if _lib.lib.wol_linear_plan(M, K, N, bits, g, ws, buf, 256) != 0:
+        return None
+    return buf.value.decode()
 
 
-def cpu_baseline(np, torch, H, w_bits, x_bits, cfg, budget_s=25.0):
+def _device_weight(torch, K, N, tdtype, seed, dev, outlier_cols=0.0):
+    """W ~ N(0, 0.02) generated on the device (the configurations' weights are
+    too many for the host generator), optionally with a fraction of the columns
+    scaled x20, cast to T."""
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    w = torch.randn((K, N), generator=gen, device=dev, dtype=torch.float32) * 0.02
+    if outlier_cols > 0:
+        n = int(-(-outlier_cols * N // 1))
+        cols = torch.randperm(N, generator=gen, device=dev)[:n]
+        w[:, cols] *= 20.0
+    return w.to(tdtype)
+
+
+def bench_configs(torch, Q, _lib, dev, quick):
+    """One entry per BASELINE configuration and row count."""
+    bf16, f16 = torch.bfloat16, torch.float16
+    cases = [
+        ("c1", 4096, 4096, 8, -1, bf16, (1,), 0.0, False),
+        ("c2", 4096, 11008, 4, -1, bf16, (1, 4, 16), 0.0, True),
+        ("c2", 11008, 4096, 4, -1, bf16, (1, 4, 16), 0.0, True),
+        ("north-star decode", 4096, 11008, 4, 128, bf16, (1,), 0.0, False),
+        ("c3", 8192, 28672, 4, 128, f16, (1, 8, 32, 64), 0.01, False),
+        ("c4", 4096, 12288, 8, -1, bf16, (512, 2048, 8192), 0.0, False),
+    ]
+    out = []
+    for ci, (name, K, N, bits, g, tdt, Ms, outl, with_bias) in enumerate(cases):
+        w = _device_weight(torch, K, N, tdt, 2000 + ci, dev, outl)
+        codes, scale = _quantize(Q, w, bits, g)
+        del w
+        wbytes = K * N * bits // 8
+        ncopies = max(2, -(-640 * 1024 * 1024 // wbytes))
+        copies = [codes.clone() for _ in range(ncopies)]
+        scales = [scale.clone() for _ in range(ncopies)]
+        bias = (torch.randn(N, device=dev) * 0.01).to(tdt) if with_bias else None
+        wd = "int8" if bits == 8 else "int4"
+        for M in Ms:
+            x = torch.randn((M, K), device=dev, dtype=torch.float32).to(tdt)
+
+            def step(i, x=x):
+                j = i % ncopies
+                return Q.weight_only_linear(x, copies[j], bias, scales[j], wd, None, g)
+
+            flops = 2.0 * M * K * N
+            est_us = max(wbytes / 4e6, flops / 1.0e9)  # rough: 4 TB/s, 1 PFLOP/s
+            launches = int(min(200, max(10, 2000.0 / est_us)))
+            if quick:
+                launches = min(launches, 20)
+            med, mn = time_graph(torch, step, launches, warm_launches=2 * launches,
+                                 warm_ms=10.0 if quick else 30.0, replays=5)
+            us, us_min = med / launches * 1e6, mn / launches * 1e6
+            e = {"config": name, "M": M, "K": K, "N": N, "weights": "int%d" % bits, "group_size": g,
+                 "dtype": "bf16" if tdt == bf16 else "f16", "bias": with_bias,
+                 "us": round(us, 3), "us_min": round(us_min, 3), "launches_per_replay": launches,
+                 "weight_copies": ncopies}
+            if M <= 64:
+                gbs = wbytes / us / 1e3
+                e.update({"bound": "hbm", "achieved": round(gbs, 1), "unit": "GB/s",
+                          "frac": round(gbs / HBM_PEAK_GBS, 4)})
+            else:
+                tf = flops / us / 1e6
+                e.update({"bound": "mfma", "achieved": round(tf, 1), "unit": "TFLOP/s",
+                          "frac": round(tf / MFMA_BF16_PEAK_TF, 4)})
+            e["path"] = _plan(_lib, M, K, N, bits, g)
+            out.append(e)
+            del x
+        del copies, scales, codes, scale
+        torch.cuda.empty_cache()
+    return out
+
+
+def bench_decoder_stack(torch, Q, _lib, dev, quick):
+    """BASELINE configuration 5 as the sequence it describes: the four linears
+    of 32 LLaMA-7B decoder layers (int8, group 64, every layer its own random
+    weights), run back to back as decode steps at batch 8 and as one prefill
+    chunk of 1024 tokens.  Attention, norms and the rest of the model are not
+    part of this path; every linear reads a fixed random input of its width."""
+    layers = 8 if quick else 32
+    shapes = [("qkv", 4096, 12288), ("o", 4096, 4096), ("gate_up", 4096, 22016), ("down", 11008, 4096)]
+    g, bf16 = 64, torch.bfloat16
+    weights = []
+    for layer in range(layers):
+        for i, (_, K, N) in enumerate(shapes):
+            w = _device_weight(torch, K, N, bf16, 1234 + layer * 4 + i, dev)
+            weights.append((K, N) + tuple(_quantize(Q, w, 8, g)))
+            del w
+    wbytes = sum(K * N for K, N, _, _ in weights)
+    res = {"layers": layers, "linears_per_layer": [s[0] for s in shapes], "weights": "int8", "group_size": g,
+           "dtype": "bf16", "weight_bytes_per_step": wbytes}
+    for tag, M, reps in (("decode_M8", 8, 4), ("prefill_M1024", 1024, 1)):
+        xs = {K: torch.randn((M, K), device=dev, dtype=torch.float32).to(bf16) for K in (4096, 11008)}
+
+        def step(_i, xs=xs):
+            for K, N, codes, scale in weights:
+                Q.weight_only_linear(xs[K], codes, None, scale, "int8", None, g)
+
+        med, mn = time_graph(torch, step, reps, warm_launches=2 * reps, warm_ms=20.0, replays=5)
+        ms, ms_min = med / reps * 1e3, mn / reps * 1e3
+        flops = 2.0 * M * wbytes
+        r = {"M": M, "ms_per_step": round(ms, 4), "ms_per_step_min": round(ms_min, 4),
+             "launches_per_step": len(weights)}
+        if M <= 64:
+            ideal = wbytes / (HBM_PEAK_GBS * 1e9) * 1e3
+            r.update({"bound": "hbm", "achieved": round(wbytes / ms / 1e6, 1), "unit": "GB/s",
+                      "ideal_ms": round(ideal, 4), "frac": round(ideal / ms, 4)})
+        else:
+            ideal = flops / (MFMA_BF16_PEAK_TF * 1e12) * 1e3
+            r.update({"bound": "mfma", "achieved": round(flops / ms / 1e9, 1), "unit": "TFLOP/s",
+                      "ideal_ms": round(ideal, 4), "frac": round(ideal / ms, 4)})
+        r["paths"] = {s[0]: _plan(_lib, M, s[1], s[2], 8, g) for s in shapes}
+        res[tag] = r
+    return res
+
+
+def cpu_decode_baseline(np, torch, H, w_bits, x_bits, cfg, budget_s=10.0):
     """Oracle quantize (single thread, like the reference's CPU kernel) +
     dequantize to fp32 + fp32 matmul (torch CPU BLAS, all cores), on a bounded
     sample: the first N_s output columns of the decode weight."""
@@ -103,11 +248,11 @@ def cpu_baseline(np, torch, H, w_bits, x_bits, cfg, budget_s=25.0):
     x32 = torch.from_numpy(H.bits_to_f32(x_bits, dt))
     cores = torch.get_num_threads()
     t_start = time.perf_counter()
-    while reps < 3 or (time.perf_counter() - t_start < min(budget_s, 10.0) and reps < 50):
+    while reps < 3 or (time.perf_counter() - t_start < budget_s and reps < 50):
         t0 = time.perf_counter()
         w32, _ = O.dequantize(codes, scale, dt, bits, g)
         t1 = time.perf_counter()
-        y = x32 @ torch.from_numpy(w32)
+        _ = x32 @ torch.from_numpy(w32)
         t2 = time.perf_counter()
         t_dq += t1 - t0
         t_mm += t2 - t1
@@ -121,10 +266,36 @@ def cpu_baseline(np, torch, H, w_bits, x_bits, cfg, budget_s=25.0):
         "cores": int(cores),
         "kind": "port",
         "sample": "first %d of %d output columns of the decode weight (K=%d, int%d, group %d), M=1; "
-                  "per call: dequantize %.2f ms (1 thread) + fp32 matmul %.2f ms (%d threads); "
-                  "one-time quantize %.1f ms (1 thread); %d repetitions"
-                  % (n_s, N, K, bits, g, t_dq * 1e3, t_mm * 1e3, cores, t_q * 1e3, reps),
+                  "per call: dequantize %.2f ms (1 thread) + fp32 matmul %.2f ms (%d threads); %d repetitions"
+                  % (n_s, N, K, bits, g, t_dq * 1e3, t_mm * 1e3, cores, reps),
+        "quantize": {"ms": round(t_q * 1e3, 2), "cores": 1, "GB/s": round(K * n_s * 2 / t_q / 1e9, 4),
+                     "what": "oracle weight_quantize of the same %d x %d sample, GB/s on the bf16 weight read"
+                             % (K, n_s)},
     }, (codes, scale, n_s)
+
+
+def cpu_prefill_baseline(np, torch, H, pw_bits, px_bits, cfg, n_s=1024):
+    """The same three stages on the prefill shape, first n_s output columns."""
+    O = H.O
+    dt = H.BF16
+    K, M, bits, g = cfg["K"], cfg["M"], cfg["bits"], cfg["group_size"]
+    wb = np.ascontiguousarray(pw_bits[:, :n_s])
+    t0 = time.perf_counter()
+    codes, scale = O.weight_quantize(wb, dt, bits, g)
+    t_q = time.perf_counter() - t0
+    x32 = torch.from_numpy(H.bits_to_f32(px_bits, dt))
+    ts = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        w32, _ = O.dequantize(codes, scale, dt, bits, g)
+        y = x32 @ torch.from_numpy(w32)
+        ts.append(time.perf_counter() - t0)
+    t = statistics.median(ts)
+    return {"value": round(2.0 * M * K * n_s / t / 1e12, 4), "unit": "TFLOP/s", "cores": int(torch.get_num_threads()),
+            "kind": "port",
+            "sample": "first %d of %d output columns, M=%d K=%d int8 per-channel: dequantize (1 thread) + fp32 matmul "
+                      "(all threads) %.1f ms per call; one-time quantize %.1f ms (1 thread)"
+                      % (n_s, cfg["N"], M, K, t * 1e3, t_q * 1e3)}, (codes, scale, y.numpy())
 
 
 def main():
@@ -133,8 +304,10 @@ def main():
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--prefill-steps", type=int, default=20)
-    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU timing (parity still runs)")
     ap.add_argument("--no-llm-int8", action="store_true", help="skip the llm_int8_linear timing")
+    ap.add_argument("--no-configs", action="store_true", help="skip the per-configuration table")
+    ap.add_argument("--quick", action="store_true", help="shorter per-configuration runs, 8 decoder layers")
     ap.add_argument("--eager", action="store_true", help="time eager launches instead of a graph")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 256 MiB device copies (a known-size kernel to scale "
@@ -149,6 +322,7 @@ def main():
     import torch
 
     import helpers as H
+    from paddle_amd import _lib
     from paddle_amd.nn import quant as Q
 
     if not torch.cuda.is_available():
@@ -156,6 +330,7 @@ def main():
         sys.exit(3)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    stream = lambda: torch.cuda.current_stream().cuda_stream  # noqa: E731
 
     if args.copy_calibration:
         src = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=dev).fill_(1)
@@ -165,6 +340,8 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    failures = []
+
     # ---------------- decode (the headline metric) ----------------
     c = DECODE
     dt = H.BF16
@@ -172,7 +349,7 @@ def main():
     x_bits = H.make_act(c["M"], c["K"], dt, seed=1235)
     w = H.bits_to_torch(w_bits, dt, dev)
     x = H.bits_to_torch(x_bits, dt, dev)
-    codes, scale = _quantize(torch, Q, w, c["bits"], c["group_size"])
+    codes, scale = _quantize(Q, w, c["bits"], c["group_size"])
     wbytes = c["K"] * c["N"] * c["bits"] // 8
     sbytes = scale.numel() * 2
     total_bytes = wbytes + sbytes + 2 * (c["M"] * c["K"] + c["M"] * c["N"])
@@ -185,44 +362,59 @@ def main():
         j = i % ncopies
         return Q.weight_only_linear(x, copies[j], None, scales[j], wd, None, c["group_size"])
 
-    timer = _time_eager if args.eager else _time_graph
-    t_dec = timer(torch, decode_step, args.steps, args.warmup)
-    dec_s = t_dec / args.steps
+    dec_med, dec_min = time_graph(torch, decode_step, args.steps, warm_launches=max(400, args.warmup),
+                                  eager=args.eager)
+    dec_s = dec_med / args.steps
     dec_gbs = wbytes / dec_s / 1e9
-
-    # parity gate on the measured configuration
     y = decode_step(0)
     torch.cuda.synchronize()
 
     # the floor of this launch shape on this machine: the same weight copies read
     # by a kernel of the decode kernel's shape that computes nothing
-    from paddle_amd import _lib
     floor_out = torch.empty(c["N"] // 16 * 8, dtype=torch.int32, device=dev)
 
     def floor_step(i):
         _lib.check(_lib.lib.wol_read_floor(copies[i % ncopies].data_ptr(), c["K"], c["N"], c["bits"],
-                                           floor_out.data_ptr(), torch.cuda.current_stream().cuda_stream))
+                                           floor_out.data_ptr(), stream()))
 
-    floor_s = timer(torch, floor_step, args.steps, args.warmup) / args.steps
+    floor_med, _ = time_graph(torch, floor_step, args.steps, warm_launches=max(400, args.warmup), eager=args.eager)
+    floor_s = floor_med / args.steps
 
     # ---------------- prefill ----------------
     p = PREFILL
     pw_bits = H.make_weight(p["K"], p["N"], dt, seed=1236)
-    px = H.bits_to_torch(H.make_act(p["M"], p["K"], dt, seed=1237), dt, dev)
-    pcodes, pscale = _quantize(torch, Q, H.bits_to_torch(pw_bits, dt, dev), p["bits"], p["group_size"])
+    px_bits = H.make_act(p["M"], p["K"], dt, seed=1237)
+    px = H.bits_to_torch(px_bits, dt, dev)
+    pcodes, pscale = _quantize(Q, H.bits_to_torch(pw_bits, dt, dev), p["bits"], p["group_size"])
+    pcopies = [(pcodes.clone(), pscale.clone()) for _ in range(6)]  # 300 MB: past the Infinity Cache
 
     def prefill_step(i):
-        return Q.weight_only_linear(px, pcodes, None, pscale, "int8", None, p["group_size"])
+        cw, cs = pcopies[i % len(pcopies)]
+        return Q.weight_only_linear(px, cw, None, cs, "int8", None, p["group_size"])
 
-    t_pre = timer(torch, prefill_step, args.prefill_steps, args.warmup)
-    pre_s = t_pre / args.prefill_steps
+    pre_med, pre_min = time_graph(torch, prefill_step, args.prefill_steps, warm_launches=40, eager=args.eager)
+    pre_s = pre_med / args.prefill_steps
     flops = 2.0 * p["M"] * p["K"] * p["N"]
     pre_tf = flops / pre_s / 1e12
+    py = prefill_step(0)
+    torch.cuda.synchronize()
+
+    # the ceiling of the matrix pipes on this machine: nothing but MFMAs on random operands
+    ops = torch.randn(8 * 64 * 8, device=dev).to(torch.bfloat16)
+    ceil_wgs, ceil_iters = 1024, 2000
+    ceil_out = torch.empty(ceil_wgs * 512, dtype=torch.float32, device=dev)
+
+    def ceil_step(_i):
+        _lib.check(_lib.lib.wol_mfma_ceiling(ops.data_ptr(), ceil_wgs, ceil_iters, ceil_out.data_ptr(), stream()))
+
+    ceil_med, _ = time_graph(torch, ceil_step, 4, warm_launches=8, warm_ms=30.0, replays=5, eager=args.eager)
+    ceil_tf = ceil_wgs * 8.0 * ceil_iters * 8 * 2 * 32 * 32 * 16 / (ceil_med / 4) / 1e12
 
     # ---------------- llm_int8_linear on the prefill shape ----------------
     # the sibling op on the same weight (algo="llm.int8"): activations N(0,1)
     # with eight columns scaled x12, so that the outlier branch runs
     llm = None
+    lx = ly = None
     if not args.no_llm_int8:
         lw, lscale = Q.weight_quantize(H.bits_to_torch(pw_bits, dt, dev), algo="llm.int8")
         lx = px.clone()
@@ -231,14 +423,18 @@ def main():
         def llm_step(i):
             return Q.llm_int8_linear(lx, lw, None, lscale, 6.0)
 
-        llm_s = timer(torch, llm_step, args.prefill_steps, args.warmup) / args.prefill_steps
+        llm_med, llm_min = time_graph(torch, llm_step, args.prefill_steps, warm_launches=40, eager=args.eager)
+        llm_s = llm_med / args.prefill_steps
         llm_tops = flops / llm_s / 1e12
+        ly = llm_step(0)
+        torch.cuda.synchronize()
         llm = {
             "workload": "llm_int8_linear M=2048, K=4096 N=12288, bf16 x with 8 outlier columns, threshold 6.0; "
                         "all stages of one call (row ranges, activation codes, int8 GEMM with the merge)",
             "value": round(llm_tops, 2),
             "unit": "TOP/s",
             "ms_per_step": round(llm_s * 1e3, 4),
+            "ms_per_step_min": round(llm_min / args.prefill_steps * 1e3, 4),
             "steps": args.prefill_steps,
             "roofline": {"bound": "mfma", "achieved": round(llm_tops, 2), "peak": MFMA_INT8_PEAK_TOPS,
                          "unit": "TOP/s", "frac": round(llm_tops / MFMA_INT8_PEAK_TOPS, 4),
@@ -248,17 +444,55 @@ def main():
                                    "v_mfma_i32_32x32x32_i8"},
         }
 
-    # ---------------- CPU baseline + parity of the decode output ----------------
-    cpu = None
+    # ---------------- every BASELINE configuration ----------------
+    configs = stack = None
+    if not args.no_configs:
+        del copies, scales
+        torch.cuda.empty_cache()
+        configs = bench_configs(torch, Q, _lib, dev, args.quick)
+        stack = bench_decoder_stack(torch, Q, _lib, dev, args.quick)
+
+    # ---------------- parity of what was measured, against the oracle ----------------
+    O = H.O
     parity = {}
+    cpu = None
+    if args.no_cpu_baseline:
+        n_s = 512
+        ocodes, oscale = O.weight_quantize(np.ascontiguousarray(w_bits[:, :n_s]), dt, c["bits"], c["group_size"])
+    else:
+        cpu, (ocodes, oscale, n_s) = cpu_decode_baseline(np, torch, H, w_bits, x_bits, c)
+    _, oT = O.linear(x_bits, ocodes, oscale, None, dt, c["bits"], c["group_size"])
+    got = H.bits_to_f32(H.torch_to_bits(y), dt)[:, :n_s]
+    parity["decode_rel_l2_vs_oracle"] = H.rel_l2(got, H.bits_to_f32(oT, dt))
+    parity["scales_bit_exact"] = bool(np.array_equal(H.torch_to_bits(scale)[:, :n_s], oscale))
+    if parity["decode_rel_l2_vs_oracle"] > REL_L2_BAR:
+        failures.append("decode output differs from the oracle")
+    if not parity["scales_bit_exact"]:
+        failures.append("decode scales differ from the oracle")
+
+    # prefill: the first rows and columns of the measured output
+    rows, cols = 64, 256
+    pq, ps = O.weight_quantize(np.ascontiguousarray(pw_bits[:, :cols]), dt, p["bits"], p["group_size"])
+    _, pT = O.linear(px_bits[:rows], pq, ps, None, dt, p["bits"], p["group_size"])
+    got = H.bits_to_f32(H.torch_to_bits(py[:rows, :cols]), dt)
+    parity["prefill_rel_l2_vs_oracle"] = H.rel_l2(got, H.bits_to_f32(pT, dt))
+    parity["prefill_sample"] = "first %d rows x %d columns" % (rows, cols)
+    if parity["prefill_rel_l2_vs_oracle"] > REL_L2_BAR:
+        failures.append("prefill output differs from the oracle")
     if not args.no_cpu_baseline:
-        cpu, (ocodes, oscale, n_s) = cpu_baseline(np, torch, H, w_bits, x_bits, c)
-        O = H.O
-        o32, oT = O.linear(x_bits, ocodes, oscale, None, dt, c["bits"], c["group_size"])
-        got = H.bits_to_f32(H.torch_to_bits(y), dt)[:, :n_s]
-        parity["decode_rel_l2_vs_oracle"] = H.rel_l2(got, H.bits_to_f32(oT, dt))
-        gs = H.torch_to_bits(scale)[:, :n_s]
-        parity["scales_bit_exact"] = bool(np.array_equal(gs, oscale))
+        pcpu, _ = cpu_prefill_baseline(np, torch, H, pw_bits, px_bits, p)
+        cpu["prefill"] = pcpu
+
+    # llm_int8_linear: all rows (the outlier columns depend on every row), the first columns
+    if ly is not None:
+        cols = 64
+        lq, ls = O.weight_quantize_llm_int8(np.ascontiguousarray(pw_bits[:, :cols]), dt)
+        ref = O.llm_int8_linear(H.torch_to_bits(lx), np.ascontiguousarray(lq.T), None, ls, 6.0, dt)
+        same = np.array_equal(ref["out"], H.torch_to_bits(ly[:, :cols]))
+        parity["llm_int8_bit_exact_vs_oracle"] = bool(same)
+        parity["llm_int8_sample"] = "all rows x first %d columns" % cols
+        if not same:
+            failures.append("llm_int8_linear output differs from the oracle")
 
     traffic = _load_traffic()
     out = {
@@ -269,15 +503,19 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(dec_s * 1e3, 6),
+        "ms_per_step_min": round(dec_min / args.steps * 1e3, 6),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
+        "timing": "one HIP graph of --steps launches, replayed untimed until >= 400 launches and >= 50 ms have run, "
+                  "then %d timed replays (events on the launching stream); ms_per_step = median replay / steps"
+                  % REPLAYS if not args.eager else "eager launches",
         "config": {
             "workload": "decode GEMV M=1, int4 group_size=128, K=4096 N=11008, bf16 x, no bias; "
-                        "%d rotating weight copies; %s" % (ncopies, "eager launches" if args.eager else "one HIP graph of all steps"),
-            "prefill_workload": "GEMM M=2048, int8 per-channel, K=4096 N=12288, bf16 x",
+                        "%d rotating weight copies" % ncopies,
+            "prefill_workload": "GEMM M=2048, int8 per-channel, K=4096 N=12288, bf16 x, 6 rotating weight copies",
         },
         "roofline": {
             "bound": "hbm",
@@ -286,7 +524,8 @@ def main():
             "unit": "GB/s",
             "frac": round(dec_gbs / HBM_PEAK_GBS, 4),
             "traffic": traffic.get("decode_bytes_per_launch"),
-            "kernel": "wol::stream_kernel<1, 4, 1, 1, 8, 1, 1, true>",
+            "traffic_source": "profiles/traffic.json (rocprofv3 --pmc runs of this command, not measured in this run)",
+            "kernel": _plan(_lib, c["M"], c["K"], c["N"], c["bits"], c["group_size"]) or "wol::stream_kernel",
             "algorithmic_bytes_per_launch": wbytes,
             "total_bytes_per_launch": total_bytes,
             "read_floor": {
@@ -301,6 +540,7 @@ def main():
             "value": round(pre_tf, 2),
             "unit": "TFLOP/s",
             "ms_per_step": round(pre_s * 1e3, 4),
+            "ms_per_step_min": round(pre_min / args.prefill_steps * 1e3, 4),
             "steps": args.prefill_steps,
             "roofline": {
                 "bound": "mfma",
@@ -309,14 +549,26 @@ def main():
                 "unit": "TFLOP/s",
                 "frac": round(pre_tf / MFMA_BF16_PEAK_TF, 4),
                 "traffic": traffic.get("prefill_bytes_per_launch"),
-                "kernel": "wol::gemm_dma_kernel<1, 8, 0, false, 2, 4, 4, 2, 3> (256x256 tiles on the columns that fill whole rounds of the 256 CUs) + <1, 8, 0, false, 2, 4, 4, 1, 3> (256x128 tiles on the rest)",
+                "kernel": _plan(_lib, p["M"], p["K"], p["N"], p["bits"], p["group_size"]) or "wol::gemm_dma_kernel",
+                "mfma_ceiling": {
+                    "what": "wol_mfma_ceiling: v_mfma_f32_32x32x16_bf16 on random operands held in registers, "
+                            "8 independent accumulator blocks per wavefront, 8 wavefronts per CU, no memory traffic",
+                    "TFLOP/s": round(ceil_tf, 1),
+                    "frac_of_peak": round(ceil_tf / MFMA_BF16_PEAK_TF, 4),
+                    "prefill_over_ceiling": round(pre_tf / ceil_tf, 4),
+                },
             },
         },
+        "configs": configs,
+        "decoder_stack": stack,
         "llm_int8": llm,
         "cpu_baseline": cpu,
         "parity": parity,
     }
     print(json.dumps(out))
+    if failures:
+        print("bench.py: PARITY FAILURE: " + "; ".join(failures), file=sys.stderr)
+        sys.exit(4)
 
 
 if __name__ == "__main__":

@@ -78,7 +78,8 @@ typedef enum wol_status {
   WOL_ERR_WORKSPACE = 8,      /* workspace NULL or smaller than the query says  */
   WOL_ERR_ALIGNMENT = 9,      /* a pointer is not 16-byte aligned               */
   WOL_ERR_HIP = 10,           /* a HIP launch failed; see hipGetLastError       */
-  WOL_ERR_NO_DEVICE = 11      /* no gfx950 device / code object not loadable    */
+  WOL_ERR_NO_DEVICE = 11      /* valid arguments, but the current device is not
+                                 a gfx950 (checked once per device)             */
 } wol_status;
 
 /* Human-readable text for a status (static storage). */
@@ -144,7 +145,7 @@ size_t wol_linear_workspace(int64_t M, int64_t K, int64_t N, int bits,
  * fp32 accumulation, one round-to-nearest-even cast to T at the end.
  * codes must be in GFX950 layout.  bias may be NULL.
  * scale: [N] T (group_size -1) or [ceil(K/g),N] T, as wol_quantize wrote it.
- * M <= 8 takes the streaming (HBM-bound) kernel, M > 64 the MFMA GEMM, and in
+ * M <= 16 takes a streaming (HBM-bound) kernel, M > 64 the MFMA GEMM, and in
  * between whichever a cost model of the two predicts to be faster; the
  * reference's split is M <= 3 (gpu/weight_only_linear_kernel.cu:60-61).
  * x, codes and scale must be 16-byte aligned.
@@ -239,8 +240,9 @@ int wol_apply_per_channel_scale(const void* x, const void* scales, int dtype,
  * than the one its quantiser writes; this library indexes weight[n,k] plainly,
  * as the operator's description and the reference's own test
  * (test/quantization/test_llm_int8_linear.py:84-111) have it.
- * Requires K % 64 == 0, K <= 262144 and N % 16 == 0 (what weight_quantize
- * accepts, and an outlier mask that fits the LDS); x,
+ * Requires K % 64 == 0, K <= 131072 and N % 16 == 0 (what weight_quantize
+ * accepts; beyond K = 133152 the int32 sums of 127 * 127 products could wrap,
+ * which the reference's int32 GEMM does silently); x,
  * weight, weight_scale, out and workspace 16-byte aligned; out must not
  * overlap an input (with many outlier columns their product waits in out
  * until it is merged).  The workspace is
@@ -265,18 +267,6 @@ int wol_llm_int8_linear(const void* x, const void* weight, const void* bias,
  * counterpart there. */
 int wol_llm_int8_linear_stage_offsets(int64_t M, int64_t K, int64_t N,
                                       int64_t* offsets);
-
-/*
- * Measurement aid with no counterpart in the reference: reads a GFX950-layout
- * weight with the launch shape of the one-row decode kernel (one workgroup of
- * eight wavefronts per 16-column strip, 16-byte non-temporal loads, all of a
- * wavefront's loads requested at once) and computes nothing.  Its duration is
- * the floor a decode call of that shape has on the machine at hand; bench.py
- * reports it beside the decode time.  out receives N/16*8 uint32 (an XOR of
- * what each wavefront read).  K*bits/8*16 must be a multiple of 8 KiB.
- */
-int wol_read_floor(const void* codes, int64_t K, int64_t N, int bits, void* out,
-                   void* stream);
 
 #ifdef __cplusplus
 }

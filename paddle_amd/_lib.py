@@ -13,7 +13,7 @@ DTYPE_F16, DTYPE_BF16 = 0, 1
 ROUND_RNE, ROUND_TRUNC = 0, 1
 LAYOUT_CANONICAL, LAYOUT_PADDLE_HIP, LAYOUT_GFX950 = 0, 1, 2
 
-# every symbol include/wol_c_api.h declares
+# every symbol include/wol_c_api.h and include/wol_diag.h declare
 SYMBOLS = (
     "wol_status_str",
     "wol_layout_version",
@@ -30,6 +30,7 @@ SYMBOLS = (
     "wol_code_offset",
     "wol_apply_per_channel_scale",
     "wol_read_floor",
+    "wol_mfma_ceiling",
     "wol_llm_int8_linear_workspace",
     "wol_llm_int8_linear",
     "wol_llm_int8_linear_stage_offsets",
@@ -78,6 +79,8 @@ def _load():
     lib.wol_apply_per_channel_scale.restype = ci
     lib.wol_read_floor.argtypes = [vp, i64, i64, ci, vp, vp]
     lib.wol_read_floor.restype = ci
+    lib.wol_mfma_ceiling.argtypes = [vp, ci, ci, vp, vp]
+    lib.wol_mfma_ceiling.restype = ci
     lib.wol_llm_int8_linear_workspace.argtypes = [i64, i64, i64]
     lib.wol_llm_int8_linear_workspace.restype = sz
     lib.wol_llm_int8_linear.argtypes = [vp, vp, vp, vp, ctypes.c_float, ci, i64, i64, i64, vp, vp, sz, vp]

@@ -1,9 +1,36 @@
 // extern "C" entry points of libwol_gfx950.so: argument validation (the
 // shape/dtype contract of the reference's InferMeta functions), kernel
 // selection, nothing else.  See include/wol_c_api.h for the contract.
+#include <atomic>
+#include <cstring>
+
 #include "wol_common.h"
 
 namespace {
+
+// WOL_OK when the current device is a gfx950, WOL_ERR_NO_DEVICE otherwise (no
+// device at all, or one this library holds no code object for).  The answer
+// is looked up once per device.
+int require_gfx950() {
+  static std::atomic<int> known[64];  // 0 = not looked up, 1 = gfx950, 2 = something else
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return WOL_ERR_NO_DEVICE;
+  }
+  if (dev < 0 || dev >= 64) return WOL_ERR_NO_DEVICE;
+  int k = known[dev].load(std::memory_order_acquire);
+  if (k == 0) {
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) {
+      (void)hipGetLastError();
+      return WOL_ERR_NO_DEVICE;
+    }
+    k = std::strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : 2;
+    known[dev].store(k, std::memory_order_release);
+  }
+  return k == 1 ? WOL_OK : WOL_ERR_NO_DEVICE;
+}
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -86,6 +113,7 @@ int linear_impl(const void* x, const void* codes, const void* bias, const void* 
   if (x == nullptr || codes == nullptr || scale == nullptr || out == nullptr)
     return WOL_ERR_NULL_POINTER;
   if (!aligned16(x) || !aligned16(codes) || !aligned16(scale)) return WOL_ERR_ALIGNMENT;
+  if (const int dv = require_gfx950(); dv != WOL_OK) return dv;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (workspace == nullptr || !aligned16(workspace)) workspace_bytes = 0;  // optional: only speeds up
   const bool have_ws = workspace_bytes / sizeof(float) / 2 >= static_cast<size_t>(M) * static_cast<size_t>(N);
@@ -114,7 +142,7 @@ const char* wol_status_str(int status) {
     case WOL_ERR_WORKSPACE: return "workspace missing or too small";
     case WOL_ERR_ALIGNMENT: return "pointer not 16-byte aligned";
     case WOL_ERR_HIP: return "HIP launch failed";
-    case WOL_ERR_NO_DEVICE: return "no gfx950 device";
+    case WOL_ERR_NO_DEVICE: return "the current device is not a gfx950 (or there is no device)";
     default: return "unknown status";
   }
 }
@@ -137,6 +165,7 @@ int wol_quantize(const void* w, int dtype, int64_t K, int64_t N, int bits, int g
   if (!aligned16(w) || !aligned16(codes_out)) return WOL_ERR_ALIGNMENT;
   const size_t need = wol_quantize_workspace(K, N, bits, group_size);
   if (need > 0 && (workspace == nullptr || workspace_bytes < need)) return WOL_ERR_WORKSPACE;
+  if (const int dv = require_gfx950(); dv != WOL_OK) return dv;
   return wol::launch_quantize(w, dtype, K, N, bits, group_size, round_mode, layout, codes_out,
                               scale_out, false, workspace, static_cast<hipStream_t>(stream));
 }
@@ -151,6 +180,7 @@ int wol_quantize_llm_int8(const void* w, int dtype, int64_t K, int64_t N, int gr
   if (!aligned16(w) || !aligned16(codes_out)) return WOL_ERR_ALIGNMENT;
   const size_t need = wol_quantize_workspace(K, N, 8, group_size);
   if (need > 0 && (workspace == nullptr || workspace_bytes < need)) return WOL_ERR_WORKSPACE;
+  if (const int dv = require_gfx950(); dv != WOL_OK) return dv;
   return wol::launch_quantize(w, dtype, K, N, 8, group_size, WOL_ROUND_RNE, layout, codes_out,
                               scale_out, true, workspace, static_cast<hipStream_t>(stream));
 }
@@ -162,6 +192,7 @@ int wol_dequantize(const void* codes, int layout, const void* scale, int dtype, 
   if (!layout_ok(layout)) return WOL_ERR_BAD_LAYOUT;
   if (codes == nullptr || scale == nullptr || out_KN == nullptr) return WOL_ERR_NULL_POINTER;
   if (!aligned16(scale) || !aligned16(out_KN)) return WOL_ERR_ALIGNMENT;
+  if (const int dv = require_gfx950(); dv != WOL_OK) return dv;
   return wol::launch_dequantize(codes, layout, scale, dtype, K, N, bits, group_size, out_KN,
                                 static_cast<hipStream_t>(stream));
 }
@@ -207,6 +238,7 @@ int wol_repack(const void* codes_in, int layout_in, void* codes_out, int layout_
   if (!layout_ok(layout_in) || !layout_ok(layout_out)) return WOL_ERR_BAD_LAYOUT;
   if (codes_in == nullptr || codes_out == nullptr) return WOL_ERR_NULL_POINTER;
   if (codes_in == codes_out) return WOL_ERR_BAD_LAYOUT;  // not in place
+  if (const int dv = require_gfx950(); dv != WOL_OK) return dv;
   return wol::launch_repack(codes_in, layout_in, codes_out, layout_out, K, N, bits,
                             static_cast<hipStream_t>(stream));
 }
@@ -228,11 +260,14 @@ int wol_apply_per_channel_scale(const void* x, const void* scales, int dtype, in
     return WOL_ERR_BAD_SHAPE;
   if (rows == 0) return WOL_OK;
   if (x == nullptr || scales == nullptr || out == nullptr) return WOL_ERR_NULL_POINTER;
+  if (const int dv = require_gfx950(); dv != WOL_OK) return dv;
   return wol::launch_prescale(x, scales, dtype, rows, cols, out, static_cast<hipStream_t>(stream));
 }
 
-// the outlier mask of a call (K / 32 words) is kept in LDS by two of its kernels
-constexpr int64_t kLlmInt8MaxK = 262144;
+// int32 accumulation: |sum| <= K * 127 * 127 must stay below 2^31, i.e.
+// K <= 133152 (the reference's cublasLt int32 GEMM has the same limit without
+// checking it); the outlier mask of a call (K / 32 words) also sits in LDS
+constexpr int64_t kLlmInt8MaxK = 131072;
 
 size_t wol_llm_int8_linear_workspace(int64_t M, int64_t K, int64_t N) {
   if (check_problem(WOL_DTYPE_F16, K, N, 8, -1) != WOL_OK || M <= 0 || M > (int64_t{1} << 24)) return 0;
@@ -262,17 +297,9 @@ int wol_llm_int8_linear(const void* x, const void* weight, const void* bias, con
     return WOL_ERR_ALIGNMENT;
   if (workspace == nullptr || workspace_bytes < wol::llm_int8_workspace(M, K, N)) return WOL_ERR_WORKSPACE;
   if (!aligned16(workspace)) return WOL_ERR_ALIGNMENT;
+  if (const int dv = require_gfx950(); dv != WOL_OK) return dv;
   return wol::launch_llm_int8_linear(x, weight, bias, weight_scale, threshold, dtype, M, K, N, out, workspace,
                                      static_cast<hipStream_t>(stream));
-}
-
-int wol_read_floor(const void* codes, int64_t K, int64_t N, int bits, void* out, void* stream) {
-  const int rc = check_problem(WOL_DTYPE_F16, K, N, bits, -1);
-  if (rc != WOL_OK) return rc;
-  if (K * bits % (8 * 1024 * 8 / 16) != 0) return WOL_ERR_BAD_SHAPE;  // whole 1 KiB pieces per wavefront
-  if (codes == nullptr || out == nullptr) return WOL_ERR_NULL_POINTER;
-  if (!aligned16(codes)) return WOL_ERR_ALIGNMENT;
-  return wol::launch_read_floor(codes, K, N, bits, out, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

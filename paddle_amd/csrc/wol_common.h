@@ -216,6 +216,8 @@ int launch_linear_gemm(const void* x, const void* codes, const void* bias, const
                        hipStream_t stream);
 int launch_read_floor(const void* codes, int64_t K, int64_t N, int bits, void* out,
                       hipStream_t stream);
+int launch_mfma_ceiling(const void* operands, int workgroups, int iters, float* out,
+                        hipStream_t stream);
 int launch_prescale(const void* x, const void* scales, int dtype, int64_t rows, int64_t cols,
                     void* out, hipStream_t stream);
 int launch_llm_int8_linear(const void* x, const void* weight, const void* bias, const float* wscale,

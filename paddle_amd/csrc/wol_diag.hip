@@ -1,4 +1,6 @@
-// Diagnostic kernel: reads a packed weight with the launch shape of the
+// Diagnostic kernels (include/wol_diag.h).
+//
+// read_floor_kernel reads a packed weight with the launch shape of the
 // one-row streaming kernel (one workgroup of 8 wavefronts per 16-column strip,
 // every wavefront loading its 1/8 of the strip's k range with 16-byte
 // non-temporal loads, all requested before the first use) and does nothing
@@ -6,6 +8,7 @@
 // machine: launch, first-byte latency and the HBM stream, without a single
 // MFMA, scale or activation.
 #include "wol_common.h"
+#include "wol_diag.h"
 
 namespace wol {
 namespace {
@@ -33,6 +36,43 @@ __global__ __launch_bounds__(512) void read_floor_kernel(const uint8_t* __restri
   if (lane == 0) out[blockIdx.x * 8 + wave] = acc;
 }
 
+// Nothing but matrix instructions: 4 x 2 blocks of 32 x 32 per wavefront (the
+// register tile of the prefill GEMM), operands loaded once.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+__global__ __launch_bounds__(512) void mfma_ceiling_kernel(const u32x4* __restrict__ operands, int iters,
+                                                           float* __restrict__ out) {
+  const int lane = threadIdx.x & 63;
+  bf16x8 a[4], b[2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) a[i] = __builtin_bit_cast(bf16x8, operands[i * 64 + lane]);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) b[i] = __builtin_bit_cast(bf16x8, operands[(4 + i) * 64 + lane]);
+  f32x16 acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+  }
+  float s = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s += acc[i][j][r];
+  out[static_cast<int64_t>(blockIdx.x) * 512 + threadIdx.x] = s;
+}
+
 }  // namespace
 
 int launch_read_floor(const void* codes, int64_t K, int64_t N, int bits, void* out,
@@ -45,4 +85,32 @@ int launch_read_floor(const void* codes, int64_t K, int64_t N, int bits, void* o
   return hipGetLastError() == hipSuccess ? WOL_OK : WOL_ERR_HIP;
 }
 
+int launch_mfma_ceiling(const void* operands, int workgroups, int iters, float* out,
+                        hipStream_t stream) {
+  mfma_ceiling_kernel<<<dim3(static_cast<unsigned>(workgroups)), dim3(512), 0, stream>>>(
+      static_cast<const u32x4*>(operands), iters, out);
+  return hipGetLastError() == hipSuccess ? WOL_OK : WOL_ERR_HIP;
+}
+
 }  // namespace wol
+
+extern "C" {
+
+int wol_read_floor(const void* codes, int64_t K, int64_t N, int bits, void* out, void* stream) {
+  if (bits != 8 && bits != 4) return WOL_ERR_BAD_BITS;
+  if (K <= 0 || N <= 0 || K % 64 != 0 || N % 16 != 0 || K > (int64_t{1} << 24) || N > (int64_t{1} << 24))
+    return WOL_ERR_BAD_SHAPE;
+  if (K * bits % (8 * 1024 * 8 / 16) != 0) return WOL_ERR_BAD_SHAPE;  // whole 1 KiB pieces per wavefront
+  if (codes == nullptr || out == nullptr) return WOL_ERR_NULL_POINTER;
+  if ((reinterpret_cast<uintptr_t>(codes) & 15u) != 0) return WOL_ERR_ALIGNMENT;
+  return wol::launch_read_floor(codes, K, N, bits, out, static_cast<hipStream_t>(stream));
+}
+
+int wol_mfma_ceiling(const void* operands, int workgroups, int iters, float* out, void* stream) {
+  if (workgroups <= 0 || workgroups > 65536 || iters <= 0 || iters > (1 << 24)) return WOL_ERR_BAD_SHAPE;
+  if (operands == nullptr || out == nullptr) return WOL_ERR_NULL_POINTER;
+  if ((reinterpret_cast<uintptr_t>(operands) & 15u) != 0) return WOL_ERR_ALIGNMENT;
+  return wol::launch_mfma_ceiling(operands, workgroups, iters, out, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -686,8 +686,9 @@ __global__ __launch_bounds__(WM* WN * 64) __attribute__((amdgpu_waves_per_eu(2))
   // own (32 rows of kSlabRow ints: with that stride the two halves of the
   // wavefront write to disjoint banks) and takes them back as rows: a lane
   // owns eight neighbouring columns of one row, so the output leaves as
-  // 16-byte stores (with K runs: as eight integer atomics into the sums).  The
-  // loop over the rows is a real loop, which keeps the epilogue's registers few.
+  // 16-byte stores (with K runs: as two 16-byte stores into this run's slab of
+  // int32 sums).  The loop over the rows is a real loop, which keeps the
+  // epilogue's registers few.
   constexpr int kSlabRow = 40;
   __syncthreads();  // every wavefront is done with the stages
   int* slab = reinterpret_cast<int*>(smem) + wave * (32 * kSlabRow);

@@ -24,6 +24,7 @@ def lib():
 
 def test_library_exports_every_declared_symbol(lib):
     hdr = open(os.path.join(ROOT, "include", "wol_c_api.h")).read()
+    hdr += open(os.path.join(ROOT, "include", "wol_diag.h")).read()
     declared = set(re.findall(r"\b(wol_[a-z0-9_]+)\s*\(", hdr))
     declared -= {"wol_status"}
     assert declared == set(lib.SYMBOLS), declared ^ set(lib.SYMBOLS)

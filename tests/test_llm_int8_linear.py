@@ -219,9 +219,9 @@ def test_c_abi_argument_errors():
     assert L.wol_llm_int8_linear(None, None, None, None, 6.0, 0, 0, 64, 16, None, None, 0, None) == 0  # empty batch
     assert L.wol_llm_int8_linear(None, None, None, None, 6.0, 0, 4, 64, 16, None, None, 0, None) == 1
     assert L.wol_llm_int8_linear(16, 16, None, 16, 6.0, 0, 4, 64, 16, 16, None, 0, None) == 8  # workspace missing
-    assert L.wol_llm_int8_linear_workspace(4, 262144, 16) > 0
-    assert L.wol_llm_int8_linear_workspace(4, 262144 + 64, 16) == 0  # the outlier mask must fit the LDS
-    assert L.wol_llm_int8_linear(16, 16, None, 16, 6.0, 0, 4, 262144 + 64, 16, 16, 16, 1 << 30, None) == 5
+    assert L.wol_llm_int8_linear_workspace(4, 131072, 16) > 0
+    assert L.wol_llm_int8_linear_workspace(4, 131072 + 64, 16) == 0  # int32 sums must not wrap
+    assert L.wol_llm_int8_linear(16, 16, None, 16, 6.0, 0, 4, 131072 + 64, 16, 16, 16, 1 << 30, None) == 5
     assert L.wol_llm_int8_linear(16, 16, None, 16, 6.0, 0, 1 << 24, 64, 1 << 20, 16, 16, 1 << 30, None) == 5  # M * N above 2^40
     assert L.wol_llm_int8_linear(24, 16, None, 16, 6.0, 0, 4, 64, 16, 16, 16, 1 << 30, None) == 9  # x not 16-byte aligned
 
