@@ -110,6 +110,23 @@ int wol_quantize(const void* w, int dtype, int64_t K, int64_t N, int bits,
                  void* stream);
 
 /*
+ * wol_quantize for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It
+ * has no counterpart in the reference.  Same arithmetic, arguments and
+ * results as wol_quantize, but without the workspace: the per-channel abs-max
+ * buffer is a static device array inside the library (256 KiB on every GPU
+ * the library runs on, held until the process ends), so per-channel
+ * quantisation (group_size -1) is limited to N <= 65536 and returns
+ * WOL_ERR_BAD_SHAPE beyond that; group-wise quantisation uses no scratch and
+ * has no extra limit.  The call allocates and frees nothing.  All calls on one
+ * GPU share that GPU's array: per-channel calls that overlap on one GPU (two
+ * streams, two threads) race and must be serialised by the caller.
+ */
+int wol_quantize_static(const void* w, int dtype, int64_t K, int64_t N, int bits,
+                        int group_size, int round_mode, int layout,
+                        void* codes_out, void* scale_out, void* stream);
+
+/*
  * weight_quantize with algo = "llm.int8" (cpu/weight_quantize_kernel.cc:163-166,
  * quant_compute<..., int8_t, 8, float>): int8 codes computed against the
  * unrounded fp32 scale amax/127, which is also what is returned.

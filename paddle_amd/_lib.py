@@ -19,6 +19,7 @@ SYMBOLS = (
     "wol_layout_version",
     "wol_quantize_workspace",
     "wol_quantize",
+    "wol_quantize_static",
     "wol_quantize_llm_int8",
     "wol_dequantize",
     "wol_linear_workspace",
@@ -57,6 +58,8 @@ def _load():
     lib.wol_quantize_workspace.restype = sz
     lib.wol_quantize.argtypes = [vp, ci, i64, i64, ci, ci, ci, ci, vp, vp, vp, sz, vp]
     lib.wol_quantize.restype = ci
+    lib.wol_quantize_static.argtypes = [vp, ci, i64, i64, ci, ci, ci, ci, vp, vp, vp]
+    lib.wol_quantize_static.restype = ci
     lib.wol_quantize_llm_int8.argtypes = [vp, ci, i64, i64, ci, ci, vp, vp, vp, sz, vp]
     lib.wol_quantize_llm_int8.restype = ci
     lib.wol_dequantize.argtypes = [vp, ci, vp, ci, i64, i64, ci, ci, vp, vp]

@@ -170,6 +170,20 @@ int wol_quantize(const void* w, int dtype, int64_t K, int64_t N, int bits, int g
                               scale_out, false, workspace, static_cast<hipStream_t>(stream));
 }
 
+int wol_quantize_static(const void* w, int dtype, int64_t K, int64_t N, int bits, int group_size,
+                        int round_mode, int layout, void* codes_out, void* scale_out, void* stream) {
+  const int rc = check_problem(dtype, K, N, bits, group_size);
+  if (rc != WOL_OK) return rc;
+  if (round_mode != WOL_ROUND_RNE && round_mode != WOL_ROUND_TRUNC) return WOL_ERR_BAD_ROUND_MODE;
+  if (!layout_ok(layout)) return WOL_ERR_BAD_LAYOUT;
+  if (group_size == -1 && N > wol::kQuantizeStaticMaxN) return WOL_ERR_BAD_SHAPE;
+  if (w == nullptr || codes_out == nullptr || scale_out == nullptr) return WOL_ERR_NULL_POINTER;
+  if (!aligned16(w) || !aligned16(codes_out)) return WOL_ERR_ALIGNMENT;
+  if (const int dv = require_gfx950(); dv != WOL_OK) return dv;
+  return wol::launch_quantize_static(w, dtype, K, N, bits, group_size, round_mode, layout, codes_out,
+                                     scale_out, static_cast<hipStream_t>(stream));
+}
+
 int wol_quantize_llm_int8(const void* w, int dtype, int64_t K, int64_t N, int group_size,
                           int layout, void* codes_out, float* scale_out, void* workspace,
                           size_t workspace_bytes, void* stream) {

@@ -203,6 +203,12 @@ inline int stream_strips_per_workgroup(int64_t M, int64_t N, int bits) {
 int launch_quantize(const void* w, int dtype, int64_t K, int64_t N, int bits, int group_size,
                     int round_mode, int layout, void* codes, void* scale, bool scale_f32,
                     void* workspace, hipStream_t stream);
+// wol_quantize without a caller's workspace: the per-channel abs-max buffer is
+// a file-scope device array of kQuantizeStaticMaxN words (256 KiB per GPU).
+constexpr int64_t kQuantizeStaticMaxN = 65536;
+int launch_quantize_static(const void* w, int dtype, int64_t K, int64_t N, int bits, int group_size,
+                           int round_mode, int layout, void* codes, void* scale,
+                           hipStream_t stream);
 int launch_dequantize(const void* codes, int layout, const void* scale, int dtype, int64_t K,
                       int64_t N, int bits, int group_size, void* out, hipStream_t stream);
 int launch_repack(const void* in, int layout_in, void* out, int layout_out, int64_t K, int64_t N,

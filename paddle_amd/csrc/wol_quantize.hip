@@ -14,6 +14,8 @@
 // all-zero column gives 0/0 = NaN which becomes code 127 (int8, through
 // std::min/std::max :94-95) or -7 (int4, through the x86 float->int
 // conversion :107).
+#include <atomic>
+
 #include "wol_common.h"
 
 namespace wol {
@@ -455,6 +457,43 @@ int launch_quantize(const void* w, int dtype, int64_t K, int64_t N, int bits, in
   }
 #undef WOL_Q
   return check_launch();
+}
+
+// ---------------------------------------------------------------------------
+// The entry point for callers that cannot allocate (code under HIP graph
+// capture, serving loops, harnesses that forbid hipMalloc): the per-channel
+// abs-max buffer lives in a file-scope device array instead of a caller's
+// workspace.  Every GPU holds its own copy of the array at its own address,
+// resolved once per device with that device current; host code only ever uses
+// the resolved pointer, never the array's name.
+// ---------------------------------------------------------------------------
+constexpr int kStaticDevices = 64;
+static __device__ __align__(256) uint32_t scratch[kQuantizeStaticMaxN];
+static std::atomic<uint32_t*> scratch_ptr[kStaticDevices];
+
+int launch_quantize_static(const void* w, int dtype, int64_t K, int64_t N, int bits, int group_size,
+                           int round_mode, int layout, void* codes, void* scale,
+                           hipStream_t stream) {
+  uint32_t* amax = nullptr;
+  if (group_size == -1) {  // group-wise scales need no scratch at all
+    if (N > kQuantizeStaticMaxN) return WOL_ERR_BAD_SHAPE;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kStaticDevices) return WOL_ERR_NO_DEVICE;
+    amax = scratch_ptr[dev].load(std::memory_order_acquire);
+    if (amax == nullptr) {
+      void* p = nullptr;
+      if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) {
+        (void)hipGetLastError();
+        return WOL_ERR_HIP;
+      }
+      amax = static_cast<uint32_t*>(p);
+      scratch_ptr[dev].store(amax, std::memory_order_release);  // every thread resolves the same address
+    }
+  }
+  // launch_quantize clears the first N words with a fill kernel before the
+  // abs-max pass, so what an earlier call left behind does not matter
+  return launch_quantize(w, dtype, K, N, bits, group_size, round_mode, layout, codes, scale, false,
+                         amax, stream);
 }
 
 int launch_dequantize(const void* codes, int layout, const void* scale, int dtype, int64_t K,
