@@ -183,8 +183,13 @@ int wol_linear_f32(const void* x, const void* codes, const void* bias,
 /* Kernel choice of wol_linear_on. */
 enum wol_kernel {
   WOL_KERNEL_AUTO = 0,   /* what wol_linear does                                */
-  WOL_KERNEL_STREAM = 1, /* the streaming kernel; M <= 64 only                  */
-  WOL_KERNEL_GEMM = 2    /* the MFMA GEMM                                       */
+  WOL_KERNEL_STREAM = 1, /* the streaming kernel (a workgroup per 16 columns);
+                            M <= 64 only                                        */
+  WOL_KERNEL_GEMM = 2,   /* the MFMA GEMM                                       */
+  WOL_KERNEL_BATCH = 3   /* the batched decode kernel (a workgroup per CU, the
+                            activations fetched once per workgroup); M <= 16
+                            and K = 2048 or 4096 (8192 for int4 with group_size
+                            -1 or 128) only                                     */
 };
 
 /*

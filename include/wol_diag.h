@@ -45,6 +45,15 @@ int wol_read_floor(const void* codes, int64_t K, int64_t N, int bits, void* out,
 int wol_mfma_ceiling(const void* operands, int workgroups, int iters, float* out,
                      void* stream);
 
+/*
+ * Writes into buf (NUL-terminated, at most buf_bytes) one line naming the
+ * kernel and launch shape wol_linear takes for a problem when it is handed
+ * workspace_bytes of scratch.  No device work.  For benchmarks and dispatch
+ * tests.
+ */
+int wol_linear_plan(int64_t M, int64_t K, int64_t N, int bits, int group_size,
+                    size_t workspace_bytes, char* buf, size_t buf_bytes);
+
 #ifdef __cplusplus
 }
 #endif

@@ -32,6 +32,7 @@ SYMBOLS = (
     "wol_apply_per_channel_scale",
     "wol_read_floor",
     "wol_mfma_ceiling",
+    "wol_linear_plan",
     "wol_llm_int8_linear_workspace",
     "wol_llm_int8_linear",
     "wol_llm_int8_linear_stage_offsets",
@@ -84,6 +85,8 @@ def _load():
     lib.wol_read_floor.restype = ci
     lib.wol_mfma_ceiling.argtypes = [vp, ci, ci, vp, vp]
     lib.wol_mfma_ceiling.restype = ci
+    lib.wol_linear_plan.argtypes = [i64, i64, i64, ci, ci, sz, ctypes.c_char_p, sz]
+    lib.wol_linear_plan.restype = ci
     lib.wol_llm_int8_linear_workspace.argtypes = [i64, i64, i64]
     lib.wol_llm_int8_linear_workspace.restype = sz
     lib.wol_llm_int8_linear.argtypes = [vp, vp, vp, vp, ctypes.c_float, ci, i64, i64, i64, vp, vp, sz, vp]
@@ -100,7 +103,7 @@ lib = _load()
 _ARG_ERRORS = {1, 2, 3, 4, 5, 6, 7, 8, 9}
 
 # wol_kernel
-KERNEL_AUTO, KERNEL_STREAM, KERNEL_GEMM = 0, 1, 2
+KERNEL_AUTO, KERNEL_STREAM, KERNEL_GEMM, KERNEL_BATCH = 0, 1, 2, 3
 
 
 def check(status):

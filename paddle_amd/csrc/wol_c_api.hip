@@ -5,6 +5,7 @@
 #include <cstring>
 
 #include "wol_common.h"
+#include "wol_diag.h"
 
 namespace {
 
@@ -93,11 +94,27 @@ bool use_stream(int64_t M, int64_t K, int64_t N, int bits, bool have_ws) {
   return t_stream <= t_gemm;
 }
 
-// kernel: a wol_kernel; AUTO resolves by M and the cost model
-bool resolve_stream(int kernel, int64_t M, int64_t K, int64_t N, int bits, bool have_ws = true) {
-  if (kernel == WOL_KERNEL_STREAM) return true;
-  if (kernel == WOL_KERNEL_GEMM) return false;
-  return use_stream(M, K, N, bits, have_ws);
+// The batched decode kernel (a workgroup per CU that owns N / 16 / CUs strips
+// and fetches the activations once for all of them) against the streaming
+// kernel (a workgroup per strip): measured on MI355X over K = 4096 and 8192,
+// N from 4096 to 28672, both bit widths, it wins from two strips per CU on
+// when the streaming kernel's activation reads weigh in -- 5 rows and more
+// (16-row and 8-row operands) and 2 rows (whose operands share the least) --
+// and for 3 and 4 rows from five strips per CU on; with one strip per CU the
+// streaming kernel has the shorter critical path at every row count.
+bool use_batch(int64_t M, int64_t K, int64_t N, int bits, int group_size) {
+  if (M < 2 || M > 16 || !wol::linear_batch_supports(M, K, bits, group_size)) return false;
+  const int64_t per_cu = N / wol::kStripCols / wol::linear_batch_cus();
+  return (M == 3 || M == 4) ? per_cu >= 5 : per_cu >= 2;
+}
+
+// kernel: a wol_kernel; AUTO resolves by M and the cost model.  Returns the
+// wol_kernel that runs.
+int resolve_kernel(int kernel, int64_t M, int64_t K, int64_t N, int bits, int group_size,
+                   bool have_ws = true) {
+  if (kernel != WOL_KERNEL_AUTO) return kernel;
+  if (use_batch(M, K, N, bits, group_size)) return WOL_KERNEL_BATCH;
+  return use_stream(M, K, N, bits, have_ws) ? WOL_KERNEL_STREAM : WOL_KERNEL_GEMM;
 }
 
 int linear_impl(const void* x, const void* codes, const void* bias, const void* scale, int dtype,
@@ -106,9 +123,11 @@ int linear_impl(const void* x, const void* codes, const void* bias, const void* 
   const int rc = check_problem(dtype, K, N, bits, group_size);
   if (rc != WOL_OK) return rc;
   if (M < 0 || M > (int64_t{1} << 24)) return WOL_ERR_BAD_SHAPE;
-  if (kernel != WOL_KERNEL_AUTO && kernel != WOL_KERNEL_STREAM && kernel != WOL_KERNEL_GEMM)
+  if (kernel != WOL_KERNEL_AUTO && kernel != WOL_KERNEL_STREAM && kernel != WOL_KERNEL_GEMM &&
+      kernel != WOL_KERNEL_BATCH)
     return WOL_ERR_BAD_SHAPE;
   if (kernel == WOL_KERNEL_STREAM && M > kStreamMaxM) return WOL_ERR_BAD_SHAPE;
+  if (kernel == WOL_KERNEL_BATCH && M > 0 && !wol::linear_batch_supports(M, K, bits, group_size)) return WOL_ERR_BAD_SHAPE;
   if (M == 0) return WOL_OK;  // empty batch: nothing to write
   if (x == nullptr || codes == nullptr || scale == nullptr || out == nullptr)
     return WOL_ERR_NULL_POINTER;
@@ -117,7 +136,11 @@ int linear_impl(const void* x, const void* codes, const void* bias, const void* 
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (workspace == nullptr || !aligned16(workspace)) workspace_bytes = 0;  // optional: only speeds up
   const bool have_ws = workspace_bytes / sizeof(float) / 2 >= static_cast<size_t>(M) * static_cast<size_t>(N);
-  if (resolve_stream(kernel, M, K, N, bits, have_ws))
+  const int which = resolve_kernel(kernel, M, K, N, bits, group_size, have_ws);
+  if (which == WOL_KERNEL_BATCH)
+    return wol::launch_linear_batch(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out,
+                                    out_f32, s);
+  if (which == WOL_KERNEL_STREAM)
     return wol::launch_linear_stream(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out,
                                      out_f32, s);
   return wol::launch_linear_gemm(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out,
@@ -219,7 +242,7 @@ size_t wol_linear_workspace_for(int64_t M, int64_t K, int64_t N, int bits, int g
                                 int kernel) {
   if (check_problem(WOL_DTYPE_F16, K, N, bits, group_size) != WOL_OK || M <= 0) return 0;
   if (kernel == WOL_KERNEL_STREAM && M > kStreamMaxM) return 0;
-  if (resolve_stream(kernel, M, K, N, bits)) return 0;  // partial sums stay on chip
+  if (resolve_kernel(kernel, M, K, N, bits, group_size) != WOL_KERNEL_GEMM) return 0;  // partial sums stay on chip
   return wol::linear_gemm_workspace(M, K, N, bits, group_size);
 }
 
@@ -314,6 +337,28 @@ int wol_llm_int8_linear(const void* x, const void* weight, const void* bias, con
   if (const int dv = require_gfx950(); dv != WOL_OK) return dv;
   return wol::launch_llm_int8_linear(x, weight, bias, weight_scale, threshold, dtype, M, K, N, out, workspace,
                                      static_cast<hipStream_t>(stream));
+}
+
+int wol_linear_plan(int64_t M, int64_t K, int64_t N, int bits, int group_size, size_t workspace_bytes,
+                    char* buf, size_t buf_bytes) {
+  if (buf == nullptr || buf_bytes == 0) return WOL_ERR_NULL_POINTER;
+  const int rc = check_problem(WOL_DTYPE_F16, K, N, bits, group_size);
+  if (rc != WOL_OK) return rc;
+  if (M <= 0 || M > (int64_t{1} << 24)) return WOL_ERR_BAD_SHAPE;
+  const bool have_ws = workspace_bytes / sizeof(float) / 2 >= static_cast<size_t>(M) * static_cast<size_t>(N);
+  const int which = resolve_kernel(WOL_KERNEL_AUTO, M, K, N, bits, group_size, have_ws);
+  if (which == WOL_KERNEL_BATCH) {
+    int grid = 1, tpw = 1;
+    wol::plan_linear_batch(K, N, bits, &grid, &tpw);
+    snprintf(buf, buf_bytes, "wol::batch_kernel: %d workgroups of 16 wavefronts, %lld or %lld strips each, "
+             "activations resident in registers (%d weight tiles of a strip per wavefront)",
+             grid, static_cast<long long>(N / 16 / grid), static_cast<long long>((N / 16 + grid - 1) / grid), tpw);
+  } else if (which == WOL_KERNEL_STREAM) {
+    wol::describe_linear_stream(M, K, N, bits, group_size, buf, buf_bytes);
+  } else {
+    wol::describe_linear_gemm(M, K, N, bits, group_size, workspace_bytes, buf, buf_bytes);
+  }
+  return WOL_OK;
 }
 
 }  // extern "C"

@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdio.h>
 
 #include "wol_c_api.h"
 
@@ -216,6 +217,18 @@ int launch_repack(const void* in, int layout_in, void* out, int layout_out, int6
 int launch_linear_stream(const void* x, const void* codes, const void* bias, const void* scale,
                          int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
                          void* out, bool out_f32, hipStream_t stream);
+// The batched decode kernel (2 to 16 rows; one row works too; K = 2048, 4096, and
+// 8192 for int4 without groups of 64).
+bool linear_batch_supports(int64_t M, int64_t K, int bits, int group_size);
+int linear_batch_cus();  // CUs of the current device (256 when it cannot be asked)
+void plan_linear_batch(int64_t K, int64_t N, int bits, int* grid, int* tpw);
+int launch_linear_batch(const void* x, const void* codes, const void* bias, const void* scale,
+                        int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
+                        void* out, bool out_f32, hipStream_t stream);
+// One-line descriptions of what the launchers would run for a problem.
+void describe_linear_stream(int64_t M, int64_t K, int64_t N, int bits, int group_size, char* buf, size_t n);
+void describe_linear_gemm(int64_t M, int64_t K, int64_t N, int bits, int group_size, size_t ws_bytes,
+                          char* buf, size_t n);
 int launch_linear_gemm(const void* x, const void* codes, const void* bias, const void* scale,
                        int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
                        void* out, bool out_f32, void* workspace, size_t workspace_bytes,

@@ -1,0 +1,410 @@
+// weight_only_linear for a small batch of rows (2 <= M <= 16): the decode
+// kernel for batched serving.
+//
+// What limits the one-row kernel's launch shape (a workgroup per 16-column
+// strip) at several rows is the activations: every workgroup needs all of x,
+// 16 rows x K, and with one workgroup per strip that is N/16 copies of x out
+// of L2 -- four times the weight bytes at 16 rows of int4.  Here the grid is
+// at most one workgroup per CU and a workgroup owns a contiguous run of strips
+// (N/16 / 256 of them), so x is fetched once per CU.
+//
+// A workgroup has 16 wavefronts that split K evenly between them (K = 2048,
+// 4096 or 8192: every wavefront owns the same whole number of 1 KiB weight
+// tiles of each strip), and the A fragments of a wavefront's run of k (16 rows
+// x 32 k each, 16 bytes per lane; 32 registers at K = 4096, 64 at 8192) are
+// loaded once and stay in registers for every strip of the workgroup -- the
+// registers are the staging buffer for x, nothing of it passes through LDS.
+// The wavefront's work is a list of items (a strip's tiles of the run, or half
+// of them) in strip order.  Weight tiles live in a register ring of D items:
+// the ring is filled before the first use, and a slot is refilled with the
+// item D places further on as soon as it has been consumed.  All loads are
+// unconditional instructions (past the last item they are buffer loads beyond
+// the end of their descriptor, which fetch nothing), which is what lets the
+// compiler wait for exactly the tile it needs while the younger loads stay in
+// flight.
+//
+// Arithmetic: as in the one-row kernel the codes become T bit patterns
+// (code + offset, exact) and v_mfma_f32_16x16x32 does the multiply and the
+// reduction over k.  The MFMAs of one chain (a tile, or a scale group inside
+// it: at most 128 k) accumulate in place, starting from the chain's cancelling
+// term mfma(A, constant B); those terms depend on the wavefront's A fragments
+// only and, where 16 registers hold them, are computed once for all strips.  Only a
+// chain's result is added to the running fp32 sums (times the group scale
+// when scales are group-wise).  Nothing is rounded to T before the final cast.
+//
+// The wavefronts never wait for each other while they stream: every
+// wavefront leaves its partial sums of every strip in LDS (16 KiB per strip),
+// and one barrier at the end of a run of up to seven strips precedes the
+// reduction (in wavefront order: deterministic), scale, bias, cast and store.
+// The per-channel scales and the bias of a run are parked in LDS at its start;
+// group-wise scales travel with their weight tiles, one 2-byte load per lane
+// and group.
+#include <atomic>
+
+#include "wol_common.h"
+#include "wol_dequant.h"
+
+namespace wol {
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <int DT>
+__device__ inline f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
+  if (DT == WOL_DTYPE_BF16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
+                                                __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+
+constexpr int kBatchWaves = 16;
+constexpr int kBatchRun = 7;  // strips whose partial sums (16 KiB each) share the LDS
+
+struct BatchParams {
+  const uint16_t* x;
+  const uint8_t* codes;
+  const uint16_t* bias;
+  const uint16_t* scale;
+  void* out;
+  int M, K, N;
+  int gshift;   // log2(group size), -1 per-channel
+  int out_f32;
+  int strips_q, strips_r;  // strips per workgroup: N / 16 = grid * strips_q + strips_r
+};
+
+// G: 0 per-channel, else the group size.  TPW: weight tiles (1 KiB, 64 or 128
+// k) of a strip that belong to one wavefront: K = 16 * TPW * tile depth
+// exactly, so that every wavefront runs the same instruction stream and every
+// load below is unconditional -- the compiler then knows at each use how many
+// younger loads may still be in flight (s_waitcnt vmcnt(n) with n > 0); a load
+// under a condition would make every later wait a wait for all loads.
+// IT: tiles per item, D: items in the ring (a multiple of TPW / IT).
+template <int DT, int BITS, int G, int TPW, int IT, int D>
+__global__ __launch_bounds__(kBatchWaves * 64) void batch_kernel(const BatchParams p) {
+  constexpr int WK = kBatchWaves;
+  constexpr int TK = BITS == 8 ? 64 : 128;   // k per 1 KiB weight tile
+  constexpr int SPT = TK / 32;               // k steps per tile
+  constexpr int kDw = BITS == 8 ? 2 : 1;     // dwords per k step and lane
+  constexpr int P = TPW / IT;                // items per strip
+  static_assert(TPW % IT == 0 && D % P == 0, "ring slot d always holds part d % P of a strip");
+  constexpr int CK = G == 0 ? TK : (G < TK ? G : TK);  // k per chain
+  constexpr int CPT = TK / CK;               // chains per tile
+  constexpr int SPC = SPT / CPT;             // k steps per chain
+  constexpr int NS = G == 0 ? 1 : IT * CPT;  // group scales per item and lane
+  constexpr bool kKeepCancel = TPW * SPT <= 8 && TPW * CPT <= 4;  // cancelling terms computed once and kept
+                                                               // where 32 registers of A leave 16 for them
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int j = lane & 15, kb = lane >> 4;
+  const int K = p.K, N = p.N, M = p.M;
+  // this workgroup's strips; this wavefront's tiles are t0 .. t0 + TPW - 1 of each
+  const int bid = static_cast<int>(blockIdx.x);
+  const int s0 = bid * p.strips_q + (bid < p.strips_r ? bid : p.strips_r);
+  const int s1 = s0 + p.strips_q + (bid < p.strips_r ? 1 : 0);
+  const int t0 = wave * TPW;
+  const int64_t sbytes = strip_bytes(K, BITS);
+
+  uint32_t magic = Dequant<DT, BITS>::kMagic;
+  asm volatile("" : "+v"(magic));  // keep the constant in a VGPR
+  const u32x4 cancel = {Dequant<DT, BITS>::kCancel, Dequant<DT, BITS>::kCancel,
+                        Dequant<DT, BITS>::kCancel, Dequant<DT, BITS>::kCancel};
+
+  // A fragment of k step `step`: lane (kb, j) holds row j, k = 32 * step + 8 * kb .. + 7.
+  // Only the lanes of rows that exist load anything (the texture unit spends
+  // its cycles per active lane: at 4 rows the fragments cost a quarter of what
+  // 16 rows cost); the other rows hold whatever the registers held (rows of an MFMA result do
+  // not mix) and are never stored.
+  const uint16_t* xrow = p.x + static_cast<int64_t>(j < M ? j : 0) * K + t0 * TK + 8 * kb;
+  u32x4 A[TPW * SPT];
+#pragma unroll
+  for (int s = 0; s < TPW * SPT; ++s) asm volatile("" : "=v"(A[s]));  // any value will do in the rows past M
+  if (j < M) {
+#pragma unroll
+    for (int s = 0; s < TPW * SPT; ++s) A[s] = *reinterpret_cast<const u32x4*>(xrow + s * 32);
+  }
+
+  u32x4 W[D][IT];
+  uint16_t S[D][NS];
+  // part `part` (IT tiles) of this wavefront's share of strip `strip`.  The
+  // tiles come through a buffer descriptor that spans the strips of the run
+  // (at most 7 x 128 KiB): with real == false the offset lies past its end,
+  // and such a load returns zeros without touching memory -- the instruction
+  // stays unconditional, the traffic does not.
+  const int lane_off = t0 * 1024 + lane * 16;
+  auto load_item = [&](__amdgpu_buffer_rsrc_t rsrc, int strip, int strip_of_run, int part, bool real,
+                       u32x4 (&w)[IT], uint16_t (&sc)[NS]) {
+    if (G != 0) {  // the item's group scales travel with it (past the last item: the last strip's again)
+#pragma unroll
+      for (int q = 0; q < NS; ++q) {
+        const int k0 = (t0 + part * IT) * TK + q * CK;
+        sc[q] = p.scale[static_cast<int64_t>(k0 >> p.gshift) * N + strip * kStripCols + j];
+      }
+    }
+    const int soff = real ? strip_of_run * static_cast<int>(sbytes) + part * IT * 1024 : 0x7FFF0000;
+#pragma unroll
+    for (int i = 0; i < IT; ++i)
+      w[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off + soff + i * 1024, 0, 0));
+  };
+
+  f32x4 ccs[kKeepCancel ? TPW * CPT : 1];  // the cancelling term of every chain of the wavefront's run
+  bool have_cc = false;
+  // the per-channel scales (first row of the scale tensor) and the bias behind
+  // bounded descriptors, for the staging loads
+  const __amdgpu_buffer_rsrc_t scale_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(p.scale), 0, N * 2, 0x00020000);
+  const __amdgpu_buffer_rsrc_t bias_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(p.bias != nullptr ? p.bias : p.scale), 0, N * 2, 0x00020000);
+
+  for (int sr = s0; sr < s1; sr += kBatchRun) {
+    const int cnt = s1 - sr < kBatchRun ? s1 - sr : kBatchRun;  // strips of this run
+    const int nitems = cnt * P;  // item it: strip sr + it / P, part it % P
+
+    const int ncols = cnt * kStripCols;
+    float* red = reinterpret_cast<float*>(smem);                          // [cnt][WK][4][64]
+    uint16_t* lsc = reinterpret_cast<uint16_t*>(smem + cnt * WK * 1024);  // [ncols] per-channel scales
+    uint16_t* lbi = lsc + ncols;                                          // [ncols] bias
+
+    // What the end of the run needs -- per-channel scales and bias of its
+    // columns -- is requested first (one load each by the first threads; the
+    // others read past the end of the descriptor: nothing) and parked in LDS
+    // once the weight ring has been requested as well.
+    const int boff = static_cast<int>(threadIdx.x) < ncols ? (sr * kStripCols + static_cast<int>(threadIdx.x)) * 2 : 0x7FFFFFF0;
+    const uint16_t sstage = __builtin_amdgcn_raw_buffer_load_b16(scale_rsrc, boff, 0, 0);
+    const uint16_t bstage = __builtin_amdgcn_raw_buffer_load_b16(bias_rsrc, boff, 0, 0);
+
+    // fill the ring; slots past the last item load nothing
+    const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(p.codes + sr * sbytes), 0, cnt * static_cast<int>(sbytes), 0x00020000);
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const int sl = d / P < cnt ? d / P : cnt - 1;
+      load_item(wrsrc, sr + sl, d / P, d % P, d < nitems, W[d], S[d]);
+    }
+
+    // the staged values have arrived before the ring (they were requested first)
+    if (static_cast<int>(threadIdx.x) < ncols) {
+      lsc[threadIdx.x] = sstage;
+      lbi[threadIdx.x] = bstage;
+    }
+
+    if (kKeepCancel && !have_cc) {
+#pragma unroll
+      for (int c = 0; c < TPW * CPT; ++c) {
+        f32x4 cc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < SPC; ++s) cc = mfma16<DT>(A[c * SPC + s], cancel, cc);
+        ccs[c] = cc;
+      }
+      have_cc = true;
+    }
+    f32x4 tot = {0.f, 0.f, 0.f, 0.f};
+    for (int base = 0; base < nitems; base += D) {
+#pragma unroll
+      for (int d = 0; d < D; ++d) {
+        const int part = d % P;  // static: D is a multiple of P and base a multiple of D
+        const int it = base + d;
+        const int sl = it / P;   // strip of the run
+        if (it < nitems) {
+#pragma unroll
+          for (int i = 0; i < IT; ++i) {
+            const uint32_t w4[4] = {W[d][i].x, W[d][i].y, W[d][i].z, W[d][i].w};
+#pragma unroll
+            for (int ch = 0; ch < CPT; ++ch) {
+              const int a0 = ((part * IT + i) * CPT + ch) * SPC;  // first A fragment of the chain
+              f32x4 acc;
+              if (kKeepCancel) {
+                acc = ccs[(part * IT + i) * CPT + ch];
+              } else {
+                acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int s = 0; s < SPC; ++s) acc = mfma16<DT>(A[a0 + s], cancel, acc);
+              }
+#pragma unroll
+              for (int s = 0; s < SPC; ++s) {
+                const u32x4 b = Dequant<DT, BITS>::run(&w4[(ch * SPC + s) * kDw], magic);
+                acc = mfma16<DT>(A[a0 + s], b, acc);
+              }
+              if (G != 0) {
+                const float sc = to_f32<DT>(S[d][i * CPT + ch]);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) tot[r] = fmaf(acc[r], sc, tot[r]);
+              } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) tot[r] += acc[r];
+              }
+            }
+          }
+          if (part == P - 1) {  // the strip is complete for this wavefront
+#pragma unroll
+            for (int r = 0; r < 4; ++r) red[((sl * WK + wave) * 4 + r) * 64 + lane] = tot[r];
+            tot = f32x4{0.f, 0.f, 0.f, 0.f};
+          }
+        }
+        // the slot is free: refill it with the item D places further on (if there is one)
+        const int nsl = (it + D) / P < cnt ? (it + D) / P : cnt - 1;
+        load_item(wrsrc, sr + nsl, (it + D) / P, part, it + D < nitems, W[d], S[d]);
+      }
+    }
+
+    // ---- the run is done: partial sums of the 16 wavefronts meet in LDS ----
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const int e = threadIdx.x + q * WK * 64;
+      if (e < cnt * 256) {
+        const int sl = e >> 8, r = (e >> 6) & 3, l = e & 63;
+        float s = 0.0f;
+#pragma unroll
+        for (int w = 0; w < WK; ++w) s += red[((sl * WK + w) * 4 + r) * 64 + l];
+        const int m = 4 * (l >> 4) + r;
+        if (m < M) {
+          const int cl = sl * kStripCols + (l & 15);
+          const float ep_scale = G == 0 ? to_f32<DT>(lsc[cl]) : 1.0f;
+          const float ep_bias = p.bias != nullptr ? to_f32<DT>(lbi[cl]) : 0.0f;
+          s = s * ep_scale + ep_bias;
+          const int64_t o = static_cast<int64_t>(m) * N + (sr + sl) * kStripCols + (l & 15);
+          if (p.out_f32)
+            static_cast<float*>(p.out)[o] = s;
+          else
+            static_cast<uint16_t*>(p.out)[o] = cast_out<DT>(s);
+        }
+      }
+    }
+    // Name the ring's registers: the loads past the last item (which fetch
+    // nothing) are then known to have completed here, and the next run starts
+    // with a load queue whose content the compiler knows exactly -- otherwise
+    // the first loads of a run would wait for older ones they do not depend on.
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+#pragma unroll
+      for (int i = 0; i < IT; ++i) asm volatile("" ::"v"(W[d][i]));
+#pragma unroll
+      for (int q = 0; q < NS; ++q) asm volatile("" ::"v"(S[d][q]));
+    }
+    if (sr + kBatchRun < s1) __syncthreads();  // the next run overwrites the partial sums
+  }
+}
+
+struct Args {
+  const void* x; const void* codes; const void* bias; const void* scale; void* out;
+  int M, K, N, gshift, out_f32; hipStream_t stream;
+};
+
+inline int num_cus() {
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    return n;
+  }();
+  return cus;
+}
+
+// Raises a kernel's dynamic LDS limit once per device.
+inline void allow_lds(const void* kern, size_t lds, std::atomic<uint32_t>& done) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+  const uint32_t bit = 1u << (dev & 31);
+  if (done.load(std::memory_order_acquire) & bit) return;
+  (void)hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+  done.fetch_or(bit, std::memory_order_release);
+}
+
+// LDS of a launch: partial sums, scales and bias of the longest run of strips
+inline size_t batch_lds(int64_t K, int64_t N, int group_size, int grid) {
+  const int64_t nstrips = N / kStripCols;
+  int64_t per_wg = (nstrips + grid - 1) / grid;
+  if (per_wg > kBatchRun) per_wg = kBatchRun;
+  (void)K;
+  (void)group_size;
+  return static_cast<size_t>(per_wg * kBatchWaves * 1024 + 2 * per_wg * kStripCols * 2);
+}
+
+template <int DT, int BITS, int G, int TPW, int IT, int D>
+void launch_one(const Args& a, int grid) {
+  const size_t lds = batch_lds(a.K, a.N, G, grid);
+  auto kern = batch_kernel<DT, BITS, G, TPW, IT, D>;
+  static std::atomic<uint32_t> configured{0};  // per instantiation
+  allow_lds(reinterpret_cast<const void*>(kern), 160 * 1024, configured);
+  BatchParams p;
+  p.x = static_cast<const uint16_t*>(a.x);
+  p.codes = static_cast<const uint8_t*>(a.codes);
+  p.bias = static_cast<const uint16_t*>(a.bias);
+  p.scale = static_cast<const uint16_t*>(a.scale);
+  p.out = a.out;
+  p.M = a.M; p.K = a.K; p.N = a.N;
+  p.gshift = a.gshift;
+  p.out_f32 = a.out_f32;
+  p.strips_q = a.N / kStripCols / grid;
+  p.strips_r = a.N / kStripCols % grid;
+  kern<<<dim3(static_cast<unsigned>(grid)), dim3(kBatchWaves * 64), lds, a.stream>>>(p);
+}
+
+// tpw = K / (16 * tile depth): 1, 2 or 4.  Items and ring depths by what the
+// 128 registers of a 16-wavefront workgroup hold next to the A fragments
+// (16 registers per tile of the run): an item of IT tiles is 4 * IT registers.
+template <int DT, int BITS, int G>
+void launch_cfg(const Args& a, int grid, int tpw) {
+  if constexpr (BITS == 4) {
+    if (tpw == 1) launch_one<DT, 4, G, 1, 1, 4>(a, grid);        // K = 2048
+    else if (tpw == 2) launch_one<DT, 4, G, 2, 2, 3>(a, grid);   // K = 4096
+    else if constexpr (G != 64) launch_one<DT, 4, G, 4, 2, 2>(a, grid);  // K = 8192
+  } else {
+    if (tpw == 2) launch_one<DT, 8, G, 2, 2, 3>(a, grid);        // K = 2048
+    else if (tpw == 4) launch_one<DT, 8, G, 4, 4, 2>(a, grid);   // K = 4096
+  }
+}
+
+template <int DT, int BITS>
+void launch_g(const Args& a, int grid, int tpw) {
+  if (a.gshift < 0) launch_cfg<DT, BITS, 0>(a, grid, tpw);
+  else if (a.gshift == 6) launch_cfg<DT, BITS, 64>(a, grid, tpw);
+  else launch_cfg<DT, BITS, 128>(a, grid, tpw);
+}
+
+}  // namespace
+
+// K must split into the same number of whole weight tiles for each of the 16
+// wavefronts, and that number must be one the kernel is built for: K = 2048
+// or 4096, and K = 8192 with int4 codes unless their groups are 64 long (64
+// registers of A fragments leave no room for more).
+bool linear_batch_supports(int64_t M, int64_t K, int bits, int group_size) {
+  if (M < 1 || M > 16) return false;
+  if (K == 2048 || K == 4096) return true;
+  return K == 8192 && bits == 4 && group_size != 64;
+}
+
+int linear_batch_cus() { return num_cus(); }
+
+// Grid (workgroups: one per CU, fewer when there are fewer strips) and the
+// weight tiles of a strip per wavefront.
+void plan_linear_batch(int64_t K, int64_t N, int bits, int* grid, int* tpw) {
+  const int64_t nstrips = N / kStripCols;
+  const int cus = num_cus();
+  *grid = static_cast<int>(nstrips < cus ? nstrips : cus);
+  *tpw = static_cast<int>(K / (bits == 8 ? 64 : 128) / kBatchWaves);
+}
+
+int launch_linear_batch(const void* x, const void* codes, const void* bias, const void* scale,
+                        int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
+                        void* out, bool out_f32, hipStream_t stream) {
+  const int gshift = group_size == 64 ? 6 : (group_size == 128 ? 7 : -1);
+  int grid = 1, tpw = 1;
+  plan_linear_batch(K, N, bits, &grid, &tpw);
+  const Args a{x, codes, bias, scale, out, static_cast<int>(M), static_cast<int>(K),
+               static_cast<int>(N), gshift, out_f32 ? 1 : 0, stream};
+  if (dtype == WOL_DTYPE_BF16) {
+    if (bits == 8) launch_g<WOL_DTYPE_BF16, 8>(a, grid, tpw); else launch_g<WOL_DTYPE_BF16, 4>(a, grid, tpw);
+  } else {
+    if (bits == 8) launch_g<WOL_DTYPE_F16, 8>(a, grid, tpw); else launch_g<WOL_DTYPE_F16, 4>(a, grid, tpw);
+  }
+  return check_launch();
+}
+
+}  // namespace wol

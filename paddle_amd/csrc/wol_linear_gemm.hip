@@ -1128,6 +1128,37 @@ size_t linear_gemm_workspace(int64_t M, int64_t K, int64_t N, int bits, int grou
   return ns > 1 ? static_cast<size_t>(ns) * M * N * sizeof(float) : 0;
 }
 
+void describe_linear_gemm(int64_t M, int64_t K, int64_t N, int bits, int group_size, size_t ws_bytes,
+                          char* buf, size_t n) {
+  const int tk = bits == 8 ? 64 : 128;
+  const int g = group_size > 0 ? group_size : 0;
+  if (K % tk != 0 || K / tk < 2) {
+    snprintf(buf, n, "wol::gemm_kernel (register-staged v_mfma_f32_16x16x32, 256 x %d tiles)", g ? 128 : 256);
+    return;
+  }
+  if (M <= kSkinnyMaxM) {
+    bool wide = false;
+    const int ns = plan_skinny(static_cast<int>(M), static_cast<int>(K), static_cast<int>(N), bits, g, ws_bytes, &wide);
+    snprintf(buf, n, "wol::gemm_dma_kernel: %d rows x %d columns per workgroup, K in %d run(s)%s",
+             bits == 4 && M <= 32 ? 32 : 64, wide ? 512 : 256, ns, ns > 1 ? " + reduce_partials_kernel" : "");
+    return;
+  }
+  int bm = 0, bn = 0, lo = 0;
+  half_tile_config(static_cast<int>(M), static_cast<int>(N), bits, g, &bm, &bn, &lo);
+  const int nstrips = static_cast<int>(N / kStripCols);
+  const TailPlan t = plan_tail(static_cast<int>(M), static_cast<int>(K), (nstrips - lo) * kStripCols, bm, bn, tk, ws_bytes);
+  const int mid = lo + t.full_tiles * (bn / kStripCols);
+  int len = 0;
+  len += snprintf(buf + len, n - len, "wol::gemm_dma_kernel (v_mfma_f32_32x32x16):");
+  if (lo > 0 && len < static_cast<int>(n))
+    len += snprintf(buf + len, n - len, " 256x256 tiles on columns [0,%d)", lo * kStripCols);
+  if (mid > lo && len < static_cast<int>(n))
+    len += snprintf(buf + len, n - len, " %dx%d tiles on [%d,%d)", bm, bn, lo * kStripCols, mid * kStripCols);
+  if (nstrips > mid && len < static_cast<int>(n))
+    len += snprintf(buf + len, n - len, " %dx%d tiles on [%d,%d)%s", bm, bn, mid * kStripCols, nstrips * kStripCols,
+                    t.ns > 1 ? " with K in runs + reduce_partials_kernel" : "");
+}
+
 int launch_linear_gemm(const void* x, const void* codes, const void* bias, const void* scale,
                        int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
                        void* out, bool out_f32, void* workspace, size_t workspace_bytes,

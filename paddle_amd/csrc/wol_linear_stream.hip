@@ -505,6 +505,17 @@ static void pick_split(int64_t M, int64_t K, int64_t N, int bits, int* wk, int* 
   *nu = 0;
 }
 
+void describe_linear_stream(int64_t M, int64_t K, int64_t N, int bits, int group_size, char* buf, size_t n) {
+  int wk = 1, nu = 0, tn = 1;
+  pick_split(M, K, N, bits, &wk, &nu, &tn);
+  int mp = 1;
+  while (mp < 16 && mp < M) mp *= 2;
+  snprintf(buf, n, "wol::stream_kernel: %lld workgroups of %d wavefronts, %d strip(s) each, %d-row operands x %d, %s",
+           static_cast<long long>((N / kStripCols + tn - 1) / tn), wk, tn, mp, static_cast<int>((M + 15) / 16),
+           nu > 0 ? "all loads of a wavefront issued at once" : "wavefronts walk their units double-buffered");
+  (void)group_size;
+}
+
 int launch_linear_stream(const void* x, const void* codes, const void* bias, const void* scale,
                          int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
                          void* out, bool out_f32, hipStream_t stream) {

@@ -22,9 +22,9 @@ def G(device):
     return gpu_calls
 
 
-def check(G, oracle, dt, bits, g, M, K, N, bias=True, seed=0, outliers=0.0, tol32=2e-5, **kw):
+def check(G, oracle, dt, bits, g, M, K, N, bias=True, seed=0, outliers=0.0, tol32=2e-5, xdist="normal", **kw):
     wb = H.make_weight(K, N, dt, seed=seed + K + N, outlier_cols=outliers)
-    xb = H.make_act(M, K, dt, seed=seed + M)
+    xb = H.make_act(M, K, dt, seed=seed + M, dist=xdist)
     bb = H.make_bias(N, dt, seed=seed + 1) if bias else None
     oc, osc = oracle.weight_quantize(wb, dt, bits, g)
     packed = H.gfx950_from_q(H.q_from_canonical(oc, bits), bits)
@@ -55,7 +55,41 @@ def test_linear_small_shapes_all_m(G, oracle, dt, bits, g):
             check(G, oracle, dt, bits, g, M, K, N, bias=(M % 2 == 1), seed=M)
 
 
-KERNEL_STREAM, KERNEL_GEMM = 1, 2
+KERNEL_STREAM, KERNEL_GEMM, KERNEL_BATCH = 1, 2, 3
+
+
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("g", [-1, 64, 128])
+def test_linear_batch_kernel_pinned(G, oracle, dt, bits, g):
+    # the batched decode kernel on every K it is built for (every wavefront
+    # owns 1, 2 or 4 tiles of a strip); fewer strips than CUs, one, two and
+    # many strips per workgroup (more than the weight ring holds, more than one
+    # run of seven strips shares the LDS); N that is 16 mod 32
+    shapes = [(2048, 1024), (4096, 4128), (8192, 272), (2048, 12368), (2048, 48), (2048, 36880), (4096, 32800)]
+    for K, N in shapes:
+        if K == 8192 and (bits == 8 or g == 64):
+            with pytest.raises(ValueError):  # not built: the A fragments alone take 64 registers
+                check(G, oracle, dt, bits, g, 4, K, N, seed=1, kernel=KERNEL_BATCH)
+            continue
+        for M in ((1, 2, 3, 5, 8, 13, 16) if K * N < 5e6 else ((2, 16) if K * N < 5e7 else (7,))):
+            print("case", dt, bits, g, K, N, M, flush=True)
+            check(G, oracle, dt, bits, g, M, K, N, bias=(M % 2 == 1), seed=M, kernel=KERNEL_BATCH)
+    # refused: more than 16 rows, any other K
+    with pytest.raises(ValueError):
+        check(G, oracle, dt, bits, g, 17, 2048, 256, seed=1, kernel=KERNEL_BATCH)
+    with pytest.raises(ValueError):
+        check(G, oracle, dt, bits, g, 4, 1024, 256, seed=1, kernel=KERNEL_BATCH)
+
+
+@pytest.mark.parametrize("kernel", [KERNEL_STREAM, KERNEL_BATCH, KERNEL_GEMM])
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+def test_linear_int4_offset_cancellation_with_biased_activations(G, oracle, dt, kernel):
+    # activations that are all positive (what follows a gelu or a relu) make the
+    # term that cancels the dequantiser's offset as large as it gets; the sums
+    # must still be far inside the bar.  Ragged N (16 mod 32) on every kernel.
+    for M, K, N in ((4, 4096, 1040), (16, 2048, 48)):
+        check(G, oracle, dt, 4, 128, M, K, N, seed=5, xdist="uniform", tol32=1e-4, kernel=kernel)
 
 
 @pytest.mark.parametrize("dt", [H.F16, H.BF16])
@@ -129,6 +163,8 @@ def test_linear_random_shapes_all_kernels(G, oracle):
         K = 64 * int(rng.integers(1, 33))
         N = (32 if bits == 4 else 16) * int(rng.integers(1, 41))
         kernels = [None, KERNEL_GEMM] + ([KERNEL_STREAM] if M <= 64 else [])
+        if M <= 16 and K == 2048:
+            kernels.append(KERNEL_BATCH)
         kernel = kernels[int(rng.integers(len(kernels)))]
         print("case", case, dt, bits, g, M, K, N, kernel, flush=True)
         kw = {} if kernel is None else {"kernel": kernel}
