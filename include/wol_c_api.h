@@ -180,6 +180,40 @@ int wol_linear_f32(const void* x, const void* codes, const void* bias,
                    int64_t N, int bits, int group_size, float* out_f32,
                    void* workspace, size_t workspace_bytes, void* stream);
 
+/* Activation fused behind the linear by wol_linear_fused.  The reference's
+ * GEMV takes act_method "None" or "gelu"
+ * (paddle/phi/kernels/funcs/weight_only_gemv.h:33, gelu formula
+ * funcs/weight_only_gemv.cu:147-157, applied to accumulator + bias in float,
+ * :1045-1046); swiglu is what its MoE FFN runs on the output of the first
+ * linear (paddle/phi/kernels/fusion/cutlass/moe_ffn.cu:133-139). */
+#define WOL_ACT_NONE 0
+#define WOL_ACT_GELU 1   /* v * 0.5 * (1 + tanh(0.7978845608 * (v + 0.044715 v^3)))      */
+#define WOL_ACT_SWIGLU 2 /* out[m, n] = silu(v[m, n]) * v[m, n + N/2], n < N/2: out is
+                            [M, N/2]; needs N % 32 == 0                                */
+
+/*
+ * weight_only_linear with what usually stands on either side of it folded in:
+ *   x' = T(x * pre_scale)            apply_per_channel_scale, when pre_scale != NULL
+ *                                    (paddle/phi/kernels/gpu/apply_per_channel_scale_kernel.cu:93-126:
+ *                                    each product rounded once to T, bit for bit
+ *                                    what wol_apply_per_channel_scale writes)
+ *   v  = x' . dequant(W) + bias      fp32 accumulation, as wol_linear
+ *   out = T(act(v))                  act applied to the fp32 sum, one rounding
+ * pre_scale: [K] T.  out: [M, N] T, or [M, N/2] T for WOL_ACT_SWIGLU.
+ * The decode kernels apply pre_scale while they load the activations and the
+ * activation in their epilogues; the MFMA GEMM applies gelu in its epilogue
+ * and takes pre-scaled activations and swiglu through the workspace (one
+ * element-wise pass each, inside this call).  The workspace is therefore
+ * required whenever wol_linear_fused_workspace() is non-zero.
+ */
+size_t wol_linear_fused_workspace(int64_t M, int64_t K, int64_t N, int bits,
+                                  int group_size, int has_pre_scale, int act);
+int wol_linear_fused(const void* x, const void* pre_scale, const void* codes,
+                     const void* bias, const void* scale, int dtype, int64_t M,
+                     int64_t K, int64_t N, int bits, int group_size, int act,
+                     void* out, void* workspace, size_t workspace_bytes,
+                     void* stream);
+
 /* Kernel choice of wol_linear_on. */
 enum wol_kernel {
   WOL_KERNEL_AUTO = 0,   /* what wol_linear does                                */

@@ -408,6 +408,86 @@ void wo_dequantize_f32(const int8_t* codes, const uint16_t* scale, int64_t K,
                 WO_CAST_RNE, out32, NULL);
 }
 
+/* ---- fused epilogues ------------------------------------------------------ */
+
+/* The activations that follow weight_only_linear, applied to the fp32 sum
+ * (accumulator + bias) before the one cast to T.
+ *   act 1, gelu: the tanh form of the reference's GEMV epilogue,
+ *     paddle/phi/kernels/funcs/weight_only_gemv.cu:147-157 (GeluActivation:
+ *     v * 0.5 * (1 + tanh(0.7978845608028654 * (v + 0.044715 v^3)))), applied
+ *     as at :1045-1046 to v + bias in float.  The reference's tanh is the
+ *     hardware approximation (tanh.approx.f32, :137-138); here the exact tanh
+ *     in double, the value every approximation approximates.
+ *   act 2, swiglu: out[m, n] = silu(g) * u for n < N/2 with g, u the sums of
+ *     columns n and n + N/2 (the halves paddle.incubate.nn.functional.swiglu
+ *     splits a single input into, paddle/phi/kernels/gpu/swiglu_kernel.cu:32-52;
+ *     silu(g) = g / (1 + exp(-g)), SwiGLUFunctor in
+ *     paddle/phi/kernels/funcs/activation_functor.h).  The reference applies
+ *     it to the rounded output of the linear (fusion/cutlass/moe_ffn.cu:133-139);
+ *     here, as in the fused kernel, to the fp32 sums, rounded once.
+ * in32: [M, N] fp32 sums (wo_linear's out32).  out32/outT: [M, N] (gelu) or
+ * [M, N/2] (swiglu). */
+void wo_activation(const float* in32, int64_t M, int64_t N, int act, int dtype,
+                   float* out32, uint16_t* outT) {
+  if (act == 2) {
+    const int64_t H = N / 2;
+    for (int64_t m = 0; m < M; ++m)
+      for (int64_t n = 0; n < H; ++n) {
+        const double g = (double)in32[m * N + n], u = (double)in32[m * N + H + n];
+        const float v = (float)(g / (1.0 + exp(-g)) * u);
+        out32[m * H + n] = v;
+        if (outT) outT[m * H + n] = wo_from_f32(v, dtype, WO_CAST_RNE);
+      }
+    return;
+  }
+  for (int64_t i = 0; i < M * N; ++i) {
+    const double x = (double)in32[i];
+    float v = in32[i];
+    if (act == 1)
+      v = (float)(x * 0.5 * (1.0 + tanh(0.7978845608028654 * (x + 0.044715 * x * x * x))));
+    out32[i] = v;
+    if (outT) outT[i] = wo_from_f32(v, dtype, WO_CAST_RNE);
+  }
+}
+
+/* ---- x_grad of weight_only_linear ----------------------------------------- */
+
+/* WeightOnlyLinearGradKernel, paddle/phi/kernels/gpu/weight_only_linear_grad_kernel.cu:27-72:
+ *   x_grad[M, K] = out_grad[M, N] . dequant(W)[K, N]^T.
+ * The reference dequantises to T first (:52-60) and hands the product to a
+ * library GEMM (:61-69), so code * scale is rounded to T there.  This path's
+ * contract keeps the dequantised weight in fp32, float(code) * float(scale)
+ * (exact), and accumulates in fp32 (acc64 = 0) or double (acc64 = 1) over n in
+ * ascending order; one cast to T at the end. */
+void wo_linear_grad(const uint16_t* out_grad, const int8_t* codes,
+                    const uint16_t* scale, int64_t M, int64_t K, int64_t N,
+                    int dtype, int bits, int64_t group_size, int nibble_bias,
+                    int acc64, float* out32, uint16_t* outT) {
+  float* wdq = (float*)malloc((size_t)K * (size_t)N * sizeof(float));
+  wo_dequantize(codes, scale, K, N, dtype, bits, group_size, nibble_bias,
+                WO_CAST_RNE, wdq, NULL);
+  float* g = (float*)malloc((size_t)N * sizeof(float));
+  for (int64_t m = 0; m < M; ++m) {
+    for (int64_t n = 0; n < N; ++n) g[n] = wo_to_f32(out_grad[m * N + n], dtype);
+    for (int64_t k = 0; k < K; ++k) {
+      const float* wr = wdq + k * N;
+      float v;
+      if (acc64) {
+        double a = 0.0;
+        for (int64_t n = 0; n < N; ++n) a += (double)g[n] * (double)wr[n];
+        v = (float)a;
+      } else {
+        float a = 0.0f;
+        for (int64_t n = 0; n < N; ++n) a += g[n] * wr[n];
+        v = a;
+      }
+      out32[m * K + k] = v;
+      if (outT) outT[m * K + k] = wo_from_f32(v, dtype, WO_CAST_RNE);
+    }
+  }
+  free(g); free(wdq);
+}
+
 /* ---- pre-quant activation smoothing ------------------------------------ */
 
 /* out[r,c] = T(x[r,c] * scales[c]): ApplyPerChannelScaleKernel

@@ -67,6 +67,11 @@ def lib():
                                     ctypes.c_void_p, ctypes.c_void_p]
         L.wo_linear.argtypes = [_u16p, _i8p, ctypes.c_void_p, _u16p, _i64, _i64, _i64, _int, _int,
                                 _i64, _int, _int, _f32p, ctypes.c_void_p]
+        L.wo_activation.argtypes = [_f32p, _i64, _i64, _int, _int, _f32p, ctypes.c_void_p]
+        L.wo_activation.restype = None
+        L.wo_linear_grad.argtypes = [_u16p, _i8p, _u16p, _i64, _i64, _i64, _int, _int, _i64, _int, _int, _f32p,
+                                     ctypes.c_void_p]
+        L.wo_linear_grad.restype = None
         _lib = L
     return _lib
 
@@ -191,6 +196,45 @@ def linear(x_bits, codes, scale, bias_bits, dtype, bits, group_size=-1, nibble_b
         bias_ptr = bias_bits.ctypes.data
     lib().wo_linear(x_bits, codes, bias_ptr, scale, M, K, N, dtype, bits, group_size, nibble_bias,
                     1 if acc64 else 0, out32, outT.ctypes.data)
+    return out32, outT
+
+
+ACT_NONE, ACT_GELU, ACT_SWIGLU = 0, 1, 2
+
+
+def activation(in32, act, dtype):
+    """The fused epilogue on fp32 sums [M,N]: returns (fp32, T-bits), [M,N] for
+    none/gelu, [M,N/2] for swiglu."""
+    in32 = np.ascontiguousarray(in32, dtype=np.float32)
+    M, N = in32.shape
+    No = N // 2 if act == ACT_SWIGLU else N
+    out32 = np.empty((M, No), np.float32)
+    outT = np.empty((M, No), np.uint16)
+    lib().wo_activation(in32, M, N, act, dtype, out32, outT.ctypes.data)
+    return out32, outT
+
+
+def linear_fused(x_bits, pre_scale_bits, codes, scale, bias_bits, dtype, bits, group_size=-1, act=ACT_NONE):
+    """apply_per_channel_scale (when pre_scale_bits is given), weight_only_linear
+    and the activation, as the fused entry point composes them."""
+    if pre_scale_bits is not None:
+        x_bits = apply_per_channel_scale(x_bits, pre_scale_bits, dtype)
+    o32, _ = linear(x_bits, codes, scale, bias_bits, dtype, bits, group_size)
+    return activation(o32, act, dtype)
+
+
+def linear_grad(out_grad_bits, codes, scale, dtype, bits, group_size=-1, acc64=False):
+    """x_grad [M,K] = out_grad [M,N] . dequant(W)[K,N]^T with the fp32 dequantised
+    weight.  Returns (fp32, T-bits)."""
+    g = np.ascontiguousarray(out_grad_bits, dtype=np.uint16)
+    codes = np.ascontiguousarray(codes, dtype=np.int8)
+    scale = np.ascontiguousarray(scale, dtype=np.uint16)
+    M, N = g.shape
+    K = codes.shape[0]
+    out32 = np.empty((M, K), np.float32)
+    outT = np.empty((M, K), np.uint16)
+    lib().wo_linear_grad(g, codes, scale, M, K, N, dtype, bits, group_size, 0, 1 if acc64 else 0, out32,
+                         outT.ctypes.data)
     return out32, outT
 
 

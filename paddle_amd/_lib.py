@@ -27,6 +27,8 @@ SYMBOLS = (
     "wol_linear_f32",
     "wol_linear_workspace_for",
     "wol_linear_on",
+    "wol_linear_fused_workspace",
+    "wol_linear_fused",
     "wol_repack",
     "wol_code_offset",
     "wol_apply_per_channel_scale",
@@ -75,6 +77,10 @@ def _load():
     lib.wol_linear_workspace_for.restype = sz
     lib.wol_linear_on.argtypes = [vp, vp, vp, vp, ci, i64, i64, i64, ci, ci, vp, ci, ci, vp, sz, vp]
     lib.wol_linear_on.restype = ci
+    lib.wol_linear_fused_workspace.argtypes = [i64, i64, i64, ci, ci, ci, ci]
+    lib.wol_linear_fused_workspace.restype = sz
+    lib.wol_linear_fused.argtypes = [vp, vp, vp, vp, vp, ci, i64, i64, i64, ci, ci, ci, vp, vp, sz, vp]
+    lib.wol_linear_fused.restype = ci
     lib.wol_repack.argtypes = [vp, ci, vp, ci, i64, i64, ci, vp]
     lib.wol_repack.restype = ci
     lib.wol_code_offset.argtypes = [ci, i64, i64, ci, i64, i64, ctypes.POINTER(ci)]
@@ -101,6 +107,8 @@ lib = _load()
 # statuses that are argument errors (the reference raises InvalidArgument,
 # which Paddle surfaces as ValueError)
 _ARG_ERRORS = {1, 2, 3, 4, 5, 6, 7, 8, 9}
+
+ACT_NONE, ACT_GELU, ACT_SWIGLU = 0, 1, 2
 
 # wol_kernel
 KERNEL_AUTO, KERNEL_STREAM, KERNEL_GEMM, KERNEL_BATCH = 0, 1, 2, 3

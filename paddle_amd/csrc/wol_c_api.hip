@@ -119,7 +119,8 @@ int resolve_kernel(int kernel, int64_t M, int64_t K, int64_t N, int bits, int gr
 
 int linear_impl(const void* x, const void* codes, const void* bias, const void* scale, int dtype,
                 int64_t M, int64_t K, int64_t N, int bits, int group_size, void* out, bool out_f32,
-                int kernel, void* workspace, size_t workspace_bytes, void* stream) {
+                int kernel, void* workspace, size_t workspace_bytes, void* stream,
+                const wol::Fuse& fuse = wol::Fuse()) {
   const int rc = check_problem(dtype, K, N, bits, group_size);
   if (rc != WOL_OK) return rc;
   if (M < 0 || M > (int64_t{1} << 24)) return WOL_ERR_BAD_SHAPE;
@@ -139,12 +140,12 @@ int linear_impl(const void* x, const void* codes, const void* bias, const void* 
   const int which = resolve_kernel(kernel, M, K, N, bits, group_size, have_ws);
   if (which == WOL_KERNEL_BATCH)
     return wol::launch_linear_batch(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out,
-                                    out_f32, s);
+                                    out_f32, s, fuse);
   if (which == WOL_KERNEL_STREAM)
     return wol::launch_linear_stream(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out,
-                                     out_f32, s);
+                                     out_f32, s, fuse);
   return wol::launch_linear_gemm(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out,
-                                 out_f32, workspace, workspace_bytes, s);
+                                 out_f32, workspace, workspace_bytes, s, fuse);
 }
 
 }  // namespace
@@ -258,6 +259,88 @@ int wol_linear_f32(const void* x, const void* codes, const void* bias, const voi
                    float* out_f32, void* workspace, size_t workspace_bytes, void* stream) {
   return linear_impl(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out_f32, true,
                      WOL_KERNEL_AUTO, workspace, workspace_bytes, stream);
+}
+
+namespace {
+
+// How wol_linear_fused lays a call out: which parts the linear kernel applies
+// itself and what goes through the workspace ([the linear's own scratch]
+// [pre-scaled activations M x K T] [fp32 sums M x N]).
+struct FusedPlan {
+  bool prepass;          // the activations are scaled by a pass of the prescale kernel
+  bool swiglu_pass;      // the linear writes fp32 sums, a pass turns them into T(swiglu)
+  size_t linear_ws, x_off, sums_off, total;
+};
+
+FusedPlan plan_fused(int64_t M, int64_t K, int64_t N, int bits, int group_size, bool has_pre, int act) {
+  FusedPlan f{};
+  const size_t lws = wol_linear_workspace(M, K, N, bits, group_size);
+  const int which = resolve_kernel(WOL_KERNEL_AUTO, M, K, N, bits, group_size, true);
+  const bool fused_pre = (which == WOL_KERNEL_BATCH && wol::linear_batch_fuses_pre_scale(K, bits, group_size)) ||
+                         (which == WOL_KERNEL_STREAM && M == 1);
+  f.prepass = has_pre && !fused_pre;
+  f.swiglu_pass = act == WOL_ACT_SWIGLU;
+  auto up = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
+  f.linear_ws = lws;
+  f.x_off = up(lws);
+  f.sums_off = f.x_off + (f.prepass ? up(static_cast<size_t>(M) * K * 2) : 0);
+  f.total = f.sums_off + (f.swiglu_pass ? up(static_cast<size_t>(M) * N * 4) : 0);
+  if (!f.prepass && !f.swiglu_pass) f.total = lws;
+  return f;
+}
+
+}  // namespace
+
+size_t wol_linear_fused_workspace(int64_t M, int64_t K, int64_t N, int bits, int group_size,
+                                  int has_pre_scale, int act) {
+  if (check_problem(WOL_DTYPE_F16, K, N, bits, group_size) != WOL_OK || M <= 0) return 0;
+  if (act != WOL_ACT_NONE && act != WOL_ACT_GELU && act != WOL_ACT_SWIGLU) return 0;
+  return plan_fused(M, K, N, bits, group_size, has_pre_scale != 0, act).total;
+}
+
+int wol_linear_fused(const void* x, const void* pre_scale, const void* codes, const void* bias,
+                     const void* scale, int dtype, int64_t M, int64_t K, int64_t N, int bits,
+                     int group_size, int act, void* out, void* workspace, size_t workspace_bytes,
+                     void* stream) {
+  const int rc = check_problem(dtype, K, N, bits, group_size);
+  if (rc != WOL_OK) return rc;
+  if (M < 0 || M > (int64_t{1} << 24)) return WOL_ERR_BAD_SHAPE;
+  if (act != WOL_ACT_NONE && act != WOL_ACT_GELU && act != WOL_ACT_SWIGLU) return WOL_ERR_BAD_SHAPE;
+  if (act == WOL_ACT_SWIGLU && N % 32 != 0) return WOL_ERR_BAD_SHAPE;
+  if (M == 0) return WOL_OK;
+  if (x == nullptr || codes == nullptr || scale == nullptr || out == nullptr) return WOL_ERR_NULL_POINTER;
+  if (!aligned16(x) || !aligned16(codes) || !aligned16(scale)) return WOL_ERR_ALIGNMENT;
+  if (pre_scale != nullptr && !aligned16(pre_scale)) return WOL_ERR_ALIGNMENT;
+  const FusedPlan f = plan_fused(M, K, N, bits, group_size, pre_scale != nullptr, act);
+  if (f.prepass || f.swiglu_pass) {
+    if (workspace == nullptr || workspace_bytes < f.total) return WOL_ERR_WORKSPACE;
+    if (!aligned16(workspace)) return WOL_ERR_ALIGNMENT;
+  }
+  if (const int dv = require_gfx950(); dv != WOL_OK) return dv;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  unsigned char* ws = static_cast<unsigned char*>(workspace);
+  wol::Fuse fuse;
+  fuse.act = act == WOL_ACT_GELU ? WOL_ACT_GELU : WOL_ACT_NONE;
+  const void* xin = x;
+  if (f.prepass) {
+    const int prc = wol::launch_prescale(x, pre_scale, dtype, M, K, ws + f.x_off, s);
+    if (prc != WOL_OK) return prc;
+    xin = ws + f.x_off;
+  } else {
+    fuse.pre_scale = pre_scale;
+  }
+  // without extra passes the caller's scratch is the linear's as it is (it stays optional)
+  const bool passes = f.prepass || f.swiglu_pass;
+  void* lws = passes ? (f.linear_ws > 0 ? ws : nullptr) : workspace;
+  const size_t lws_bytes = passes ? f.linear_ws : workspace_bytes;
+  if (!f.swiglu_pass)
+    return linear_impl(xin, codes, bias, scale, dtype, M, K, N, bits, group_size, out, false, WOL_KERNEL_AUTO,
+                       lws, lws_bytes, stream, fuse);
+  float* sums = reinterpret_cast<float*>(ws + f.sums_off);
+  const int lrc = linear_impl(xin, codes, bias, scale, dtype, M, K, N, bits, group_size, sums, true,
+                              WOL_KERNEL_AUTO, lws, lws_bytes, stream, fuse);
+  if (lrc != WOL_OK) return lrc;
+  return wol::launch_swiglu_f32(sums, dtype, M, N, out, s);
 }
 
 int wol_linear_on(const void* x, const void* codes, const void* bias, const void* scale, int dtype,

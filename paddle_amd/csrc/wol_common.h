@@ -182,6 +182,50 @@ __device__ inline uint16_t cast_out(float f) {
   return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
 }
 
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// ---------------------------------------------------------------------------
+// What wol_linear_fused adds around the linear: the activation smoothing
+// (apply_per_channel_scale) in front and an activation behind.
+// ---------------------------------------------------------------------------
+
+// x * s for two T values packed in a dword, each product rounded once to T
+// (RNE): the arithmetic of apply_per_channel_scale (the product of two T values
+// is exact in fp32).
+template <int DT>
+__device__ inline uint32_t prescale_pair(uint32_t x2, uint32_t s2) {
+  const float lo = to_f32<DT>(static_cast<uint16_t>(x2 & 0xFFFFu)) * to_f32<DT>(static_cast<uint16_t>(s2 & 0xFFFFu));
+  const float hi = to_f32<DT>(static_cast<uint16_t>(x2 >> 16)) * to_f32<DT>(static_cast<uint16_t>(s2 >> 16));
+  return static_cast<uint32_t>(cast_out<DT>(lo)) | (static_cast<uint32_t>(cast_out<DT>(hi)) << 16);
+}
+
+// The same for the eight values of an A fragment and the scales of their eight k.
+template <int DT>
+__device__ inline u32x4 prescale_frag(u32x4 a, u32x4 s) {
+  u32x4 o;
+  o.x = prescale_pair<DT>(a.x, s.x);
+  o.y = prescale_pair<DT>(a.y, s.y);
+  o.z = prescale_pair<DT>(a.z, s.z);
+  o.w = prescale_pair<DT>(a.w, s.w);
+  return o;
+}
+
+// gelu in its tanh form (paddle/phi/kernels/funcs/weight_only_gemv.cu:147-157),
+// on the fp32 sum; tanh(u) = 1 - 2 / (exp(2u) + 1), which saturates correctly
+// at both ends.
+__device__ inline float act_gelu(float v) {
+  const float u = 0.7978845608028654f * (v + 0.044715f * v * v * v);
+  const float t = 1.0f - 2.0f / (__expf(2.0f * u) + 1.0f);
+  return v * 0.5f * (1.0f + t);
+}
+
+// silu(g) * u, the swiglu of a gate and an up value
+// (paddle/phi/kernels/gpu/swiglu_kernel.cu:32-52).
+__device__ inline float act_swiglu(float g, float u) { return g / (1.0f + __expf(-g)) * u; }
+
+// act: WOL_ACT_NONE or WOL_ACT_GELU (swiglu combines two sums and is applied where both are at hand)
+__device__ inline float act_apply(float v, int act) { return act == WOL_ACT_GELU ? act_gelu(v) : v; }
+
 // Strips (16 columns) that share a workgroup of the streaming linear kernel.
 // Two halve the activation traffic out of L2 (N/16 * rows * K * 2 bytes, rows
 // = M rounded up to a power of two, at most 16 per operand) but also the
@@ -200,6 +244,13 @@ inline int stream_strips_per_workgroup(int64_t M, int64_t N, int bits) {
   return 1;
 }
 
+// What wol_linear_fused adds to a linear call.  pre_scale: [K] T or null.
+// act: a WOL_ACT_* value.  The launchers say which parts they apply themselves.
+struct Fuse {
+  const void* pre_scale = nullptr;
+  int act = 0;
+};
+
 // Launchers implemented in the .hip files; each returns a wol_status.
 int launch_quantize(const void* w, int dtype, int64_t K, int64_t N, int bits, int group_size,
                     int round_mode, int layout, void* codes, void* scale, bool scale_f32,
@@ -216,15 +267,16 @@ int launch_repack(const void* in, int layout_in, void* out, int layout_out, int6
                   int bits, hipStream_t stream);
 int launch_linear_stream(const void* x, const void* codes, const void* bias, const void* scale,
                          int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
-                         void* out, bool out_f32, hipStream_t stream);
+                         void* out, bool out_f32, hipStream_t stream, const Fuse& f = Fuse());
 // The batched decode kernel (2 to 16 rows; one row works too; K = 2048, 4096, and
 // 8192 for int4 without groups of 64).
 bool linear_batch_supports(int64_t M, int64_t K, int bits, int group_size);
+bool linear_batch_fuses_pre_scale(int64_t K, int bits, int group_size);
 int linear_batch_cus();  // CUs of the current device (256 when it cannot be asked)
 void plan_linear_batch(int64_t K, int64_t N, int bits, int* grid, int* tpw);
 int launch_linear_batch(const void* x, const void* codes, const void* bias, const void* scale,
                         int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
-                        void* out, bool out_f32, hipStream_t stream);
+                        void* out, bool out_f32, hipStream_t stream, const Fuse& f = Fuse());
 // One-line descriptions of what the launchers would run for a problem.
 void describe_linear_stream(int64_t M, int64_t K, int64_t N, int bits, int group_size, char* buf, size_t n);
 void describe_linear_gemm(int64_t M, int64_t K, int64_t N, int bits, int group_size, size_t ws_bytes,
@@ -232,13 +284,14 @@ void describe_linear_gemm(int64_t M, int64_t K, int64_t N, int bits, int group_s
 int launch_linear_gemm(const void* x, const void* codes, const void* bias, const void* scale,
                        int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
                        void* out, bool out_f32, void* workspace, size_t workspace_bytes,
-                       hipStream_t stream);
+                       hipStream_t stream, const Fuse& f = Fuse());
 int launch_read_floor(const void* codes, int64_t K, int64_t N, int bits, void* out,
                       hipStream_t stream);
 int launch_mfma_ceiling(const void* operands, int workgroups, int iters, float* out,
                         hipStream_t stream);
 int launch_prescale(const void* x, const void* scales, int dtype, int64_t rows, int64_t cols,
                     void* out, hipStream_t stream);
+int launch_swiglu_f32(const float* in, int dtype, int64_t M, int64_t N, void* out, hipStream_t stream);
 int launch_llm_int8_linear(const void* x, const void* weight, const void* bias, const float* wscale,
                            float threshold, int dtype, int64_t M, int64_t K, int64_t N, void* out,
                            void* workspace, hipStream_t stream);

@@ -9,8 +9,6 @@
 
 namespace wol {
 
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-
 // Codes of one k step (8 per lane) -> four dwords of T pairs holding
 // code + offset exactly, and the B operand that cancels the offset.
 //   int4/bf16: nibble | 0x4300      = 128 + (code + 8)      offset 136

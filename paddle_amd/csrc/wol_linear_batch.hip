@@ -73,6 +73,8 @@ struct BatchParams {
   int gshift;   // log2(group size), -1 per-channel
   int out_f32;
   int strips_q, strips_r;  // strips per workgroup: N / 16 = grid * strips_q + strips_r
+  const uint16_t* pre;     // [K] per-channel scales of the activations, or null
+  int act;                 // WOL_ACT_NONE or WOL_ACT_GELU
 };
 
 // G: 0 per-channel, else the group size.  TPW: weight tiles (1 KiB, 64 or 128
@@ -82,7 +84,9 @@ struct BatchParams {
 // younger loads may still be in flight (s_waitcnt vmcnt(n) with n > 0); a load
 // under a condition would make every later wait a wait for all loads.
 // IT: tiles per item, D: items in the ring (a multiple of TPW / IT).
-template <int DT, int BITS, int G, int TPW, int IT, int D>
+// PRE: the activations are multiplied by p.pre (each product rounded to T as
+// apply_per_channel_scale rounds it) once, in the registers they stay in.
+template <int DT, int BITS, int G, int TPW, int IT, int D, bool PRE>
 __global__ __launch_bounds__(kBatchWaves * 64) void batch_kernel(const BatchParams p) {
   constexpr int WK = kBatchWaves;
   constexpr int TK = BITS == 8 ? 64 : 128;   // k per 1 KiB weight tile
@@ -127,6 +131,11 @@ __global__ __launch_bounds__(kBatchWaves * 64) void batch_kernel(const BatchPara
 #pragma unroll
     for (int s = 0; s < TPW * SPT; ++s) A[s] = *reinterpret_cast<const u32x4*>(xrow + s * 32);
   }
+  // The activation scales of the wavefront's k (the same for every row): lane
+  // 4 * s + kb holds the eight scales that go with A[s] in lane group kb, one
+  // 16-byte load for the whole run; they are handed out by lane permutes later.
+  u32x4 PS = {0u, 0u, 0u, 0u};
+  if (PRE) PS = *reinterpret_cast<const u32x4*>(p.pre + t0 * TK + (lane % (TPW * SPT * 4)) * 8);
 
   u32x4 W[D][IT];
   uint16_t S[D][NS];
@@ -192,6 +201,18 @@ __global__ __launch_bounds__(kBatchWaves * 64) void batch_kernel(const BatchPara
       lbi[threadIdx.x] = bstage;
     }
 
+    if (PRE && !have_cc) {  // once, after the first ring has been requested
+#pragma unroll
+      for (int s = 0; s < TPW * SPT; ++s) {
+        const int src = (4 * s + kb) * 4;  // byte address of the source lane for ds_bpermute
+        u32x4 ps;
+        ps.x = __builtin_amdgcn_ds_bpermute(src, PS.x);
+        ps.y = __builtin_amdgcn_ds_bpermute(src, PS.y);
+        ps.z = __builtin_amdgcn_ds_bpermute(src, PS.z);
+        ps.w = __builtin_amdgcn_ds_bpermute(src, PS.w);
+        A[s] = prescale_frag<DT>(A[s], ps);
+      }
+    }
     if (kKeepCancel && !have_cc) {
 #pragma unroll
       for (int c = 0; c < TPW * CPT; ++c) {
@@ -200,8 +221,8 @@ __global__ __launch_bounds__(kBatchWaves * 64) void batch_kernel(const BatchPara
         for (int s = 0; s < SPC; ++s) cc = mfma16<DT>(A[c * SPC + s], cancel, cc);
         ccs[c] = cc;
       }
-      have_cc = true;
     }
+    have_cc = true;
     f32x4 tot = {0.f, 0.f, 0.f, 0.f};
     for (int base = 0; base < nitems; base += D) {
 #pragma unroll
@@ -266,7 +287,7 @@ __global__ __launch_bounds__(kBatchWaves * 64) void batch_kernel(const BatchPara
           const int cl = sl * kStripCols + (l & 15);
           const float ep_scale = G == 0 ? to_f32<DT>(lsc[cl]) : 1.0f;
           const float ep_bias = p.bias != nullptr ? to_f32<DT>(lbi[cl]) : 0.0f;
-          s = s * ep_scale + ep_bias;
+          s = act_apply(s * ep_scale + ep_bias, p.act);
           const int64_t o = static_cast<int64_t>(m) * N + (sr + sl) * kStripCols + (l & 15);
           if (p.out_f32)
             static_cast<float*>(p.out)[o] = s;
@@ -293,6 +314,7 @@ __global__ __launch_bounds__(kBatchWaves * 64) void batch_kernel(const BatchPara
 struct Args {
   const void* x; const void* codes; const void* bias; const void* scale; void* out;
   int M, K, N, gshift, out_f32; hipStream_t stream;
+  const void* pre; int act;
 };
 
 inline int num_cus() {
@@ -326,10 +348,10 @@ inline size_t batch_lds(int64_t K, int64_t N, int group_size, int grid) {
   return static_cast<size_t>(per_wg * kBatchWaves * 1024 + 2 * per_wg * kStripCols * 2);
 }
 
-template <int DT, int BITS, int G, int TPW, int IT, int D>
-void launch_one(const Args& a, int grid) {
+template <int DT, int BITS, int G, int TPW, int IT, int D, bool PRE>
+void launch_pre(const Args& a, int grid) {
   const size_t lds = batch_lds(a.K, a.N, G, grid);
-  auto kern = batch_kernel<DT, BITS, G, TPW, IT, D>;
+  auto kern = batch_kernel<DT, BITS, G, TPW, IT, D, PRE>;
   static std::atomic<uint32_t> configured{0};  // per instantiation
   allow_lds(reinterpret_cast<const void*>(kern), 160 * 1024, configured);
   BatchParams p;
@@ -343,7 +365,27 @@ void launch_one(const Args& a, int grid) {
   p.out_f32 = a.out_f32;
   p.strips_q = a.N / kStripCols / grid;
   p.strips_r = a.N / kStripCols % grid;
+  p.pre = PRE ? static_cast<const uint16_t*>(a.pre) : nullptr;
+  p.act = a.act;
   kern<<<dim3(static_cast<unsigned>(grid)), dim3(kBatchWaves * 64), lds, a.stream>>>(p);
+}
+
+// The fused activation scales are built where the registers allow: A
+// fragments of 32 registers or fewer (K <= 4096), except int8 codes with
+// group-wise scales at K = 4096.
+constexpr bool pre_fits(int bits, int group, int k_steps_per_wave) {
+  return k_steps_per_wave <= 8 && !(bits == 8 && group != 0 && k_steps_per_wave == 8);
+}
+
+template <int DT, int BITS, int G, int TPW, int IT, int D>
+void launch_one(const Args& a, int grid) {
+  if constexpr (pre_fits(BITS, G, TPW * (BITS == 8 ? 2 : 4))) {
+    if (a.pre != nullptr) {
+      launch_pre<DT, BITS, G, TPW, IT, D, true>(a, grid);
+      return;
+    }
+  }
+  launch_pre<DT, BITS, G, TPW, IT, D, false>(a, grid);
 }
 
 // tpw = K / (16 * tile depth): 1, 2 or 4.  Items and ring depths by what the
@@ -382,6 +424,11 @@ bool linear_batch_supports(int64_t M, int64_t K, int bits, int group_size) {
 
 int linear_batch_cus() { return num_cus(); }
 
+// Whether launch_linear_batch applies a Fuse::pre_scale itself for this K.
+bool linear_batch_fuses_pre_scale(int64_t K, int bits, int group_size) {
+  return pre_fits(bits, group_size > 0 ? group_size : 0, static_cast<int>(K / 32 / kBatchWaves));
+}
+
 // Grid (workgroups: one per CU, fewer when there are fewer strips) and the
 // weight tiles of a strip per wavefront.
 void plan_linear_batch(int64_t K, int64_t N, int bits, int* grid, int* tpw) {
@@ -393,12 +440,13 @@ void plan_linear_batch(int64_t K, int64_t N, int bits, int* grid, int* tpw) {
 
 int launch_linear_batch(const void* x, const void* codes, const void* bias, const void* scale,
                         int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
-                        void* out, bool out_f32, hipStream_t stream) {
+                        void* out, bool out_f32, hipStream_t stream, const Fuse& f) {
   const int gshift = group_size == 64 ? 6 : (group_size == 128 ? 7 : -1);
   int grid = 1, tpw = 1;
   plan_linear_batch(K, N, bits, &grid, &tpw);
   const Args a{x, codes, bias, scale, out, static_cast<int>(M), static_cast<int>(K),
-               static_cast<int>(N), gshift, out_f32 ? 1 : 0, stream};
+               static_cast<int>(N), gshift, out_f32 ? 1 : 0, stream,
+               linear_batch_fuses_pre_scale(K, bits, group_size) ? f.pre_scale : nullptr, f.act};
   if (dtype == WOL_DTYPE_BF16) {
     if (bits == 8) launch_g<WOL_DTYPE_BF16, 8>(a, grid, tpw); else launch_g<WOL_DTYPE_BF16, 4>(a, grid, tpw);
   } else {

@@ -1,18 +1,20 @@
-// weight_only_linear for large M (prefill): an MFMA GEMM.
+// weight_only_linear for large M (prefill): MFMA GEMMs.
 //
-// A workgroup of WM x WN wavefronts computes a BM x BN tile of the output,
-// each wavefront a (16*TM) x (16*TN) sub-tile with v_mfma_f32_16x16x32.  The
-// activations of a k tile are staged in LDS (double buffered, padded rows,
-// read back as A fragments).  The packed weights need no staging: the GFX950
-// layout already stores them in B-fragment order, so every lane loads its 16
-// bytes per strip straight from global memory (prefetched one k tile ahead)
-// and dequantises them in registers to exact signed bf16/fp16 integers; the
-// cost of that is amortised over the TM row tiles of the wavefront.  Scales
-// are applied to fp32 accumulators -- in the epilogue (per-channel) or once
-// per 64-k sub-block (group-wise) -- so code*scale is never rounded to T.
-// The epilogue passes each 16-row slab through LDS so that rows leave as
-// 16-byte stores.  Workgroups are numbered so that each XCD (one L2 each)
-// works on a compact block of neighbouring tiles.
+// gemm_dma_kernel is the kernel that runs whenever K is made of whole k tiles
+// (64 k for int8, 128 k for int4): a workgroup of WM x WN wavefronts computes a
+// BM x BN tile of the output from TM x TN blocks of v_mfma_f32_32x32x16 per
+// wavefront.  Both operands travel global -> LDS with direct-to-LDS loads,
+// two or three k tiles deep; the packed weights land as they lie in memory and
+// are dequantised in registers to exact signed bf16/fp16 integers on their way
+// into the B operand; scales are applied to fp32 accumulators -- in the
+// epilogue (per-channel) or once per group -- so code * scale is never rounded
+// to T.  For few rows K is cut into runs across workgroups whose fp32 partial
+// sums reduce_partials_kernel adds.  Workgroups are numbered so that each XCD
+// (one L2 each) works on a compact block of neighbouring tiles.
+//
+// gemm_kernel (v_mfma_f32_16x16x32, activations staged through registers into
+// padded LDS rows, weights loaded straight into B-fragment order) takes the
+// remaining K: those that end in a partial k tile.
 #include <atomic>
 
 #include "wol_common.h"
@@ -151,7 +153,7 @@ template <int DT, int BITS, bool GROUPED, int WM, int WN, int TM, int TN>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(
     const uint16_t* __restrict__ x, const uint8_t* __restrict__ codes,
     const uint16_t* __restrict__ bias, const uint16_t* __restrict__ scale, void* __restrict__ out,
-    int M, int K, int N, int gshift, int out_f32, int nbx, int nby) {
+    int M, int K, int N, int gshift, int out_f32, int nbx, int nby, int act) {
   constexpr int NT = 64 * WM * WN;
   constexpr int BM = WM * TM * 16, BN = WN * TN * 16;
   constexpr int TK = BITS == 8 ? 64 : 128;     // k per 16-byte lane load
@@ -307,7 +309,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int m = m0 + (wm * TM + a) * 16 + kb * 4 + r;
-          if (m < M) static_cast<float*>(out)[static_cast<int64_t>(m) * N + n] = tot[a][s][r] * sc[s] + bv[s];
+          if (m < M) static_cast<float*>(out)[static_cast<int64_t>(m) * N + n] = act_apply(tot[a][s][r] * sc[s] + bv[s], act);
         }
     }
     return;
@@ -322,7 +324,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(
     for (int s = 0; s < TN; ++s)
 #pragma unroll
       for (int r = 0; r < 4; ++r)
-        slab[(kb * 4 + r) * kSlabRow + s * 16 + j] = cast_out<DT>(tot[a][s][r] * sc[s] + bv[s]);
+        slab[(kb * 4 + r) * kSlabRow + s * 16 + j] = cast_out<DT>(act_apply(tot[a][s][r] * sc[s] + bv[s], act));
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int p = lane; p < kPieces; p += 64) {
@@ -381,6 +383,7 @@ struct DmaParams {
   int nbx, nby;                 // output tiles of the launch
   int nsplit, tiles_per_split;  // K is cut into nsplit runs of k tiles, one workgroup each
   int xcd_rows;                 // row groups of the XCD grid (tile_of_block), 0 = plain order
+  int act;                      // WOL_ACT_NONE or WOL_ACT_GELU, applied where the final sum is formed
 };
 
 // Fast path: K a multiple of the tile depth.
@@ -727,7 +730,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int m = m0 + (wm * TM + a) * 32 + 8 * (r / 4) + 4 * b + r % 4;
-          if (m < M && n < n_hi) outf[static_cast<int64_t>(m) * ld + (n - ncol0)] = tot[a][c][r] * sc[c] + bv[c];
+          if (m < M && n < n_hi) {
+            const float v = tot[a][c][r] * sc[c] + bv[c];  // a partial sum when K is cut into runs
+            outf[static_cast<int64_t>(m) * ld + (n - ncol0)] = p.nsplit > 1 ? v : act_apply(v, p.act);
+          }
         }
       }
     return;
@@ -744,7 +750,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
 #pragma unroll
       for (int r = 0; r < 16; ++r)
         slab[(8 * (r / 4) + 4 * b + r % 4) * kSlabRow + c * 32 + r32] =
-            cast_out<DT>(tot[a][c][r] * sc[c] + bv[c]);
+            cast_out<DT>(act_apply(tot[a][c][r] * sc[c] + bv[c], p.act));
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int q = lane; q < kPieces; q += 64) {
@@ -764,7 +770,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
 template <int DT>
 __global__ __launch_bounds__(256) void reduce_partials_kernel(
     const float* __restrict__ part, int nsplit, const uint16_t* __restrict__ bias,
-    void* __restrict__ out, int out_f32, int64_t total, int N, int col0, int ncols) {
+    void* __restrict__ out, int out_f32, int64_t total, int N, int col0, int ncols, int act) {
   const int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
   if (i >= total) return;
   const int64_t o = i / ncols * N + col0 + i % ncols;  // position in out
@@ -788,6 +794,8 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(
 #pragma unroll
     for (int e = 0; e < 4; ++e) s[e] += to_f32<DT>(bias[n + e]);
   }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) s[e] = act_apply(s[e], act);
   if (out_f32) {
     *reinterpret_cast<f32x4*>(static_cast<float*>(out) + o) = s;
   } else {
@@ -803,6 +811,7 @@ struct Args {
   int M, K, N, gshift, out_f32;
   void* ws; size_t ws_bytes;  // scratch for split-K partial sums, may be null
   hipStream_t stream;
+  int act;
 };
 
 // Raises a kernel's dynamic LDS limit once per device (the attribute belongs to
@@ -838,7 +847,7 @@ void launch_one(const Args& a) {
   kern<<<dim3(static_cast<unsigned>(nbx * nby)), dim3(64 * WM * WN), lds, a.stream>>>(
       static_cast<const uint16_t*>(a.x), static_cast<const uint8_t*>(a.codes),
       static_cast<const uint16_t*>(a.bias), static_cast<const uint16_t*>(a.scale), a.out, a.M, a.K,
-      a.N, a.gshift, a.out_f32, nbx, nby);
+      a.N, a.gshift, a.out_f32, nbx, nby, a.act);
 }
 
 // Row groups rg of the XCD grid for tile_of_block_2d: among the divisors of 8
@@ -892,12 +901,13 @@ void launch_dma(const Args& a, int strip_lo, int strip_hi, int nsplit) {
   p.tiles_per_split = (tiles + nsplit - 1) / nsplit;
   p.nsplit = (tiles + p.tiles_per_split - 1) / p.tiles_per_split;
   p.xcd_rows = plan_xcd_rows(p.nbx, p.nby, BM * 2, BN * BITS / 8);
+  p.act = a.act;
   kern<<<dim3(static_cast<unsigned>(p.nbx * p.nby * p.nsplit)), dim3(64 * WM * WN), lds, a.stream>>>(p);
   if (nsplit > 1) {
     const int64_t total = static_cast<int64_t>(a.M) * ncols;
     reduce_partials_kernel<DT><<<dim3(static_cast<unsigned>((total / 4 + 255) / 256)), dim3(256), 0, a.stream>>>(
         static_cast<const float*>(a.ws), p.nsplit, p.bias, a.out, a.out_f32, total, a.N,
-        strip_lo * kStripCols, ncols);
+        strip_lo * kStripCols, ncols, a.act);
   }
 }
 
@@ -1162,10 +1172,10 @@ void describe_linear_gemm(int64_t M, int64_t K, int64_t N, int bits, int group_s
 int launch_linear_gemm(const void* x, const void* codes, const void* bias, const void* scale,
                        int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
                        void* out, bool out_f32, void* workspace, size_t workspace_bytes,
-                       hipStream_t stream) {
+                       hipStream_t stream, const Fuse& f) {
   const int gshift = group_size == 64 ? 6 : (group_size == 128 ? 7 : -1);
   const Args a{x, codes, bias, scale, out, static_cast<int>(M), static_cast<int>(K),
-               static_cast<int>(N), gshift, out_f32 ? 1 : 0, workspace, workspace_bytes, stream};
+               static_cast<int>(N), gshift, out_f32 ? 1 : 0, workspace, workspace_bytes, stream, f.act};
   if (dtype == WOL_DTYPE_BF16) {
     if (bits == 8) launch_cfg<WOL_DTYPE_BF16, 8>(a); else launch_cfg<WOL_DTYPE_BF16, 4>(a);
   } else {

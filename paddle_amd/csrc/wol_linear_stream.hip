@@ -66,7 +66,12 @@ __device__ inline float sum_lane_groups(float v, bool x16, bool x32) {
 // TN strips (16 columns each) share one workgroup and with it every load of
 // the activations: the activation traffic out of L2, which grows with M, drops
 // by TN.
-template <int DT, int BITS, int MP, int MT, int WK, int NU, int TN, bool GROUPED>
+//
+// PRE: the activations are multiplied by a per-channel scale vector on their
+// way into the A operand, each product rounded to T as
+// apply_per_channel_scale rounds it (built for one row only; other row counts
+// get the scaled activations from a pass of that kernel).
+template <int DT, int BITS, int MP, int MT, int WK, int NU, int TN, bool GROUPED, bool PRE>
 struct StreamKernel {
   static_assert(MT == 1 || MP == 16, "several M tiles only with full 16-row operands");
   static constexpr int kS = 16 / MP;                  // k steps sharing one A operand
@@ -90,6 +95,8 @@ struct StreamKernel {
 
   const uint16_t* x;
   const uint16_t* scale;
+  const uint16_t* pre;  // [K] per-channel scales of the activations (PRE)
+  int act;              // WOL_ACT_NONE or WOL_ACT_GELU
   int M, K, N;
   int gshift;  // log2(group_size) when GROUPED
   int vsteps;  // k steps that lie in whole 16-byte weight tiles (all but an int4 half tile)
@@ -105,6 +112,7 @@ struct StreamKernel {
   struct Unit {
     u32x4 wv[TN][kNT];
     u32x4 av[kNA][MT];
+    u32x4 pv[PRE ? kNA : 1];  // the activation scales of the same k as av
     uint16_t sraw[TN][kNS];
   };
 
@@ -126,6 +134,14 @@ struct StreamKernel {
     return *reinterpret_cast<const u32x4*>(x + static_cast<int64_t>(m) * K + step * 32 + 8 * kb);
   }
 
+  // The activation scales that go with load_a(., step0, spread, tail): the same
+  // k for every row.
+  __device__ inline u32x4 load_pre(int step0, bool spread, bool tail = false) const {
+    int step = step0 + (spread ? j / MP : 0);
+    if (tail) step = step < vsteps ? step : vsteps - 1;
+    return *reinterpret_cast<const u32x4*>(pre + step * 32 + 8 * kb);
+  }
+
   __device__ inline uint16_t load_scale_raw(int step, int t) const {
     const uint16_t* row = scale + static_cast<int64_t>((step * 32) >> gshift) * N;
     return row[n[t]];
@@ -145,6 +161,10 @@ struct StreamKernel {
     for (int a = 0; a < kNA; ++a)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) d.av[a][mt] = load_a(mt, step0 + a * kS, true, tail);
+    if (PRE) {
+#pragma unroll
+      for (int a = 0; a < kNA; ++a) d.pv[a] = load_pre(step0 + a * kS, true, tail);
+    }
     if (GROUPED) {
       const int mine = MP == 8 ? (kb >> 1) : kb;
 #pragma unroll
@@ -197,10 +217,14 @@ struct StreamKernel {
 
   __device__ inline void compute_unit(const Unit& d) {
     f32x4 cc[kNA][MT];
+    u32x4 av[kNA][MT];
 #pragma unroll
     for (int a = 0; a < kNA; ++a)
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) cc[a][mt] = cancel_term(d.av[a][mt]);
+      for (int mt = 0; mt < MT; ++mt) {
+        av[a][mt] = PRE ? prescale_frag<DT>(d.av[a][mt], d.pv[a]) : d.av[a][mt];
+        cc[a][mt] = cancel_term(av[a][mt]);
+      }
 #pragma unroll
     for (int s = 0; s < kU; ++s)
 #pragma unroll
@@ -208,7 +232,7 @@ struct StreamKernel {
         const u32x4 v = d.wv[t][s / kSPT];
         const uint32_t w[4] = {v.x, v.y, v.z, v.w};
         const float sc = GROUPED ? to_f32<DT>(d.sraw[t][scale_slot(s)]) : 1.0f;
-        step_mfma(w + (s % kSPT) * kDw, d.av[s / kS], cc[s / kS], s % kS, sc, t);
+        step_mfma(w + (s % kSPT) * kDw, av[s / kS], cc[s / kS], s % kS, sc, t);
       }
   }
 
@@ -289,6 +313,7 @@ struct StreamKernel {
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
               a[st][mt] = load_a(mt, step + st, false);
+              if (PRE) a[st][mt] = prescale_frag<DT>(a[st][mt], load_pre(step + st, false));
               cc[st][mt] = cancel_term(a[st][mt]);
             }
 #pragma unroll
@@ -359,7 +384,7 @@ struct StreamKernel {
 #pragma unroll
         for (int w = 0; w < WK; ++w)
           s += red[(((t * WK + w) * MT + mt) * 4 + (row % 4)) * 64 + (row / 4) * 16 + nl];
-        s = s * ep_scale + ep_bias;
+        s = act_apply(s * ep_scale + ep_bias, act);
         const int64_t o = static_cast<int64_t>(m) * N + n[t];
         if (out_f32)
           static_cast<float*>(out)[o] = s;
@@ -370,15 +395,17 @@ struct StreamKernel {
   }
 };
 
-template <int DT, int BITS, int MP, int MT, int WK, int NU, int TN, bool GROUPED>
+template <int DT, int BITS, int MP, int MT, int WK, int NU, int TN, bool GROUPED, bool PRE>
 __global__ __launch_bounds__(WK * 64) void stream_kernel(
     const uint16_t* __restrict__ x, const uint8_t* __restrict__ codes,
     const uint16_t* __restrict__ bias, const uint16_t* __restrict__ scale, void* __restrict__ out,
-    int M, int K, int N, int gshift, int out_f32) {
+    int M, int K, int N, int gshift, int out_f32, const uint16_t* __restrict__ pre, int act) {
   extern __shared__ float red[];
-  StreamKernel<DT, BITS, MP, MT, WK, NU, TN, GROUPED> k;
+  StreamKernel<DT, BITS, MP, MT, WK, NU, TN, GROUPED, PRE> k;
   k.x = x;
   k.scale = scale;
+  k.pre = pre;
+  k.act = act;
   k.M = M;
   k.K = K;
   k.N = N;
@@ -389,6 +416,7 @@ __global__ __launch_bounds__(WK * 64) void stream_kernel(
 struct Args {
   const void* x; const void* codes; const void* bias; const void* scale; void* out;
   int M, K, N, gshift, out_f32, tn; hipStream_t stream;
+  const void* pre; int act;
 };
 
 template <int DT, int BITS, int MP, int MT, int WK, int NU, int TN>
@@ -399,12 +427,24 @@ void launch_tn(const Args& a) {
   const uint8_t* codes = static_cast<const uint8_t*>(a.codes);
   const uint16_t* bias = static_cast<const uint16_t*>(a.bias);
   const uint16_t* scale = static_cast<const uint16_t*>(a.scale);
+  const uint16_t* pre = static_cast<const uint16_t*>(a.pre);
+  if constexpr (MP == 1) {  // the fused activation scales exist for one row
+    if (pre != nullptr) {
+      if (a.gshift >= 0)
+        stream_kernel<DT, BITS, MP, MT, WK, NU, TN, true, true><<<grid, block, lds, a.stream>>>(
+            x, codes, bias, scale, a.out, a.M, a.K, a.N, a.gshift, a.out_f32, pre, a.act);
+      else
+        stream_kernel<DT, BITS, MP, MT, WK, NU, TN, false, true><<<grid, block, lds, a.stream>>>(
+            x, codes, bias, scale, a.out, a.M, a.K, a.N, a.gshift, a.out_f32, pre, a.act);
+      return;
+    }
+  }
   if (a.gshift >= 0)
-    stream_kernel<DT, BITS, MP, MT, WK, NU, TN, true><<<grid, block, lds, a.stream>>>(
-        x, codes, bias, scale, a.out, a.M, a.K, a.N, a.gshift, a.out_f32);
+    stream_kernel<DT, BITS, MP, MT, WK, NU, TN, true, false><<<grid, block, lds, a.stream>>>(
+        x, codes, bias, scale, a.out, a.M, a.K, a.N, a.gshift, a.out_f32, nullptr, a.act);
   else
-    stream_kernel<DT, BITS, MP, MT, WK, NU, TN, false><<<grid, block, lds, a.stream>>>(
-        x, codes, bias, scale, a.out, a.M, a.K, a.N, a.gshift, a.out_f32);
+    stream_kernel<DT, BITS, MP, MT, WK, NU, TN, false, false><<<grid, block, lds, a.stream>>>(
+        x, codes, bias, scale, a.out, a.M, a.K, a.N, a.gshift, a.out_f32, nullptr, a.act);
 }
 
 // Two strips per workgroup exist for the operand shapes whose activation
@@ -516,14 +556,16 @@ void describe_linear_stream(int64_t M, int64_t K, int64_t N, int bits, int group
   (void)group_size;
 }
 
+// f.pre_scale is honoured for one row only (the caller scales the activations
+// itself otherwise); f.act may be none or gelu.
 int launch_linear_stream(const void* x, const void* codes, const void* bias, const void* scale,
                          int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
-                         void* out, bool out_f32, hipStream_t stream) {
+                         void* out, bool out_f32, hipStream_t stream, const Fuse& f) {
   const int gshift = group_size == 64 ? 6 : (group_size == 128 ? 7 : -1);
   int wk = 1, nu = 0, tn = 1;
   pick_split(M, K, N, bits, &wk, &nu, &tn);
   const Args a{x, codes, bias, scale, out, static_cast<int>(M), static_cast<int>(K),
-               static_cast<int>(N), gshift, out_f32 ? 1 : 0, tn, stream};
+               static_cast<int>(N), gshift, out_f32 ? 1 : 0, tn, stream, M == 1 ? f.pre_scale : nullptr, f.act};
   if (dtype == WOL_DTYPE_BF16) {
     if (bits == 8) launch_m<WOL_DTYPE_BF16, 8>(a, wk, nu); else launch_m<WOL_DTYPE_BF16, 4>(a, wk, nu);
   } else {

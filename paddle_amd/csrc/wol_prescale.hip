@@ -16,6 +16,7 @@ constexpr int kRowsPerBlock = 8;  // rows a thread walks with its scales in regi
 
 template <int DT>
 __device__ inline uint32_t mul_pair(uint32_t x2, float s_lo, float s_hi) {
+  // the same arithmetic as prescale_pair (wol_common.h), with the scales already widened
   const float lo = to_f32<DT>(static_cast<uint16_t>(x2 & 0xFFFFu)) * s_lo;
   const float hi = to_f32<DT>(static_cast<uint16_t>(x2 >> 16)) * s_hi;
   return static_cast<uint32_t>(cast_out<DT>(lo)) | (static_cast<uint32_t>(cast_out<DT>(hi)) << 16);
@@ -89,7 +90,36 @@ int launch(const void* x, const void* scales, int64_t rows, int64_t cols, void* 
   return hipGetLastError() == hipSuccess ? WOL_OK : WOL_ERR_HIP;
 }
 
+// swiglu of fp32 sums: out[m, n] = T(silu(in[m, n]) * in[m, n + H]), H = N / 2,
+// four columns per thread (H is a multiple of 16).
+template <int DT>
+__global__ __launch_bounds__(kThreads) void swiglu_f32_kernel(const float* __restrict__ in, int64_t M, int64_t N,
+                                                              uint16_t* __restrict__ out) {
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+  const int64_t H = N / 2;
+  const int64_t i = (static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x) * 4;
+  if (i >= M * H) return;
+  const int64_t m = i / H, n = i % H;
+  const f32x4 g = *reinterpret_cast<const f32x4*>(in + m * N + n);
+  const f32x4 u = *reinterpret_cast<const f32x4*>(in + m * N + H + n);
+  u32x2 o;
+  o.x = cast_out<DT>(act_swiglu(g[0], u[0])) | (static_cast<uint32_t>(cast_out<DT>(act_swiglu(g[1], u[1]))) << 16);
+  o.y = cast_out<DT>(act_swiglu(g[2], u[2])) | (static_cast<uint32_t>(cast_out<DT>(act_swiglu(g[3], u[3]))) << 16);
+  *reinterpret_cast<u32x2*>(out + m * H + n) = o;
+}
+
 }  // namespace
+
+int launch_swiglu_f32(const float* in, int dtype, int64_t M, int64_t N, void* out, hipStream_t stream) {
+  const int64_t quads = M * (N / 2) / 4;
+  const dim3 grid(static_cast<unsigned>((quads + kThreads - 1) / kThreads));
+  if (dtype == WOL_DTYPE_BF16)
+    swiglu_f32_kernel<WOL_DTYPE_BF16><<<grid, kThreads, 0, stream>>>(in, M, N, static_cast<uint16_t*>(out));
+  else
+    swiglu_f32_kernel<WOL_DTYPE_F16><<<grid, kThreads, 0, stream>>>(in, M, N, static_cast<uint16_t*>(out));
+  return hipGetLastError() == hipSuccess ? WOL_OK : WOL_ERR_HIP;
+}
 
 int launch_prescale(const void* x, const void* scales, int dtype, int64_t rows, int64_t cols,
                     void* out, hipStream_t stream) {

@@ -5,8 +5,9 @@ from .quantized_linear import (  # noqa: F401
     llm_int8_linear,
     weight_dequantize,
     weight_only_linear,
+    weight_only_linear_fused,
     weight_quantize,
 )
 
 __all__ = ["weight_only_linear", "weight_quantize", "weight_dequantize", "apply_per_channel_scale",
-           "llm_int8_linear"]
+           "llm_int8_linear", "weight_only_linear_fused"]

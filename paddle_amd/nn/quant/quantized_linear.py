@@ -376,6 +376,67 @@ def weight_only_linear(x, weight, bias=None, weight_scale=None, weight_dtype="in
                         group_size, None)
 
 
+_ACTS = {None: 0, "none": 0, "None": 0, "gelu": 1, "swiglu": 2}
+
+
+def weight_only_linear_fused(x, weight, bias=None, weight_scale=None, weight_dtype="int8", group_size=-1,
+                             pre_scale=None, act="none"):
+    """weight_only_linear with its neighbours folded in: apply_per_channel_scale
+    in front (pre_scale: [K] in x's dtype, each product rounded to x's dtype as
+    that op rounds it) and an activation behind, applied to the fp32 sums before
+    the one rounding: act "none", "gelu" (the tanh form of the reference's GEMV
+    epilogue, act_method in paddle/phi/kernels/funcs/weight_only_gemv.h:33) or
+    "swiglu" (silu of the first half of the output columns times the second
+    half: the result has N/2 columns).  No counterpart in the reference's Python
+    API, which composes these from separate ops."""
+    assert (
+        group_size == -1 or group_size == 64 or group_size == 128
+    ), f"Currently weight_quantize only support group size of -1, 64 or 128. but got {group_size} "
+    if act not in _ACTS:
+        raise ValueError("(InvalidArgument) act must be 'none', 'gelu' or 'swiglu', but got %r" % (act,))
+    if weight_scale is None:
+        raise ValueError("(InvalidArgument) weight_scale is required")
+    out_shape, N = weight_only_linear_infer_meta(
+        tuple(x.shape), tuple(weight.shape), None if bias is None else tuple(bias.shape),
+        tuple(weight_scale.shape), weight_dtype, group_size,
+    )
+    dt = _dtype_id(x, "x")
+    _require_gpu(x, "x")
+    if weight.dtype != torch.int8:
+        raise ValueError("(InvalidArgument) weight must be int8, but got %s" % weight.dtype)
+    if weight_scale.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
+        raise ValueError("(InvalidArgument) weight_scale and bias must have x's dtype")
+    bits = 8 if weight_dtype == "int8" else 4
+    K = int(weight.shape[1])
+    if pre_scale is not None and (pre_scale.dtype != x.dtype or tuple(pre_scale.shape) != (K,)):
+        raise ValueError("(InvalidArgument) pre_scale must be [%d] in x's dtype" % K)
+    a = _ACTS[act]
+    if a == 2:
+        if N % 32 != 0:
+            raise ValueError("(InvalidArgument) swiglu needs an even number of 16-column strips")
+        out_shape = tuple(out_shape[:-1]) + (N // 2,)
+    x = x.contiguous()
+    weight = weight.contiguous()
+    weight_scale = weight_scale.contiguous()
+    bias = None if bias is None else bias.contiguous()
+    pre_scale = None if pre_scale is None else pre_scale.contiguous()
+    M = x.numel() // K
+    out = torch.empty(out_shape, dtype=x.dtype, device=x.device)
+    if M == 0:
+        return out
+    ws_bytes = _lib.lib.wol_linear_fused_workspace(M, K, N, bits, group_size, 0 if pre_scale is None else 1, a)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
+    with torch.cuda.device(x.device):
+        _lib.check(
+            _lib.lib.wol_linear_fused(
+                x.data_ptr(), None if pre_scale is None else pre_scale.data_ptr(), weight.data_ptr(),
+                None if bias is None else bias.data_ptr(), weight_scale.data_ptr(), dt, M, K, N, bits,
+                group_size, a, out.data_ptr(), None if ws is None else ws.data_ptr(), ws_bytes, _stream_ptr(x),
+            )
+        )
+    return out
+
+
 def weight_only_linear_fp32(x, weight, bias=None, weight_scale=None, weight_dtype="int8",
                             group_size=-1):
     """weight_only_linear without the final cast: returns the fp32 accumulators

@@ -1,0 +1,158 @@
+"""weight_only_linear with apply_per_channel_scale folded in front and an
+activation (gelu, swiglu) behind: wol_linear_fused against the oracle's
+composition of the three (apply_per_channel_scale -> linear -> activation on
+the fp32 sums), through the C ABI; and the pins of the oracle's activation
+formulas (no GPU)."""
+import numpy as np
+import pytest
+
+import helpers as H
+
+TOL = 1e-3
+
+
+# ---- the oracle's formulas, pinned without a GPU ---------------------------
+def test_oracle_gelu_against_numpy_float64(oracle):
+    # the tanh form of the reference's GEMV epilogue
+    # (paddle/phi/kernels/funcs/weight_only_gemv.cu:147-157), evaluated by numpy
+    # in float64 and rounded once to float32; known values and both tails
+    rng = np.random.default_rng(3)
+    v = np.concatenate([rng.standard_normal(4000) * 3, [0.0, -0.0, 1.0, -1.0, 40.0, -40.0, 1e-8, 88.0, -88.0]])
+    v = v.astype(np.float32).reshape(1, -1)
+    o32, oT = oracle.activation(v, oracle.ACT_GELU, H.F16)
+    x = v.astype(np.float64)
+    want = (x * 0.5 * (1.0 + np.tanh(0.7978845608028654 * (x + 0.044715 * x ** 3)))).astype(np.float32)
+    # 1 + tanh cancels in the far negative tail, where libm's and numpy's tanh
+    # may differ in the last place: identical bits elsewhere, absolute there
+    assert np.allclose(o32, want, rtol=1e-6, atol=1e-9)
+    assert np.array_equal(o32[np.abs(v) < 4], want[np.abs(v) < 4])
+    assert np.array_equal(oT, H.f32_to_bits(o32, H.F16))
+    # known answers: gelu(0) = 0, gelu(x) -> x for large x, -> -0 for very negative x, gelu(1) = 0.8411919906...
+    i = 4000
+    assert o32[0, i] == 0.0 and o32[0, i + 4] == 40.0 and o32[0, i + 5] == 0.0
+    assert abs(float(o32[0, i + 2]) - 0.8411919906082768) < 1e-7
+    # act 0 is the identity
+    n32, _ = oracle.activation(v, oracle.ACT_NONE, H.BF16)
+    assert np.array_equal(n32, v)
+
+
+def test_oracle_swiglu_against_numpy_float64(oracle):
+    # silu(first half) * second half (paddle/phi/kernels/gpu/swiglu_kernel.cu:32-52)
+    rng = np.random.default_rng(4)
+    v = (rng.standard_normal((7, 64)) * 4).astype(np.float32)
+    v[0, :4] = [0.0, 30.0, -30.0, 1.0]
+    v[0, 32:36] = [5.0, 2.0, 2.0, 3.0]
+    o32, oT = oracle.activation(v, oracle.ACT_SWIGLU, H.BF16)
+    g, u = v[:, :32].astype(np.float64), v[:, 32:].astype(np.float64)
+    want = (g / (1.0 + np.exp(-g)) * u).astype(np.float32)
+    assert o32.shape == (7, 32) and np.array_equal(o32, want)
+    assert np.array_equal(oT, H.f32_to_bits(want, H.BF16))
+    assert o32[0, 0] == 0.0 and abs(o32[0, 1] - 60.0) < 1e-5 and abs(o32[0, 2]) < 1e-10
+    assert abs(float(o32[0, 3]) - 3 * 0.7310585786300049) < 1e-6
+
+
+# ---- the fused entry point ----------------------------------------------------
+def _fused(x_bits, pre_bits, packed, bias_bits, scale_bits, dt, N, bits, g, act):
+    import torch
+    from paddle_amd import _lib
+
+    dev = "cuda:0"
+    x = H.bits_to_torch(x_bits, dt, dev)
+    M, K = x.shape
+    c = torch.from_numpy(np.ascontiguousarray(packed)).to(dev)
+    s = H.bits_to_torch(scale_bits, dt, dev)
+    b = None if bias_bits is None else H.bits_to_torch(bias_bits, dt, dev)
+    ps = None if pre_bits is None else H.bits_to_torch(pre_bits, dt, dev)
+    No = N // 2 if act == 2 else N
+    out = torch.full((M, No), float("nan"), dtype=x.dtype, device=dev)
+    wsb = _lib.lib.wol_linear_fused_workspace(M, K, N, bits, g, 0 if ps is None else 1, act)
+    ws = torch.full((max(wsb, 16),), 0x5A, dtype=torch.uint8, device=dev)
+    _lib.check(_lib.lib.wol_linear_fused(x.data_ptr(), None if ps is None else ps.data_ptr(), c.data_ptr(),
+                                         None if b is None else b.data_ptr(), s.data_ptr(), dt, M, K, N, bits, g, act,
+                                         out.data_ptr(), ws.data_ptr() if wsb else None, wsb, None))
+    torch.cuda.synchronize()
+    return H.torch_to_bits(out)
+
+
+# rows x (K, N): one row (streaming kernel), a small batch on a K and N the
+# batched decode kernel takes, and row counts / shapes that go to the streaming
+# kernel with several rows and to the GEMM
+SHAPES = [(1, 512, 256), (1, 4096, 1024), (8, 2048, 8192), (5, 4096, 8704), (3, 512, 256), (40, 1024, 512),
+          (100, 512, 1024)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("g", [-1, 64, 128])
+def test_fused_against_oracle(device, oracle, dt, bits, g):
+    rng = np.random.default_rng(11)
+    for M, K, N in SHAPES:
+        wb = H.make_weight(K, N, dt, seed=K + N)
+        xb = H.make_act(M, K, dt, seed=M)
+        bb = H.make_bias(N, dt, seed=5)
+        pre = H.f32_to_bits((0.5 + rng.random(K, dtype=np.float32)).astype(np.float32), dt)
+        oc, osc = oracle.weight_quantize(wb, dt, bits, g)
+        packed = H.gfx950_from_q(H.q_from_canonical(oc, bits), bits)
+        for act in (0, 1, 2):
+            for use_pre in (False, True):
+                for bias in (None, bb):
+                    if act == 0 and not use_pre:
+                        continue  # plain wol_linear, covered elsewhere
+                    print("case", dt, bits, g, M, K, N, act, use_pre, bias is not None, flush=True)
+                    _, wantT = oracle.linear_fused(xb, pre if use_pre else None, oc, osc, bias, dt, bits, g, act)
+                    got = _fused(xb, pre if use_pre else None, packed, bias, osc, dt, N, bits, g, act)
+                    err = H.rel_l2(H.bits_to_f32(got, dt), H.bits_to_f32(wantT, dt))
+                    assert err <= TOL, (err, dt, bits, g, M, K, N, act, use_pre)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+def test_fused_pre_scale_equals_the_two_ops(device, oracle, dt):
+    # folding apply_per_channel_scale into the linear must not change a bit:
+    # the same products, rounded the same way, enter the same kernel
+    import gpu_calls as G
+    import torch
+    from paddle_amd import _lib
+
+    rng = np.random.default_rng(12)
+    for M, K, N, bits, g in ((1, 4096, 512, 4, 128), (8, 4096, 8192, 4, -1), (16, 2048, 8192, 8, 64), (6, 512, 256, 8, -1),
+                             (200, 1024, 512, 8, -1)):
+        wb = H.make_weight(K, N, dt, seed=K + N)
+        xb = H.make_act(M, K, dt, seed=M)
+        pre = H.f32_to_bits((0.25 + 2 * rng.random(K, dtype=np.float32)).astype(np.float32), dt)
+        oc, osc = oracle.weight_quantize(wb, dt, bits, g)
+        packed = H.gfx950_from_q(H.q_from_canonical(oc, bits), bits)
+        fused = _fused(xb, pre, packed, None, osc, dt, N, bits, g, 0)
+        x = H.bits_to_torch(xb, dt, "cuda:0")
+        ps = H.bits_to_torch(pre, dt, "cuda:0")
+        xs = torch.empty_like(x)
+        _lib.check(_lib.lib.wol_apply_per_channel_scale(x.data_ptr(), ps.data_ptr(), dt, M, K, xs.data_ptr(), None))
+        torch.cuda.synchronize()
+        assert np.array_equal(H.torch_to_bits(xs), oracle.apply_per_channel_scale(xb, pre, dt))
+        two = G.linear(H.torch_to_bits(xs), packed, None, osc, dt, N, bits, g)
+        assert np.array_equal(fused, two), (M, K, N, bits, g)
+
+
+@pytest.mark.gpu
+def test_fused_python_wrapper_and_errors(device):
+    import torch
+    from paddle_amd.nn import quant as Q
+
+    w = (torch.randn(512, 256, device="cuda") * 0.02).half()
+    codes, scale = Q.weight_quantize(w, algo="weight_only_int4", group_size=64)
+    x = torch.randn(2, 3, 512, device="cuda").half()
+    ps = (torch.rand(512, device="cuda") + 0.5).half()
+    out = Q.weight_only_linear_fused(x, codes, None, scale, "int4", 64, pre_scale=ps, act="swiglu")
+    assert list(out.shape) == [2, 3, 128] and out.dtype == torch.float16
+    lin = Q.weight_only_linear(Q.apply_per_channel_scale(x.reshape(-1, 512), ps), codes, None, scale, "int4", None, 64)
+    ref = torch.nn.functional.silu(lin[:, :128].float()) * lin[:, 128:].float()
+    assert torch.allclose(out.reshape(-1, 128).float(), ref, rtol=2e-2, atol=2e-3)
+    gel = Q.weight_only_linear_fused(x, codes, None, scale, "int4", 64, act="gelu")
+    lin2 = Q.weight_only_linear(x, codes, None, scale, "int4", None, 64)
+    assert torch.allclose(gel.float(), torch.nn.functional.gelu(lin2.float(), approximate="tanh"), rtol=2e-2, atol=2e-3)
+    with pytest.raises(ValueError):
+        Q.weight_only_linear_fused(x, codes, None, scale, "int4", 64, act="relu")
+    with pytest.raises(ValueError):
+        Q.weight_only_linear_fused(x, codes, None, scale, "int4", 64, pre_scale=ps[:100])
+    assert list(Q.weight_only_linear_fused(x[:0], codes, None, scale, "int4", 64, act="swiglu").shape) == [0, 3, 128]
