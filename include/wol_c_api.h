@@ -214,6 +214,40 @@ int wol_linear_fused(const void* x, const void* pre_scale, const void* codes,
                      void* out, void* workspace, size_t workspace_bytes,
                      void* stream);
 
+/*
+ * Replaces MoeFFNKernel<T, GPUContext> for quant_method "weight_only_int8" /
+ * "weight_only_int4" (paddle/phi/kernels/fusion/cutlass/moe_ffn.cu:36-183,
+ * whose CUTLASS grouped GEMMs :74-154 have no ROCm build): the expert FFN of a
+ * mixture-of-experts layer on tokens already permuted into expert order,
+ *   fc1  = permute_input . dequant(ffn1_weight[e]) + ffn1_bias[e]     [rows, inter]  T
+ *   act  = T( silu(fc1[:, :inter/2]) * fc1[:, inter/2:] )            [rows, inter/2] (swiglu, :133-139)
+ *   out  = act . dequant(ffn2_weight[e])                              [rows, hidden] T
+ * where e is the expert of the row.  token_nums_per_expert: [num_experts]
+ * int64 on the device, holding what the reference's moe_dispatch writes there
+ * -- the running total of rows up to and including each expert
+ * (fusion/cutlass/moe_dispatch.cu:174-182, moe/fused_moe_op.h:896-908), so
+ * expert e owns rows [t[e-1], t[e]) and t[num_experts-1] <= rows.  It is read
+ * on the device only: nothing returns to the host.
+ * Weights: num_experts consecutive tensors as wol_quantize writes them
+ * (GFX950 layout, per-channel scales): ffn1_weight [E] x (K = hidden,
+ * N = inter), ffn1_scale [E, inter] T, ffn1_bias [E, inter] T or NULL,
+ * ffn2_weight [E] x (K = inter/2, N = hidden), ffn2_scale [E, hidden] T.
+ * Each of the two products is ONE grouped launch (128 x 256 tiles looked up
+ * in a row-tile table that a one-workgroup kernel derives from
+ * token_nums_per_expert); the swiglu between them is an element-wise pass.
+ * Requires hidden % 128 == 0, inter % 256 == 0, num_experts <= 1024; the
+ * workspace (wol_moe_ffn_workspace bytes, 16-byte aligned) holds the table and
+ * the two intermediate tensors.
+ */
+size_t wol_moe_ffn_workspace(int64_t rows, int64_t hidden, int64_t inter,
+                             int num_experts);
+int wol_moe_ffn(const void* permute_input, const int64_t* token_nums_per_expert,
+                const void* ffn1_weight, const void* ffn1_bias,
+                const void* ffn1_scale, const void* ffn2_weight,
+                const void* ffn2_scale, int dtype, int64_t rows, int64_t hidden,
+                int64_t inter, int num_experts, int bits, void* ffn_out,
+                void* workspace, size_t workspace_bytes, void* stream);
+
 /* Kernel choice of wol_linear_on. */
 enum wol_kernel {
   WOL_KERNEL_AUTO = 0,   /* what wol_linear does                                */

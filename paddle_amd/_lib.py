@@ -29,6 +29,8 @@ SYMBOLS = (
     "wol_linear_on",
     "wol_linear_fused_workspace",
     "wol_linear_fused",
+    "wol_moe_ffn_workspace",
+    "wol_moe_ffn",
     "wol_repack",
     "wol_code_offset",
     "wol_apply_per_channel_scale",
@@ -81,6 +83,10 @@ def _load():
     lib.wol_linear_fused_workspace.restype = sz
     lib.wol_linear_fused.argtypes = [vp, vp, vp, vp, vp, ci, i64, i64, i64, ci, ci, ci, vp, vp, sz, vp]
     lib.wol_linear_fused.restype = ci
+    lib.wol_moe_ffn_workspace.argtypes = [i64, i64, i64, ci]
+    lib.wol_moe_ffn_workspace.restype = sz
+    lib.wol_moe_ffn.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, i64, i64, i64, ci, ci, vp, vp, sz, vp]
+    lib.wol_moe_ffn.restype = ci
     lib.wol_repack.argtypes = [vp, ci, vp, ci, i64, i64, ci, vp]
     lib.wol_repack.restype = ci
     lib.wol_code_offset.argtypes = [ci, i64, i64, ci, i64, i64, ctypes.POINTER(ci)]

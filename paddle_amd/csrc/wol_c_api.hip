@@ -343,6 +343,46 @@ int wol_linear_fused(const void* x, const void* pre_scale, const void* codes, co
   return wol::launch_swiglu_f32(sums, dtype, M, N, out, s);
 }
 
+namespace {
+int check_moe(int64_t rows, int64_t hidden, int64_t inter, int num_experts) {
+  if (rows < 0 || rows > (int64_t{1} << 24) || hidden <= 0 || inter <= 0) return WOL_ERR_BAD_SHAPE;
+  if (hidden % 128 != 0 || inter % 256 != 0 || hidden > (int64_t{1} << 24) || inter > (int64_t{1} << 24))
+    return WOL_ERR_BAD_SHAPE;
+  if (hidden < 256 || inter < 512) return WOL_ERR_BAD_SHAPE;  // at least two k tiles in both products
+  if (num_experts <= 0 || num_experts > 1024) return WOL_ERR_BAD_SHAPE;
+  return WOL_OK;
+}
+}  // namespace
+
+size_t wol_moe_ffn_workspace(int64_t rows, int64_t hidden, int64_t inter, int num_experts) {
+  if (check_moe(rows, hidden, inter, num_experts) != WOL_OK || rows == 0) return 0;
+  return wol::moe_ffn_workspace(rows, inter, num_experts);
+}
+
+int wol_moe_ffn(const void* permute_input, const int64_t* token_nums_per_expert, const void* ffn1_weight,
+                const void* ffn1_bias, const void* ffn1_scale, const void* ffn2_weight, const void* ffn2_scale,
+                int dtype, int64_t rows, int64_t hidden, int64_t inter, int num_experts, int bits, void* ffn_out,
+                void* workspace, size_t workspace_bytes, void* stream) {
+  if (dtype != WOL_DTYPE_F16 && dtype != WOL_DTYPE_BF16) return WOL_ERR_BAD_DTYPE;
+  if (bits != 8 && bits != 4) return WOL_ERR_BAD_BITS;
+  const int rc = check_moe(rows, hidden, inter, num_experts);
+  if (rc != WOL_OK) return rc;
+  if (rows == 0) return WOL_OK;
+  if (permute_input == nullptr || token_nums_per_expert == nullptr || ffn1_weight == nullptr ||
+      ffn1_scale == nullptr || ffn2_weight == nullptr || ffn2_scale == nullptr || ffn_out == nullptr)
+    return WOL_ERR_NULL_POINTER;
+  if (!aligned16(permute_input) || !aligned16(ffn1_weight) || !aligned16(ffn2_weight) || !aligned16(ffn1_scale) ||
+      !aligned16(ffn2_scale) || !aligned16(ffn_out))
+    return WOL_ERR_ALIGNMENT;
+  if (workspace == nullptr || workspace_bytes < wol::moe_ffn_workspace(rows, inter, num_experts))
+    return WOL_ERR_WORKSPACE;
+  if (!aligned16(workspace)) return WOL_ERR_ALIGNMENT;
+  if (const int dv = require_gfx950(); dv != WOL_OK) return dv;
+  return wol::launch_moe_ffn(permute_input, token_nums_per_expert, ffn1_weight, ffn1_bias, ffn1_scale, ffn2_weight,
+                             ffn2_scale, dtype, rows, hidden, inter, num_experts, bits, ffn_out, workspace,
+                             static_cast<hipStream_t>(stream));
+}
+
 int wol_linear_on(const void* x, const void* codes, const void* bias, const void* scale, int dtype,
                   int64_t M, int64_t K, int64_t N, int bits, int group_size, void* out,
                   int out_is_f32, int kernel, void* workspace, size_t workspace_bytes,

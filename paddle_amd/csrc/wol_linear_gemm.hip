@@ -384,6 +384,20 @@ struct DmaParams {
   int nsplit, tiles_per_split;  // K is cut into nsplit runs of k tiles, one workgroup each
   int xcd_rows;                 // row groups of the XCD grid (tile_of_block), 0 = plain order
   int act;                      // WOL_ACT_NONE or WOL_ACT_GELU, applied where the final sum is formed
+  // Grouped launch (mixture of experts): row tile `by` of the launch is entry
+  // `by` of this table -- {expert, first row, rows} -- written on the device by
+  // moe_plan_kernel; an expert's rows use that expert's weights, scales and
+  // bias (consecutive tensors, the strides below apart).  Null: one problem.
+  const int* moe_table;
+  int64_t moe_codes_stride;     // bytes between two experts' packed weights
+};
+
+// One entry of the row-tile table of a grouped launch.
+struct MoeTile {
+  int expert;  // -1: the tile is not used
+  int row0;    // first row of the tile in the permuted input
+  int rows;    // rows of the tile that exist (1 .. tile height)
+  int pad;
 };
 
 // Fast path: K a multiple of the tile depth.
@@ -451,7 +465,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
 
   const uint16_t* __restrict__ x = p.x;
   const uint16_t* __restrict__ scale = p.scale;
-  const int M = p.M, K = p.K, N = p.N;
+  const uint16_t* __restrict__ bias = p.bias;
+  const uint8_t* __restrict__ codes = p.codes;
+  void* outp = p.out;
+  int M = p.M;
+  const int K = p.K, N = p.N;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WN, wn = wave % WN;
@@ -460,7 +478,20 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   const int split = blockIdx.x / ntiles;
   int bx, by;
   tile_of_block_2d(blockIdx.x - split * ntiles, p.nbx, p.nby, p.xcd_rows, &bx, &by);
-  const int m0 = by * BM;
+  int m0 = by * BM;
+  if (p.moe_table != nullptr) {
+    // this row tile belongs to one expert: shift every base to that expert and
+    // to the tile's first row, and let M be the rows that exist
+    const MoeTile t = reinterpret_cast<const MoeTile*>(p.moe_table)[by];
+    if (t.expert < 0) return;
+    x += static_cast<int64_t>(t.row0) * K;
+    outp = static_cast<uint16_t*>(outp) + static_cast<int64_t>(t.row0) * N;
+    codes += static_cast<int64_t>(t.expert) * p.moe_codes_stride;
+    scale += static_cast<int64_t>(t.expert) * N;
+    if (bias != nullptr) bias += static_cast<int64_t>(t.expert) * N;
+    M = t.rows;
+    m0 = 0;
+  }
   const int strip_blk = p.strip_lo + bx * (BN / 16);
   const int nstrips = p.strip_hi;
   const int n_hi = p.strip_hi * kStripCols;
@@ -488,7 +519,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   for (int c = 0; c < kBLoads; ++c) {
     int st = strip_blk + c * NW + wave;
     st = st < nstrips ? st : nstrips - 1;  // past the last column: valid data, never stored
-    bsrc[c] = p.codes + static_cast<int64_t>(st) * strip_bytes(K, BITS) +
+    bsrc[c] = codes + static_cast<int64_t>(st) * strip_bytes(K, BITS) +
               static_cast<int64_t>(t0) * 1024 + lane * 16;
   }
   const int swz = a_swizzle<C>(lane & 15);  // fragment rows are 32*t + r32; the swizzle has period 16
@@ -706,7 +737,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
 #pragma unroll
   for (int c = 0; c < TN; ++c) {
     sc[c] = G == 0 ? to_f32<DT>(scale[ncol[c]]) : 1.0f;
-    bv[c] = (p.bias != nullptr && p.nsplit == 1) ? to_f32<DT>(p.bias[ncol[c]]) : 0.0f;
+    bv[c] = (bias != nullptr && p.nsplit == 1) ? to_f32<DT>(bias[ncol[c]]) : 0.0f;
   }
   if (OFFS && G == 0) {
 #pragma unroll
@@ -721,7 +752,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
     // partial sums are kept compact: row length = the columns of this launch
     const int64_t ld = p.nsplit > 1 ? static_cast<int64_t>(p.strip_hi - p.strip_lo) * kStripCols : N;
     const int ncol0 = p.nsplit > 1 ? p.strip_lo * kStripCols : 0;
-    float* outf = static_cast<float*>(p.out) + (p.nsplit > 1 ? static_cast<int64_t>(split) * M * ld : 0);
+    float* outf = static_cast<float*>(outp) + (p.nsplit > 1 ? static_cast<int64_t>(split) * M * ld : 0);
 #pragma unroll
     for (int a = 0; a < TM; ++a)
 #pragma unroll
@@ -738,7 +769,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
       }
     return;
   }
-  uint16_t* out = static_cast<uint16_t*>(p.out);
+  uint16_t* out = static_cast<uint16_t*>(outp);
   constexpr int kSlabRow = TN * 32 + 8;  // padded, in elements
   static_assert(NW * 32 * kSlabRow * 2 <= kStages * kStage, "slabs must fit in the stage buffers");
   uint16_t* slab = reinterpret_cast<uint16_t*>(smem) + wave * 32 * kSlabRow;
@@ -902,6 +933,8 @@ void launch_dma(const Args& a, int strip_lo, int strip_hi, int nsplit) {
   p.nsplit = (tiles + p.tiles_per_split - 1) / p.tiles_per_split;
   p.xcd_rows = plan_xcd_rows(p.nbx, p.nby, BM * 2, BN * BITS / 8);
   p.act = a.act;
+  p.moe_table = nullptr;
+  p.moe_codes_stride = 0;
   kern<<<dim3(static_cast<unsigned>(p.nbx * p.nby * p.nsplit)), dim3(64 * WM * WN), lds, a.stream>>>(p);
   if (nsplit > 1) {
     const int64_t total = static_cast<int64_t>(a.M) * ncols;
@@ -1103,6 +1136,72 @@ void launch_fast(const Args& a) {
 #undef WOL_HALF
 }
 
+// Row-tile table of a grouped launch with tiles of `bm` rows.  cum[e] is the
+// number of rows of experts 0 .. e (the inclusive running total that the
+// reference's moe_dispatch returns as token_nums_per_expert,
+// paddle/phi/kernels/fusion/cutlass/moe_dispatch.cu:174-182): expert e owns
+// rows cum[e-1] .. cum[e]-1 and ceil(rows / bm) tiles.  One workgroup; the
+// table has max_tiles entries, unused ones marked -1.
+__global__ __launch_bounds__(256) void moe_plan_kernel(const int64_t* __restrict__ cum, int num_experts, int bm,
+                                                       int max_tiles, MoeTile* __restrict__ table) {
+  __shared__ int first_tile[1025];  // exclusive running total of tiles, by expert
+  for (int i = threadIdx.x; i < max_tiles; i += 256) table[i] = MoeTile{-1, 0, 0, 0};
+  if (threadIdx.x == 0) {
+    int acc = 0;
+    int64_t prev = 0;
+    for (int e = 0; e < num_experts; ++e) {
+      first_tile[e] = acc;
+      const int64_t rows = cum[e] - prev;
+      prev = cum[e];
+      acc += static_cast<int>((rows + bm - 1) / bm);
+    }
+    first_tile[num_experts] = acc;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < num_experts; e += 256) {
+    const int64_t r0 = e > 0 ? cum[e - 1] : 0, r1 = cum[e];
+    const int t0 = first_tile[e], nt = first_tile[e + 1] - t0;
+    for (int t = 0; t < nt && t0 + t < max_tiles; ++t) {
+      const int64_t row = r0 + static_cast<int64_t>(t) * bm;
+      const int64_t left = r1 - row;
+      table[t0 + t] = MoeTile{e, static_cast<int>(row), static_cast<int>(left < bm ? left : bm), 0};
+    }
+  }
+}
+
+constexpr int kMoeTileRows = 128;
+
+// One grouped GEMM: every expert's rows against that expert's weights, 128 x
+// 256 tiles, per-channel scales, out [rows, N] T.
+template <int DT, int BITS>
+void launch_moe_gemm(const void* x, const int* table, int max_tiles, const void* codes, const void* bias,
+                     const void* scale, int64_t K, int64_t N, void* out, hipStream_t stream) {
+  constexpr bool kOffs = BITS == 4 && DT == WOL_DTYPE_BF16;  // as the ungrouped launch chooses
+  constexpr int WM = 2, WN = 4, TM = 2, TN = 2, BN = WN * TN * 32;
+  constexpr size_t lds = dma_lds_bytes<BITS, 0, WM, WN, TM, TN, 3>();
+  auto kern = gemm_dma_kernel<DT, BITS, 0, kOffs, WM, WN, TM, TN, 3>;
+  static std::atomic<uint32_t> configured{0};
+  allow_lds(reinterpret_cast<const void*>(kern), lds, configured);
+  DmaParams p;
+  p.x = static_cast<const uint16_t*>(x);
+  p.codes = static_cast<const uint8_t*>(codes);
+  p.bias = static_cast<const uint16_t*>(bias);
+  p.scale = static_cast<const uint16_t*>(scale);
+  p.out = out;
+  p.M = kMoeTileRows; p.K = static_cast<int>(K); p.N = static_cast<int>(N);
+  p.out_f32 = 0;
+  p.strip_lo = 0; p.strip_hi = static_cast<int>(N / kStripCols);
+  p.nbx = static_cast<int>((N + BN - 1) / BN);
+  p.nby = max_tiles;
+  p.nsplit = 1;
+  p.tiles_per_split = static_cast<int>(K / (BITS == 8 ? 64 : 128));
+  p.xcd_rows = 0;
+  p.act = WOL_ACT_NONE;
+  p.moe_table = table;
+  p.moe_codes_stride = K * N * BITS / 8;
+  kern<<<dim3(static_cast<unsigned>(p.nbx * p.nby)), dim3(64 * WM * WN), lds, stream>>>(p);
+}
+
 template <int DT, int BITS>
 void launch_cfg(const Args& a) {
   constexpr int TK = BITS == 8 ? 64 : 128;
@@ -1181,6 +1280,46 @@ int launch_linear_gemm(const void* x, const void* codes, const void* bias, const
   } else {
     if (bits == 8) launch_cfg<WOL_DTYPE_F16, 8>(a); else launch_cfg<WOL_DTYPE_F16, 4>(a);
   }
+  return check_launch();
+}
+
+// ---- mixture-of-experts FFN ---------------------------------------------------
+// Scratch: [row-tile table][fc1 output rows x inter T][activation rows x inter/2 T]
+static size_t moe_up(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
+
+int moe_max_tiles(int64_t rows, int num_experts) {
+  return static_cast<int>((rows + kMoeTileRows - 1) / kMoeTileRows) + num_experts;
+}
+
+size_t moe_ffn_workspace(int64_t rows, int64_t inter, int num_experts) {
+  return moe_up(static_cast<size_t>(moe_max_tiles(rows, num_experts)) * sizeof(MoeTile)) +
+         moe_up(static_cast<size_t>(rows) * inter * 2) + moe_up(static_cast<size_t>(rows) * (inter / 2) * 2);
+}
+
+int launch_moe_ffn(const void* x, const int64_t* rows_before_expert, const void* ffn1_codes,
+                   const void* ffn1_bias, const void* ffn1_scale, const void* ffn2_codes,
+                   const void* ffn2_scale, int dtype, int64_t rows, int64_t hidden, int64_t inter,
+                   int num_experts, int bits, void* out, void* workspace, hipStream_t stream) {
+  unsigned char* ws = static_cast<unsigned char*>(workspace);
+  const int max_tiles = moe_max_tiles(rows, num_experts);
+  MoeTile* table = reinterpret_cast<MoeTile*>(ws);
+  unsigned char* fc1 = ws + moe_up(static_cast<size_t>(max_tiles) * sizeof(MoeTile));
+  unsigned char* act = fc1 + moe_up(static_cast<size_t>(rows) * inter * 2);
+  moe_plan_kernel<<<dim3(1), dim3(256), 0, stream>>>(rows_before_expert, num_experts, kMoeTileRows, max_tiles, table);
+  const int* tb = reinterpret_cast<const int*>(table);
+#define WOL_MOE(DT, B)                                                                                        \
+  do {                                                                                                        \
+    launch_moe_gemm<DT, B>(x, tb, max_tiles, ffn1_codes, ffn1_bias, ffn1_scale, hidden, inter, fc1, stream);  \
+    const int rc = launch_swiglu_t(fc1, dtype, rows, inter, act, stream);                                     \
+    if (rc != WOL_OK) return rc;                                                                              \
+    launch_moe_gemm<DT, B>(act, tb, max_tiles, ffn2_codes, nullptr, ffn2_scale, inter / 2, hidden, out, stream); \
+  } while (0)
+  if (dtype == WOL_DTYPE_BF16) {
+    if (bits == 8) WOL_MOE(WOL_DTYPE_BF16, 8); else WOL_MOE(WOL_DTYPE_BF16, 4);
+  } else {
+    if (bits == 8) WOL_MOE(WOL_DTYPE_F16, 8); else WOL_MOE(WOL_DTYPE_F16, 4);
+  }
+#undef WOL_MOE
   return check_launch();
 }
 

@@ -109,7 +109,42 @@ __global__ __launch_bounds__(kThreads) void swiglu_f32_kernel(const float* __res
   *reinterpret_cast<u32x2*>(out + m * H + n) = o;
 }
 
+// swiglu of a T tensor: out[m, n] = T(silu(in[m, n]) * in[m, n + H]) computed in
+// float (paddle/phi/kernels/gpu/swiglu_kernel.cu:32-52), eight columns per thread.
+template <int DT>
+__global__ __launch_bounds__(kThreads) void swiglu_t_kernel(const uint16_t* __restrict__ in, int64_t M, int64_t N,
+                                                            uint16_t* __restrict__ out) {
+  const int64_t H = N / 2;
+  const int64_t i = (static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x) * 8;
+  if (i >= M * H) return;
+  const int64_t m = i / H, n = i % H;
+  const u32x4 g = *reinterpret_cast<const u32x4*>(in + m * N + n);
+  const u32x4 u = *reinterpret_cast<const u32x4*>(in + m * N + H + n);
+  const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
+  uint32_t ow[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const float lo = act_swiglu(to_f32<DT>(static_cast<uint16_t>(gw[q] & 0xFFFFu)), to_f32<DT>(static_cast<uint16_t>(uw[q] & 0xFFFFu)));
+    const float hi = act_swiglu(to_f32<DT>(static_cast<uint16_t>(gw[q] >> 16)), to_f32<DT>(static_cast<uint16_t>(uw[q] >> 16)));
+    ow[q] = static_cast<uint32_t>(cast_out<DT>(lo)) | (static_cast<uint32_t>(cast_out<DT>(hi)) << 16);
+  }
+  *reinterpret_cast<u32x4*>(out + m * H + n) = u32x4{ow[0], ow[1], ow[2], ow[3]};
+}
+
 }  // namespace
+
+// N / 2 must be a multiple of 8 and both tensors 16-byte aligned.
+int launch_swiglu_t(const void* in, int dtype, int64_t M, int64_t N, void* out, hipStream_t stream) {
+  const int64_t pieces = M * (N / 2) / 8;
+  const dim3 grid(static_cast<unsigned>((pieces + kThreads - 1) / kThreads));
+  if (dtype == WOL_DTYPE_BF16)
+    swiglu_t_kernel<WOL_DTYPE_BF16><<<grid, kThreads, 0, stream>>>(static_cast<const uint16_t*>(in), M, N,
+                                                                 static_cast<uint16_t*>(out));
+  else
+    swiglu_t_kernel<WOL_DTYPE_F16><<<grid, kThreads, 0, stream>>>(static_cast<const uint16_t*>(in), M, N,
+                                                                static_cast<uint16_t*>(out));
+  return hipGetLastError() == hipSuccess ? WOL_OK : WOL_ERR_HIP;
+}
 
 int launch_swiglu_f32(const float* in, int dtype, int64_t M, int64_t N, void* out, hipStream_t stream) {
   const int64_t quads = M * (N / 2) / 4;
