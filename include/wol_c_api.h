@@ -284,6 +284,19 @@ int wol_repack(const void* codes_in, int layout_in, void* codes_out,
                int layout_out, int64_t K, int64_t N, int bits, void* stream);
 
 /*
+ * wol_repack on HOST memory (no device work, no stream): the same re-layout
+ * done by the calling thread.  It is what a CPU weight_quantize kernel calls to
+ * hand out GFX950 weights -- the reference's CPU kernel ends in a layout step
+ * of its own (a byte transpose on HIP builds,
+ * paddle/phi/kernels/cpu/weight_quantize_kernel.cc:113-125) which this call
+ * replaces with layout_in = WOL_LAYOUT_CANONICAL, layout_out = WOL_LAYOUT_GFX950
+ * -- and what a loader uses for checkpoints that hold the reference's layout.
+ * codes_in and codes_out must not overlap.
+ */
+int wol_repack_host(const void* codes_in, int layout_in, void* codes_out,
+                    int layout_out, int64_t K, int64_t N, int bits);
+
+/*
  * Host-side index helper (no device work): byte offset of element (k, n) in a
  * code tensor of the given layout, and through *nibble_shift which nibble of
  * that byte holds it (0 or 4; always 0 for int8).  Returns -1 for arguments

@@ -32,6 +32,7 @@ SYMBOLS = (
     "wol_moe_ffn_workspace",
     "wol_moe_ffn",
     "wol_repack",
+    "wol_repack_host",
     "wol_code_offset",
     "wol_apply_per_channel_scale",
     "wol_read_floor",
@@ -89,6 +90,8 @@ def _load():
     lib.wol_moe_ffn.restype = ci
     lib.wol_repack.argtypes = [vp, ci, vp, ci, i64, i64, ci, vp]
     lib.wol_repack.restype = ci
+    lib.wol_repack_host.argtypes = [vp, ci, vp, ci, i64, i64, ci]
+    lib.wol_repack_host.restype = ci
     lib.wol_code_offset.argtypes = [ci, i64, i64, ci, i64, i64, ctypes.POINTER(ci)]
     lib.wol_code_offset.restype = i64
     lib.wol_apply_per_channel_scale.argtypes = [vp, vp, ci, i64, i64, vp, vp]

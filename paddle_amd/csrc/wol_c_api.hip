@@ -403,6 +403,29 @@ int wol_repack(const void* codes_in, int layout_in, void* codes_out, int layout_
                             static_cast<hipStream_t>(stream));
 }
 
+int wol_repack_host(const void* codes_in, int layout_in, void* codes_out, int layout_out, int64_t K,
+                    int64_t N, int bits) {
+  const int rc = check_problem(WOL_DTYPE_F16, K, N, bits, -1);
+  if (rc != WOL_OK) return rc;
+  if (!layout_ok(layout_in) || !layout_ok(layout_out)) return WOL_ERR_BAD_LAYOUT;
+  if (codes_in == nullptr || codes_out == nullptr) return WOL_ERR_NULL_POINTER;
+  if (codes_in == codes_out) return WOL_ERR_BAD_LAYOUT;  // not in place
+  const uint8_t* in = static_cast<const uint8_t*>(codes_in);
+  uint8_t* out = static_cast<uint8_t*>(codes_out);
+  if (bits == 4) std::memset(out, 0, static_cast<size_t>(K) * N / 2);  // nibbles are ORed in
+  for (int64_t k = 0; k < K; ++k)
+    for (int64_t n = 0; n < N; ++n) {
+      int si = 0, so = 0;
+      const int64_t oi = wol::code_offset(layout_in, K, N, bits, k, n, &si);
+      const int64_t oo = wol::code_offset(layout_out, K, N, bits, k, n, &so);
+      const int q = wol::decode_code(layout_in, bits, in[oi] >> si);
+      const int v = wol::encode_code(layout_out, bits, q);
+      if (bits == 8) out[oo] = static_cast<uint8_t>(v);
+      else out[oo] = static_cast<uint8_t>(out[oo] | (v << so));
+    }
+  return WOL_OK;
+}
+
 int64_t wol_code_offset(int layout, int64_t K, int64_t N, int bits, int64_t k, int64_t n,
                         int* nibble_shift) {
   if (check_problem(WOL_DTYPE_F16, K, N, bits, -1) != WOL_OK || !layout_ok(layout)) return -1;

@@ -245,3 +245,25 @@ def test_linear_plan_names_the_kernel_per_shape(lib):
     assert "gemm_dma_kernel" in plan(2048, 4096, 12288, 8, -1)
     assert "256x256" in plan(2048, 4096, 12288, 8, -1)
     assert lib.lib.wol_linear_plan(4, 4096, 100, 8, -1, 0, ctypes.create_string_buffer(8), 8) == 5
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+def test_repack_host_matches_the_layout_definitions(lib, bits):
+    # the CPU-side re-layout (what a CPU weight_quantize calls to hand out GFX950
+    # weights) against the numpy statements of the three layouts, every pair
+    from oracle import wo_oracle as O
+
+    K, N = 192, 96
+    wb = H.make_weight(K, N, H.BF16, seed=8)
+    oc, _ = O.weight_quantize(wb, H.BF16, bits, 64)
+    q = H.q_from_canonical(oc, bits)
+    forms = {0: np.ascontiguousarray(oc).view(np.uint8).reshape(-1),
+             1: H.paddle_hip_from_q(q, bits).view(np.uint8).reshape(-1),
+             2: H.gfx950_from_q(q, bits).reshape(-1)}
+    for li, src in forms.items():
+        for lo, want in forms.items():
+            out = np.full(src.size, 0xEE, np.uint8)
+            rc = lib.lib.wol_repack_host(src.ctypes.data, li, out.ctypes.data, lo, K, N, bits)
+            assert rc == 0 and np.array_equal(out, want), (li, lo)
+    assert lib.lib.wol_repack_host(forms[0].ctypes.data, 0, forms[0].ctypes.data, 2, K, N, bits) == 6
+    assert lib.lib.wol_repack_host(forms[0].ctypes.data, 5, forms[1].ctypes.data, 2, K, N, bits) == 6
