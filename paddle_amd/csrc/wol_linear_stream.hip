@@ -92,6 +92,11 @@ struct StreamKernel {
   // Walking wavefronts: K's whole weight tiles may end with a partial unit when
   // a unit spans several tiles (otherwise they divide into whole units).
   static constexpr bool kPartial = NU == 0 && kU > kSPT;
+  // Walking wavefronts: units in the ring, from the registers one unit takes.
+  // The ring stays within 64 registers: 16 wavefronts leave 128 each, and a
+  // narrower workgroup that needs more than 128 loses its neighbour on the CU.
+  static constexpr int kUnitRegs = 4 * (TN * kNT + kNA * MT + (PRE ? kNA : 0)) + (GROUPED ? TN * kNS : 0);
+  static constexpr int kD = 64 / kUnitRegs < 2 ? 2 : (64 / kUnitRegs > 4 ? 4 : 64 / kUnitRegs);
 
   const uint16_t* x;
   const uint16_t* scale;
@@ -155,6 +160,56 @@ struct StreamKernel {
   // The small loads (activations, scales) go first: the memory system returns
   // loads in order, so the first weight tile can be consumed while the later
   // ones are still on their way.
+  // Walking wavefronts load through buffer descriptors: `wr` ends with the
+  // wavefront's share of the strip, `xr` covers the activations.  A unit past
+  // the share (u > ulast) is requested like any other, from offsets beyond the
+  // descriptors: it costs no traffic and arrives as zeros, and with a zero A
+  // operand every sum it is added to stays exactly as it was.  Its scales repeat
+  // those of unit `ulast`.  Nothing in the walk is loaded under a condition, so
+  // the compiler counts precisely how many loads may still be in flight when a
+  // unit is consumed.
+  __device__ inline void load_unit_walk(Unit& d, const __amdgpu_buffer_rsrc_t (&wr)[TN],
+                                        __amdgpu_buffer_rsrc_t xr, int u, int ulast) const {
+    const bool real = u <= ulast;
+    const int step0 = (real ? u : ulast) * kU;
+    constexpr uint32_t kNowhere = 0xC0000000u;  // beyond every descriptor (activations end below 2^31 bytes)
+#pragma unroll
+    for (int a = 0; a < kNA; ++a)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        int m = mt * 16 + (j % MP);
+        if (MP > 1 || MT > 1) m = m < M ? m : M - 1;
+        const uint32_t off = static_cast<uint32_t>(m) * static_cast<uint32_t>(K) * 2u +
+                             static_cast<uint32_t>(step0 + a * kS + j / MP) * 64u + 16u * kb;
+        d.av[a][mt] = __builtin_bit_cast(
+            u32x4, __builtin_amdgcn_raw_buffer_load_b128(xr, static_cast<int>(real ? off : kNowhere), 0, 0));
+      }
+    if (PRE) {
+#pragma unroll
+      for (int a = 0; a < kNA; ++a) d.pv[a] = load_pre(step0 + a * kS, true);
+    }
+    if (GROUPED) {
+      const int mine = MP == 8 ? (kb >> 1) : kb;
+#pragma unroll
+      for (int p = 0; p < kNS; ++p) {
+        const int step = MP == 16 ? step0 + 2 * p
+                                  : step0 + (p / kPairs) * kS + mine * kRowsPerGroup + 2 * (p % kPairs);
+#pragma unroll
+        for (int t = 0; t < TN; ++t) d.sraw[t][p] = load_scale_raw(step, t);
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+#pragma unroll
+      for (int i = 0; i < kNT; ++i) {
+        // the whole offset in the vector operand: that is the one the
+        // hardware checks against the descriptor's size
+        const uint32_t off = real ? static_cast<uint32_t>(u * kNT + i) * 1024u + 16u * lane : kNowhere;
+        d.wv[t][i] = __builtin_bit_cast(
+            u32x4, __builtin_amdgcn_raw_buffer_load_b128(wr[t], static_cast<int>(off), 0, 2));
+      }
+  }
+
   __device__ inline void load_unit(Unit& d, const u32x4* const (&tp)[TN], int u, bool tail = false) const {
     const int step0 = u * kU;
 #pragma unroll
@@ -287,18 +342,43 @@ struct StreamKernel {
       // gives it the fewest whole units), ahead of its walk
       const bool tail = kPartial && wave == 0 && nunits * kU < vsteps;
       if (u0 < u1 || tail) {
-        Unit d0, d1;
         int u = u0;
-        if (tail) load_unit(d1, tp, nunits, true);
-        if (u0 < u1) load_unit(d0, tp, u);
-        if (tail) compute_unit(d1);
-        if (u0 < u1) while (true) {
-          if (u + 1 < u1) load_unit(d1, tp, u + 1);
-          compute_unit(d0);
-          if (++u >= u1) break;
-          if (u + 1 < u1) load_unit(d0, tp, u + 1);
-          compute_unit(d1);
-          if (++u >= u1) break;
+        if (tail) {
+          Unit dt;
+          load_unit(dt, tp, nunits, true);
+          compute_unit(dt);
+        }
+        if (u0 < u1) {
+          __amdgpu_buffer_rsrc_t wr[TN];
+#pragma unroll
+          for (int t = 0; t < TN; ++t)
+            wr[t] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(strip[t]), 0, u1 * kNT * 1024,
+                                                      0x00020000);
+          const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(
+              const_cast<uint16_t*>(x), 0, static_cast<int>(static_cast<uint32_t>(M) * static_cast<uint32_t>(K) * 2u),
+              0x00020000);
+          // A ring of kD units, kD - 1 of them on their way while one is
+          // consumed: what hides the memory latency is the number of bytes in
+          // flight, and a unit is small when the operand has many rows.  The
+          // barriers keep every load ahead of the arithmetic that follows it
+          // in program order.
+          Unit d[kD];
+#pragma unroll
+          for (int i = 0; i < kD - 1; ++i) load_unit_walk(d[i], wr, xr, u + i, u1 - 1);
+          for (; u + kD <= u1; u += kD) {
+#pragma unroll
+            for (int i = 0; i < kD; ++i) {
+              load_unit_walk(d[(i + kD - 1) % kD], wr, xr, u + i + kD - 1, u1 - 1);
+              __builtin_amdgcn_sched_barrier(0);
+              compute_unit(d[i]);
+              __builtin_amdgcn_sched_barrier(0);
+            }
+          }
+          // fewer than kD units are left, all of them requested already
+#pragma unroll
+          for (int i = 0; i < kD - 1; ++i) {
+            if (u + i < u1) compute_unit(d[i]);
+          }
         }
       }
       if (BITS == 4 && wave == 0) {
