@@ -231,6 +231,70 @@ def bench_decoder_stack(torch, Q, _lib, dev, quick):
     return res
 
 
+def bench_linear_grad(torch, np, Q, _lib, H, dev, quick, failures):
+    """weight_only_linear_grad on the prefill weight shape (int8 per-channel,
+    K = N = 4096, bf16): wol_linear_grad (scale preparation, out_grad
+    preparation and the MFMA product, three launches) beside the reference's
+    composition (weight_dequantize to T, then the library GEMM; torch.matmul
+    stands in for phi::MatmulKernel, both call hipBLASLt).  The composition is
+    only timed for comparison; a sample of the kernel's result is checked
+    against the oracle."""
+    K = N = 4096
+    bits, g, bf16, dt = 8, -1, torch.bfloat16, H.BF16
+    w = _device_weight(torch, K, N, bf16, 77, dev)
+    codes, scale = _quantize(Q, w, bits, g)
+    del w
+    rows = []
+    for M in ((2048,) if quick else (512, 2048, 8192)):
+        go = torch.randn((M, N), device=dev, dtype=torch.float32).to(bf16)
+        out = torch.empty((M, K), device=dev, dtype=bf16)
+        wsb = _lib.lib.wol_linear_grad_workspace(M, K, N, bits, g)
+        ws = torch.empty(wsb, dtype=torch.uint8, device=dev)
+
+        def step(_i):
+            _lib.check(_lib.lib.wol_linear_grad(go.data_ptr(), codes.data_ptr(), scale.data_ptr(), _lib.DTYPE_BF16, M, K,
+                                                N, bits, g, out.data_ptr(), ws.data_ptr(), wsb,
+                                                torch.cuda.current_stream().cuda_stream))
+
+        def comp(_i):
+            wdq = Q.weight_dequantize(codes, scale, algo="weight_only_int8", out_dtype="bfloat16", group_size=g)
+            return torch.matmul(go, wdq.t())
+
+        n = 10
+        med, mn = time_graph(torch, step, n, warm_launches=40, warm_ms=30.0, replays=5)
+        cmed, _ = time_graph(torch, comp, n, warm_launches=40, warm_ms=30.0, replays=5)
+        us, cus = med / n * 1e6, cmed / n * 1e6
+        tf = 2.0 * M * K * N / (med / n) / 1e12
+        step(0)
+        torch.cuda.synchronize()
+        r_s = 4  # rows checked against the oracle (scalar code)
+        rows.append({"M": M, "us": round(us, 2), "us_min": round(mn / n * 1e6, 2), "achieved": round(tf, 1),
+                     "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TF, 4),
+                     "dequantize_plus_library_gemm_us": round(cus, 2), "speed_vs_composition": round(cus / us, 3),
+                     "path": _plan_grad(_lib, M, K, N)})
+        if M == 2048:
+            gq = H.torch_to_bits(go[:r_s])
+            sample = (gq, H.torch_to_bits(out[:r_s]))
+    # the oracle needs canonical codes: quantise the same weight on the CPU
+    w_bits = H.torch_to_bits(_device_weight(torch, K, N, bf16, 77, dev))
+    oq, os_ = H.O.weight_quantize(w_bits, dt, bits, g)
+    _, wantT = H.O.linear_grad(sample[0], oq, os_, dt, bits, g)
+    err = H.rel_l2(H.bits_to_f32(sample[1], dt), H.bits_to_f32(wantT, dt))
+    if err > REL_L2_BAR:
+        failures.append("linear_grad output differs from the oracle")
+    return {"workload": "x_grad = out_grad [M, 4096] . dequant(W)[4096, 4096]^T, int8 per-channel, bf16",
+            "arithmetic": "fp16 MFMA operands, code*scale rounded once to 11 bits, fp32 sums",
+            "rows": rows, "rel_l2_vs_oracle": err, "parity_sample": "first 4 rows of the M=2048 result"}
+
+
+def _plan_grad(_lib, M, K, N):
+    import ctypes
+    buf = ctypes.create_string_buffer(256)
+    if _lib.lib.wol_linear_grad_plan(M, K, N, buf, 256) != 0:
+        return None
+    return buf.value.decode()
+
+
 def cpu_decode_baseline(np, torch, H, w_bits, x_bits, cfg, budget_s=10.0):
     """Oracle quantize (single thread, like the reference's CPU kernel) +
     dequantize to fp32 + fp32 matmul (torch CPU BLAS, all cores), on a bounded
@@ -445,12 +509,13 @@ def main():
         }
 
     # ---------------- every BASELINE configuration ----------------
-    configs = stack = None
+    configs = stack = grad = None
     if not args.no_configs:
         del copies, scales
         torch.cuda.empty_cache()
         configs = bench_configs(torch, Q, _lib, dev, args.quick)
         stack = bench_decoder_stack(torch, Q, _lib, dev, args.quick)
+        grad = bench_linear_grad(torch, np, Q, _lib, H, dev, args.quick, failures)
 
     # ---------------- parity of what was measured, against the oracle ----------------
     O = H.O
@@ -561,6 +626,7 @@ def main():
         },
         "configs": configs,
         "decoder_stack": stack,
+        "linear_grad": grad,
         "llm_int8": llm,
         "cpu_baseline": cpu,
         "parity": parity,

@@ -215,6 +215,37 @@ int wol_linear_fused(const void* x, const void* pre_scale, const void* codes,
                      void* stream);
 
 /*
+ * Replaces WeightOnlyLinearGradKernel<T, GPUContext>
+ * (paddle/phi/kernels/gpu/weight_only_linear_grad_kernel.cu:27-72; op
+ * paddle/phi/ops/yaml/backward.yaml:3651-3661): the only gradient of
+ * weight_only_linear,
+ *   x_grad[M, K] = out_grad[M, N] . dequant(W)[K, N]^T.
+ * The reference dequantises the whole weight to T and calls a library GEMM
+ * (per-channel scales only, :38-49).  Here one MFMA kernel contracts over n
+ * straight from the packed codes, for every group size; code * scale is
+ * rounded once to 11 significant bits (fp16 operands for both T, powers of two
+ * taken out per column and per row and put back exactly), never to T, and
+ * the sums are kept in fp32.  No bias and no activations are involved (x is
+ * no_need_buffer in the reference).
+ * codes: GFX950 layout.  scale: as for wol_linear.  The workspace holds the
+ * scaled out_grad and scales; wol_linear_grad_workspace() bytes are required.
+ */
+size_t wol_linear_grad_workspace(int64_t M, int64_t K, int64_t N, int bits,
+                                 int group_size);
+int wol_linear_grad(const void* out_grad, const void* codes, const void* scale,
+                    int dtype, int64_t M, int64_t K, int64_t N, int bits,
+                    int group_size, void* x_grad, void* workspace,
+                    size_t workspace_bytes, void* stream);
+
+/* Same as wol_linear_grad but writes the fp32 sums (times 2^-e[m]) instead of
+ * casting to T: x_grad_f32 is [M,K] float.  Used to check the arithmetic
+ * without the final rounding. */
+int wol_linear_grad_f32(const void* out_grad, const void* codes,
+                        const void* scale, int dtype, int64_t M, int64_t K,
+                        int64_t N, int bits, int group_size, float* x_grad_f32,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Replaces MoeFFNKernel<T, GPUContext> for quant_method "weight_only_int8" /
  * "weight_only_int4" (paddle/phi/kernels/fusion/cutlass/moe_ffn.cu:36-183,
  * whose CUTLASS grouped GEMMs :74-154 have no ROCm build): the expert FFN of a

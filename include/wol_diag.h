@@ -54,6 +54,10 @@ int wol_mfma_ceiling(const void* operands, int workgroups, int iters, float* out
 int wol_linear_plan(int64_t M, int64_t K, int64_t N, int bits, int group_size,
                     size_t workspace_bytes, char* buf, size_t buf_bytes);
 
+/* The same for wol_linear_grad: the tile of its MFMA kernel. */
+int wol_linear_grad_plan(int64_t M, int64_t K, int64_t N, char* buf,
+                         size_t buf_bytes);
+
 #ifdef __cplusplus
 }
 #endif

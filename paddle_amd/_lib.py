@@ -29,6 +29,9 @@ SYMBOLS = (
     "wol_linear_on",
     "wol_linear_fused_workspace",
     "wol_linear_fused",
+    "wol_linear_grad_workspace",
+    "wol_linear_grad",
+    "wol_linear_grad_f32",
     "wol_moe_ffn_workspace",
     "wol_moe_ffn",
     "wol_repack",
@@ -38,6 +41,7 @@ SYMBOLS = (
     "wol_read_floor",
     "wol_mfma_ceiling",
     "wol_linear_plan",
+    "wol_linear_grad_plan",
     "wol_llm_int8_linear_workspace",
     "wol_llm_int8_linear",
     "wol_llm_int8_linear_stage_offsets",
@@ -84,6 +88,12 @@ def _load():
     lib.wol_linear_fused_workspace.restype = sz
     lib.wol_linear_fused.argtypes = [vp, vp, vp, vp, vp, ci, i64, i64, i64, ci, ci, ci, vp, vp, sz, vp]
     lib.wol_linear_fused.restype = ci
+    lib.wol_linear_grad_workspace.argtypes = [i64, i64, i64, ci, ci]
+    lib.wol_linear_grad_workspace.restype = sz
+    lib.wol_linear_grad.argtypes = [vp, vp, vp, ci, i64, i64, i64, ci, ci, vp, vp, sz, vp]
+    lib.wol_linear_grad.restype = ci
+    lib.wol_linear_grad_f32.argtypes = [vp, vp, vp, ci, i64, i64, i64, ci, ci, vp, vp, sz, vp]
+    lib.wol_linear_grad_f32.restype = ci
     lib.wol_moe_ffn_workspace.argtypes = [i64, i64, i64, ci]
     lib.wol_moe_ffn_workspace.restype = sz
     lib.wol_moe_ffn.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, i64, i64, i64, ci, ci, vp, vp, sz, vp]
@@ -102,6 +112,8 @@ def _load():
     lib.wol_mfma_ceiling.restype = ci
     lib.wol_linear_plan.argtypes = [i64, i64, i64, ci, ci, sz, ctypes.c_char_p, sz]
     lib.wol_linear_plan.restype = ci
+    lib.wol_linear_grad_plan.argtypes = [i64, i64, i64, ctypes.c_char_p, sz]
+    lib.wol_linear_grad_plan.restype = ci
     lib.wol_llm_int8_linear_workspace.argtypes = [i64, i64, i64]
     lib.wol_llm_int8_linear_workspace.restype = sz
     lib.wol_llm_int8_linear.argtypes = [vp, vp, vp, vp, ctypes.c_float, ci, i64, i64, i64, vp, vp, sz, vp]

@@ -343,6 +343,44 @@ int wol_linear_fused(const void* x, const void* pre_scale, const void* codes, co
   return wol::launch_swiglu_f32(sums, dtype, M, N, out, s);
 }
 
+size_t wol_linear_grad_workspace(int64_t M, int64_t K, int64_t N, int bits, int group_size) {
+  if (check_problem(WOL_DTYPE_F16, K, N, bits, group_size) != WOL_OK || M <= 0 || M > (int64_t{1} << 24)) return 0;
+  return wol::linear_grad_workspace(M, K, N, group_size);
+}
+
+namespace {
+int linear_grad_impl(const void* out_grad, const void* codes, const void* scale, int dtype, int64_t M,
+                     int64_t K, int64_t N, int bits, int group_size, void* x_grad, bool out_f32,
+                     void* workspace, size_t workspace_bytes, void* stream) {
+  const int rc = check_problem(dtype, K, N, bits, group_size);
+  if (rc != WOL_OK) return rc;
+  if (M < 0 || M > (int64_t{1} << 24)) return WOL_ERR_BAD_SHAPE;
+  if (M == 0) return WOL_OK;
+  if (out_grad == nullptr || codes == nullptr || scale == nullptr || x_grad == nullptr) return WOL_ERR_NULL_POINTER;
+  if (!aligned16(out_grad) || !aligned16(codes) || !aligned16(x_grad)) return WOL_ERR_ALIGNMENT;
+  if (workspace == nullptr || workspace_bytes < wol::linear_grad_workspace(M, K, N, group_size))
+    return WOL_ERR_WORKSPACE;
+  if (!aligned16(workspace)) return WOL_ERR_ALIGNMENT;
+  if (const int dv = require_gfx950(); dv != WOL_OK) return dv;
+  return wol::launch_linear_grad(out_grad, codes, scale, dtype, M, K, N, bits, group_size, x_grad, out_f32,
+                                 workspace, static_cast<hipStream_t>(stream));
+}
+}  // namespace
+
+int wol_linear_grad(const void* out_grad, const void* codes, const void* scale, int dtype, int64_t M,
+                    int64_t K, int64_t N, int bits, int group_size, void* x_grad, void* workspace,
+                    size_t workspace_bytes, void* stream) {
+  return linear_grad_impl(out_grad, codes, scale, dtype, M, K, N, bits, group_size, x_grad, false, workspace,
+                          workspace_bytes, stream);
+}
+
+int wol_linear_grad_f32(const void* out_grad, const void* codes, const void* scale, int dtype, int64_t M,
+                        int64_t K, int64_t N, int bits, int group_size, float* x_grad_f32, void* workspace,
+                        size_t workspace_bytes, void* stream) {
+  return linear_grad_impl(out_grad, codes, scale, dtype, M, K, N, bits, group_size, x_grad_f32, true, workspace,
+                          workspace_bytes, stream);
+}
+
 namespace {
 int check_moe(int64_t rows, int64_t hidden, int64_t inter, int num_experts) {
   if (rows < 0 || rows > (int64_t{1} << 24) || hidden <= 0 || inter <= 0) return WOL_ERR_BAD_SHAPE;
@@ -483,6 +521,15 @@ int wol_llm_int8_linear(const void* x, const void* weight, const void* bias, con
   if (const int dv = require_gfx950(); dv != WOL_OK) return dv;
   return wol::launch_llm_int8_linear(x, weight, bias, weight_scale, threshold, dtype, M, K, N, out, workspace,
                                      static_cast<hipStream_t>(stream));
+}
+
+int wol_linear_grad_plan(int64_t M, int64_t K, int64_t N, char* buf, size_t buf_bytes) {
+  if (buf == nullptr || buf_bytes == 0) return WOL_ERR_NULL_POINTER;
+  const int rc = check_problem(WOL_DTYPE_F16, K, N, 8, -1);
+  if (rc != WOL_OK) return rc;
+  if (M <= 0 || M > (int64_t{1} << 24)) return WOL_ERR_BAD_SHAPE;
+  wol::describe_linear_grad(M, K, N, buf, buf_bytes);
+  return WOL_OK;
 }
 
 int wol_linear_plan(int64_t M, int64_t K, int64_t N, int bits, int group_size, size_t workspace_bytes,

@@ -285,6 +285,12 @@ int launch_linear_gemm(const void* x, const void* codes, const void* bias, const
                        int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
                        void* out, bool out_f32, void* workspace, size_t workspace_bytes,
                        hipStream_t stream, const Fuse& f = Fuse());
+// x_grad[M, K] = out_grad[M, N] . dequant(W)[K, N]^T from the packed codes.
+size_t linear_grad_workspace(int64_t M, int64_t K, int64_t N, int group_size);
+void describe_linear_grad(int64_t M, int64_t K, int64_t N, char* buf, size_t n);
+int launch_linear_grad(const void* out_grad, const void* codes, const void* scale, int dtype, int64_t M,
+                       int64_t K, int64_t N, int bits, int group_size, void* x_grad, bool out_f32,
+                       void* workspace, hipStream_t stream);
 int launch_read_floor(const void* codes, int64_t K, int64_t N, int bits, void* out,
                       hipStream_t stream);
 int launch_mfma_ceiling(const void* operands, int workgroups, int iters, float* out,

@@ -1,0 +1,551 @@
+// x_grad of weight_only_linear straight from the packed codes:
+//   x_grad[M, K] = out_grad[M, N] . dequant(W)[K, N]^T
+// (what paddle/phi/kernels/gpu/weight_only_linear_grad_kernel.cu:27-72
+// computes by dequantising the whole weight to T and calling a library GEMM).
+//
+// Arithmetic.  The contraction runs over n on v_mfma_f32_32x32x16_f16 with fp32
+// accumulation, for both element types T:
+//   c[n]    = the power of two that brings max_g |scale[g, n]| into [2^7, 2^8)
+//   s'[g,n] = scale[g, n] * 2^c[n]                 (exact: a T value fits fp16)
+//   B[n,k]  = fp16(code[k, n] * s'[g(k), n])       one rounding, 11 bits
+//   e[m]    = the power of two that brings max_n |out_grad[m, n]| * 2^-c[n]
+//             into [2^14, 2^15)
+//   A[m,n]  = fp16(out_grad[m, n] * 2^(e[m] - c[n]))  (exact unless the value
+//             lies more than 2^-29 below the row's largest: then it is tiny)
+//   x_grad[m,k] = T( 2^-e[m] * sum_n A[m,n] * B[n,k] )
+// so code * scale is rounded once, to 11 significant bits, whatever T is; it is
+// never rounded to T.  fp16 is used for bfloat16 tensors as well: a bfloat16
+// product code * scale would keep 8 bits.
+//
+// Three launches:
+//   grad_scales_kernel   c[n] and s' (fp16 bits) from the scale tensor
+//   grad_prepare_kernel  e[m] and A, one workgroup per row of out_grad
+//   grad_gemm_kernel     the product
+//
+// grad_gemm_kernel.  A workgroup of 8 wavefronts (2 along m, 4 along k) owns an
+// output tile of 64*TM rows by 128*TB columns and walks N in chunks of 64.
+// The packed layout keeps, per lane, eight consecutive k of one column n: the
+// transpose of what an MFMA operand wants for a contraction over n (eight
+// consecutive n of one k).  The weight therefore takes a detour through LDS:
+// a wavefront loads its share of the chunk's codes (a unit: 64 k of one
+// 16-column strip, 16 codes per lane), turns them into fp16 pairs (k, k+1),
+// trades halves with the neighbouring lane (one DPP move and one byte
+// permute) so that a dword holds columns (n, n+1) of one k, and stores dwords
+// into a [k][64 n] tile whose 16-byte pieces are XOR-swizzled such that both
+// these stores and the 128-bit operand reads are free of bank conflicts.
+// out_grad's tile goes global -> LDS with direct-to-LDS loads, as in the
+// forward GEMM.  Two stages: while chunk `it` is multiplied, chunk it+1 is
+// loaded, converted and stored; one workgroup barrier per chunk.
+#include <atomic>
+
+#include "wol_common.h"
+
+namespace wol {
+namespace {
+
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+constexpr int kChunk = 64;  // n per step of the contraction
+
+inline int64_t round_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
+
+// ---- preparation ---------------------------------------------------------
+
+// One thread per column n: c[n] and s'[g, n] for every group g.
+template <int DT>
+__global__ __launch_bounds__(256) void grad_scales_kernel(const uint16_t* __restrict__ scale, int groups,
+                                                          int N, uint16_t* __restrict__ sp,
+                                                          int* __restrict__ cexp) {
+  const int n = blockIdx.x * 256 + threadIdx.x;
+  if (n >= N) return;
+  float mx = 0.0f;
+  for (int g = 0; g < groups; ++g) mx = fmaxf(mx, fabsf(to_f32<DT>(scale[static_cast<int64_t>(g) * N + n])));
+  int c = 0;
+  if (mx > 0.0f && mx < __builtin_inff()) {
+    int e;
+    (void)frexpf(mx, &e);  // mx = f * 2^e, f in [0.5, 1)
+    c = 8 - e;
+  }
+  cexp[n] = c;
+  for (int g = 0; g < groups; ++g) {
+    const float s = to_f32<DT>(scale[static_cast<int64_t>(g) * N + n]);
+    sp[static_cast<int64_t>(g) * N + n] = f32_to_f16_rne(ldexpf(s, c));
+  }
+}
+
+// One workgroup per row m of out_grad: e[m], A[m, :] (row length npad, zeros
+// behind column N) and rowf[m] = 2^-e[m].
+template <int DT>
+__global__ __launch_bounds__(256) void grad_prepare_kernel(const uint16_t* __restrict__ dout,
+                                                           const int* __restrict__ cexp, int N, int npad,
+                                                           uint16_t* __restrict__ a, float* __restrict__ rowf) {
+  __shared__ float red[4];
+  const int m = blockIdx.x;
+  const uint16_t* row = dout + static_cast<int64_t>(m) * N;
+  float mx = 0.0f;
+  for (int n0 = threadIdx.x * 8; n0 < N; n0 += 256 * 8) {  // N is a multiple of 16
+    const u32x4 v = *reinterpret_cast<const u32x4*>(row + n0);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint16_t h = static_cast<uint16_t>(w[i / 2] >> (16 * (i % 2)));
+      mx = fmaxf(mx, ldexpf(fabsf(to_f32<DT>(h)), -cexp[n0 + i]));
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  int em = 0;
+  if (mx > 0.0f && mx < __builtin_inff()) {
+    int e;
+    (void)frexpf(mx, &e);
+    em = 15 - e;
+    em = em > 100 ? 100 : (em < -100 ? -100 : em);
+  }
+  if (threadIdx.x == 0) rowf[m] = ldexpf(1.0f, -em);
+  uint16_t* arow = a + static_cast<int64_t>(m) * npad;
+  for (int n0 = threadIdx.x * 8; n0 < npad; n0 += 256 * 8) {
+    u32x4 o = {0u, 0u, 0u, 0u};
+    if (n0 < N) {
+      const u32x4 v = *reinterpret_cast<const u32x4*>(row + n0);
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+      uint32_t r[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float lo = ldexpf(to_f32<DT>(static_cast<uint16_t>(w[i] & 0xFFFFu)), em - cexp[n0 + 2 * i]);
+        const float hi = ldexpf(to_f32<DT>(static_cast<uint16_t>(w[i] >> 16)), em - cexp[n0 + 2 * i + 1]);
+        r[i] = static_cast<uint32_t>(f32_to_f16_rne(lo)) | (static_cast<uint32_t>(f32_to_f16_rne(hi)) << 16);
+      }
+      o = u32x4{r[0], r[1], r[2], r[3]};
+    }
+    *reinterpret_cast<u32x4*>(arow + n0) = o;
+  }
+}
+
+// ---- the product ---------------------------------------------------------
+
+struct GradParams {
+  const uint16_t* a;     // [M, npad] fp16
+  const uint8_t* codes;  // GFX950 layout of the [K, N] weight
+  const uint16_t* sp;    // [groups, N] fp16
+  const float* rowf;     // [M]
+  void* out;             // [M, K] T, or float when out_f32
+  int out_f32;
+  int M, K, N, npad;
+  int gshift;            // log2(group size), -1: one scale row
+  int nbm, nbk;          // output tiles along m and k
+};
+
+// Every load (direct-to-LDS ones included) and LDS store of the wavefront has
+// completed, then the workgroup meets.
+__device__ inline void sync_stage() {
+  __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+  __syncthreads();
+}
+
+// XOR applied to the 16-byte piece index of a row of out_grad's tile (rows of
+// 128 bytes): a lane group reads the same piece of 16 consecutive rows.
+__device__ inline int a_swizzle(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+// The same for the weight tile, rows k of 128 bytes.  Stores of one instruction
+// go to rows k = i + 8*kb (kb = 0..3): bits 3 and 4 of k must move the
+// 32-byte window of a strip; operand reads go to 16 consecutive rows: bits 1
+// to 3 must spread over all eight pieces.
+__device__ inline int b_swizzle(int k) {
+  return ((k >> 1) & 1) | ((((k >> 2) ^ (k >> 4)) & 1) << 1) | (((k >> 3) & 1) << 2);
+}
+
+// s_waitcnt that only bounds the number of outstanding vector-memory loads.
+template <int N_>
+__device__ inline void wait_vmcnt() {
+  // gfx9 encoding: vmcnt = [15:14][3:0], expcnt = [6:4], lgkmcnt = [11:8]
+  __builtin_amdgcn_s_waitcnt((N_ & 0xF) | ((N_ >> 4) << 14) | (0x7 << 4) | (0xF << 8));
+}
+
+// AS: LDS stages of out_grad's tile (2 or 3); the weight tile has two.
+template <int DT, int BITS, int TM, int TB, int AS>
+__global__ __launch_bounds__(512) void grad_gemm_kernel(const GradParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int NW = 8, WKW = 4;
+  constexpr int BMR = 2 * TM * 32;    // rows of the output tile
+  constexpr int BKC = WKW * TB * 32;  // columns (k) of the output tile
+  constexpr int kABytes = BMR * 128, kBBytes = BKC * 128;
+  constexpr int kBBase = AS * kABytes;  // the weight stages lie behind out_grad's
+  constexpr int kLds = AS * kABytes + 2 * kBBytes;
+  constexpr int kALoads = BMR / 64;   // 1 KiB direct-to-LDS loads per wavefront
+  constexpr int kUnits = TB;          // units (64 k of one strip) per wavefront and chunk
+  constexpr int kCLoads = 2 * kUnits; // register loads per chunk: codes and scale of every unit
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WKW, wk = wave % WKW;
+  const int j = lane & 15, kb = lane >> 4, b = lane >> 5, r32 = lane & 31;
+  const int bm = blockIdx.x % p.nbm, bk = blockIdx.x / p.nbm;
+  const int m0 = bm * BMR, k0 = bk * BKC;
+  const int M = p.M, K = p.K, N = p.N;
+  const int nstrips = N / kStripCols;
+  const int niter = p.npad / kChunk;
+
+  // ---- out_grad's tile: sources of this lane's direct-to-LDS loads
+  const uint16_t* asrc[kALoads];
+#pragma unroll
+  for (int c = 0; c < kALoads; ++c) {
+    const int q = (c * NW + wave) * 64 + lane;
+    const int row = q / 8, slot = q % 8;
+    int m = m0 + row;
+    m = m < M ? m : M - 1;  // rows past M: valid data, never stored
+    asrc[c] = p.a + static_cast<int64_t>(m) * p.npad + (slot ^ a_swizzle(row)) * 8;
+  }
+
+  // ---- the weight units of this wavefront: unit u = wave * TB + c covers k
+  // chunk u / 4 (64 k) of strip u % 4 of the n chunk
+  int ustrip[kUnits];
+  const uint8_t* ucode[kUnits];   // the lane's codes in strip 0
+  const uint16_t* uscale[kUnits]; // the lane's scale in strip 0
+  uint32_t ulds[kUnits];          // byte offset of the lane's first store inside a weight tile
+#pragma unroll
+  for (int c = 0; c < kUnits; ++c) {
+    const int u = wave * TB + c;
+    ustrip[c] = u % 4;
+    const int ukc = u / 4;
+    int kc = k0 / 64 + ukc;
+    kc = kc < K / 64 ? kc : K / 64 - 1;  // columns past K: valid data, never stored
+    int64_t off;
+    if (BITS == 8) {
+      off = static_cast<int64_t>(kc) * 1024 + lane * 16;
+    } else {
+      const int full = K / 128;  // a K that is 64 mod 128 ends with a half tile, 8 bytes per lane
+      off = kc / 2 < full ? static_cast<int64_t>(kc / 2) * 1024 + lane * 16 + (kc % 2) * 8
+                          : static_cast<int64_t>(full) * 1024 + lane * 8;
+    }
+    ucode[c] = p.codes + off;
+    uscale[c] = p.sp + static_cast<int64_t>(p.gshift >= 0 ? (kc * 64) >> p.gshift : 0) * N + j;
+    // pair pr of k step `step` goes to row 64*ukc + 32*step + 8*kb + 2*pr + (j & 1),
+    // logical piece 2*strip + j / 8, dword (j / 2) % 4 of the piece
+    const int row = 64 * ukc + 8 * kb + (j & 1);
+    ulds[c] = static_cast<uint32_t>(row * 128 + ((j >> 1) & 3) * 4);
+  }
+  // piece index of the lane's stores before the part of the swizzle that
+  // depends on the pair: bits 3 and 4 of k come from kb
+  const int wpiece_lane = ((kb >> 1) << 1) | ((kb & 1) << 2);
+  const uint32_t xsel = (j & 1) ? 0x03020706u : 0x05040100u;  // see the trade below
+  const int64_t sbytes = strip_bytes(K, BITS);
+
+  // registers of one chunk's units
+  struct Raw {
+    uint32_t c[kUnits][BITS == 8 ? 4 : 2];
+    uint16_t s[kUnits];
+  };
+  auto load_units = [&](int it, Raw& r) {
+#pragma unroll
+    for (int c = 0; c < kUnits; ++c) {
+      int st = it * 4 + ustrip[c];
+      st = st < nstrips ? st : nstrips - 1;  // past N: finite codes against zeros of out_grad's tile
+      const uint8_t* src = ucode[c] + st * sbytes;
+      r.s[c] = uscale[c][st * kStripCols];
+      if (BITS == 8) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(src);
+        r.c[c][0] = v.x; r.c[c][1] = v.y; r.c[c][2] = v.z; r.c[c][3] = v.w;
+      } else {
+        const u32x2 v = *reinterpret_cast<const u32x2*>(src);
+        r.c[c][0] = v.x; r.c[c][1] = v.y;
+      }
+    }
+  };
+  // chunk `it` of out_grad's tile into stage it % AS; past the last chunk the
+  // last one is fetched again (into a stage nobody reads any more)
+  auto issue_a = [&](int it) {
+    unsigned char* stage = smem + (it % AS) * kABytes;
+    const int src = it < niter ? it : niter - 1;
+#pragma unroll
+    for (int c = 0; c < kALoads; ++c)
+      __builtin_amdgcn_global_load_lds(asrc[c] + src * kChunk, (lds_ptr_t)(stage + (c * NW + wave) * 1024), 16, 0, 0);
+  };
+  // Converts pairs (2*h, 2*h+1) of k step `step` of every unit and stores them
+  // into the weight tile `tile`: a quarter of a chunk's conversion work.
+  auto store_quarter = [&](unsigned char* tile, const Raw& r, int step, int h) {
+#pragma unroll
+    for (int c = 0; c < kUnits; ++c) {
+      const _Float16 sh = __builtin_bit_cast(_Float16, r.s[c]);
+      const f16x2 s2 = {sh, sh};
+      const int piece0 = (2 * ustrip[c] + (j >> 3)) ^ wpiece_lane;
+#pragma unroll
+      for (int pr = 2 * h; pr < 2 * h + 2; ++pr) {
+        // fp16 bits of (1024 + stored code) for k = 2*pr and 2*pr + 1 of the step
+        uint32_t bits2;
+        f16x2 off;
+        if (BITS == 8) {
+          const uint32_t d = r.c[c][2 * step + pr / 2];
+          // bytes (2*(pr%2), 2*(pr%2)+1) into the low bytes of the halves, 0x64 above them
+          bits2 = __builtin_amdgcn_perm(0x64646464u, d, (pr % 2) ? 0x04030402u : 0x04010400u);
+          off = f16x2{static_cast<_Float16>(-1152.0f), static_cast<_Float16>(-1152.0f)};
+        } else {
+          bits2 = ((r.c[c][step] >> (4 * pr)) & 0x000F000Fu) | 0x64006400u;
+          off = f16x2{static_cast<_Float16>(-1032.0f), static_cast<_Float16>(-1032.0f)};
+        }
+        // exact code, then one rounding in the product with s'
+        const f16x2 w2 = (__builtin_bit_cast(f16x2, bits2) + off) * s2;
+        // trade halves with the neighbouring lane (column n ^ 1): even lanes end
+        // up with row k (columns n, n+1), odd lanes with row k+1 (columns n-1, n)
+        const uint32_t mine = __builtin_bit_cast(uint32_t, w2);
+        int fresh;
+        asm volatile("" : "=v"(fresh));  // an undefined register for the lanes DPP does not write (none)
+        const uint32_t other = static_cast<uint32_t>(
+            __builtin_amdgcn_update_dpp(fresh, static_cast<int>(mine), 0xB1, 0xF, 0xF, false));
+        const uint32_t d = __builtin_amdgcn_perm(other, mine, xsel);
+        // the swizzle's pair-dependent bits: bit 1 and bit 2 of k = 2*pr + (j & 1)
+        const int piece = piece0 ^ ((pr & 1) | (((pr >> 1) & 1) << 1));
+        *reinterpret_cast<uint32_t*>(tile + ulds[c] + (32 * step + 2 * pr) * 128 + piece * 16) = d;
+      }
+    }
+  };
+
+  f32x16 acc[TM][TB];
+#pragma unroll
+  for (int a = 0; a < TM; ++a)
+#pragma unroll
+    for (int c = 0; c < TB; ++c)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][c][r] = 0.0f;
+
+  // operand reads: rows 32*t + r32 of a tile; the swizzles have period 16 (out_grad) and 32 (weight)
+  const int a_off = (wm * TM * 32 + r32) * 128;
+  const int a_swz = a_swizzle(r32 & 15);
+  const int b_off = (wk * TB * 32 + r32) * 128;
+  const int b_swz = b_swizzle(r32);
+  auto read_frags = [&](const unsigned char* at, const unsigned char* bt, u32x4 (&af)[TM], u32x4 (&bf)[TB], int q) {
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+      af[a] = *reinterpret_cast<const u32x4*>(at + a_off + a * 32 * 128 + (((2 * q + b) ^ a_swz) * 16));
+#pragma unroll
+    for (int c = 0; c < TB; ++c)
+      bf[c] = *reinterpret_cast<const u32x4*>(bt + b_off + c * 32 * 128 + (((2 * q + b) ^ b_swz) * 16));
+  };
+  auto chunk_of = [&](int it) { return it < niter ? it : niter - 1; };  // past the end: the last chunk again
+
+  // What is in flight.  While chunk `it` is multiplied, out_grad's tiles up to
+  // chunk it+AS-1 are on their way into LDS, the codes of chunk it+2 are on
+  // their way into registers, and the codes of chunk it+1 (loaded during the
+  // previous chunk) are converted and stored into the other weight tile.
+  // Loads past the last chunk repeat it into places nobody reads any more.
+  Raw raw[2];
+  issue_a(0);
+  load_units(0, raw[0]);
+  if (AS == 3) issue_a(1);
+  load_units(chunk_of(1), raw[1]);
+#pragma unroll
+  for (int q = 0; q < 4; ++q) store_quarter(smem + kBBase, raw[0], q / 2, q % 2);
+  // chunk 0 has landed: everything but the loads of chunk 1
+  wait_vmcnt<(AS == 3 ? kALoads : 0) + kCLoads>();
+  __builtin_amdgcn_s_waitcnt(0x0070 | (0xF << 0) | (3 << 14));  // lgkmcnt(0)
+  __builtin_amdgcn_s_barrier();
+
+  auto chunk = [&](int it, Raw& spare, const Raw& ready) {
+    const unsigned char* at = smem + (it % AS) * kABytes;
+    const unsigned char* bt = smem + kBBase + (it & 1) * kBBytes;
+    unsigned char* bnext = smem + kBBase + ((it + 1) & 1) * kBBytes;
+    // `spare` held chunk it (converted during the previous chunk)
+    issue_a(it + AS - 1);  // with three stages: the stage last read for chunk it-1
+    load_units(chunk_of(it + 2), spare);
+    __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of everything below
+    u32x4 af[2][TM], bf[2][TB];
+    read_frags(at, bt, af[0], bf[0], 0);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (q < 3) read_frags(at, bt, af[(q + 1) & 1], bf[(q + 1) & 1], q + 1);
+#pragma unroll
+      for (int a = 0; a < TM; ++a)
+#pragma unroll
+        for (int c = 0; c < TB; ++c)
+          acc[a][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, af[q & 1][a]),
+                                                             __builtin_bit_cast(f16x8, bf[q & 1][c]),
+                                                             acc[a][c], 0, 0, 0);
+      // a quarter of the next chunk's weight is converted in the shadow of the matrix pipe
+      store_quarter(bnext, ready, q / 2, q % 2);
+    }
+    // out_grad's tile of chunk it+1 has landed (loads issued since may still fly),
+    // this wavefront's stores are done, then the workgroup meets
+    wait_vmcnt<(AS == 3 ? kALoads : 0) + kCLoads>();
+    __builtin_amdgcn_s_waitcnt(0x0070 | (0xF << 0) | (3 << 14));  // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+  };
+  for (int it = 0; it < niter; it += 2) {
+    chunk(it, raw[0], raw[1]);
+    if (it + 1 < niter) chunk(it + 1, raw[1], raw[0]);
+  }
+  wait_vmcnt<0>();
+  __builtin_amdgcn_s_barrier();  // the spare loads are done and every wavefront has stopped reading
+
+  // ---- epilogue: 2^-e[m], cast, 32-row slabs leave through LDS as 16-byte stores
+  // accumulator element r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its block
+  const int col0 = k0 + wk * TB * 32;
+  if (p.out_f32) {  // verification mode: the sums before the cast, plain stores
+    float* outf = static_cast<float*>(p.out);
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+      for (int c = 0; c < TB; ++c)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = m0 + (wm * TM + a) * 32 + 8 * (r / 4) + 4 * b + r % 4;
+          const int k = col0 + c * 32 + r32;
+          if (m < M && k < K) outf[static_cast<int64_t>(m) * K + k] = acc[a][c][r] * p.rowf[m];
+        }
+    return;
+  }
+  uint16_t* out = static_cast<uint16_t*>(p.out);
+  constexpr int kSlabRow = TB * 32 + 8;  // padded, in elements
+  static_assert(NW * 32 * kSlabRow * 2 <= kLds, "slabs must fit in the stage buffers");
+  uint16_t* slab = reinterpret_cast<uint16_t*>(smem) + wave * 32 * kSlabRow;
+  constexpr int kPieces = 32 * (TB * 32 / 8);
+#pragma unroll
+  for (int a = 0; a < TM; ++a) {
+    float rf[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      int m = m0 + (wm * TM + a) * 32 + 8 * (r / 4) + 4 * b + r % 4;
+      m = m < M ? m : M - 1;
+      rf[r] = p.rowf[m];
+    }
+#pragma unroll
+    for (int c = 0; c < TB; ++c)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        slab[(8 * (r / 4) + 4 * b + r % 4) * kSlabRow + c * 32 + r32] = cast_out<DT>(acc[a][c][r] * rf[r]);
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int q = lane; q < kPieces; q += 64) {
+      const int r = q / (TB * 4), cc = q % (TB * 4);
+      const int m = m0 + (wm * TM + a) * 32 + r;
+      const int k = col0 + cc * 8;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(&slab[r * kSlabRow + cc * 8]);
+      if (m < M && k < K) *reinterpret_cast<u32x4*>(out + static_cast<int64_t>(m) * K + k) = v;
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+#endif
+}
+
+template <int DT, int BITS, int TM, int TB, int AS>
+void launch_cfg(const GradParams& p0, hipStream_t stream) {
+  GradParams p = p0;
+  constexpr int BMR = 2 * TM * 32, BKC = 4 * TB * 32;
+  p.nbm = (p.M + BMR - 1) / BMR;
+  p.nbk = (p.K + BKC - 1) / BKC;
+  const size_t lds = static_cast<size_t>(AS * BMR + 2 * BKC) * 128;
+  auto kern = grad_gemm_kernel<DT, BITS, TM, TB, AS>;
+  // more than 64 KiB of LDS must be allowed once per device
+  static std::atomic<uint32_t> done{0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+  const uint32_t bit = 1u << (dev & 31);
+  if (!(done.load(std::memory_order_acquire) & bit)) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              static_cast<int>(lds));
+    done.fetch_or(bit, std::memory_order_release);
+  }
+  kern<<<dim3(static_cast<unsigned>(p.nbm * p.nbk)), dim3(512), lds, stream>>>(p);
+}
+
+// Tile choice.  Every element of the weight is converted once per row tile, so
+// tall tiles are preferred; a tile count of at least 7/8 of the CUs (256) keeps
+// the device busy.
+void pick_tile(int64_t M, int64_t K, int* tm, int* tb) {
+  auto count = [&](int t_m, int t_b) {
+    return ((M + 64 * t_m - 1) / (64 * t_m)) * ((K + 128 * t_b - 1) / (128 * t_b));
+  };
+  if (count(4, 2) >= 224) { *tm = 4; *tb = 2; return; }
+  if (count(4, 1) >= 224) { *tm = 4; *tb = 1; return; }
+  if (count(2, 2) >= 224) { *tm = 2; *tb = 2; return; }
+  *tm = 2; *tb = 1;
+}
+
+template <int DT, int BITS>
+void launch_gemm(const GradParams& p, hipStream_t stream) {
+  int tm, tb;
+  pick_tile(p.M, p.K, &tm, &tb);
+  if (tm == 4 && tb == 2) launch_cfg<DT, BITS, 4, 2, 2>(p, stream);
+  else if (tm == 4) launch_cfg<DT, BITS, 4, 1, 3>(p, stream);
+  else if (tb == 2) launch_cfg<DT, BITS, 2, 2, 3>(p, stream);
+  else launch_cfg<DT, BITS, 2, 1, 3>(p, stream);
+}
+
+struct Layout {
+  size_t sp, cexp, rowf, a, total;
+  int64_t npad, groups;
+};
+
+Layout layout_of(int64_t M, int64_t K, int64_t N, int group_size) {
+  Layout l;
+  l.npad = round_up(N, kChunk);
+  l.groups = group_size > 0 ? (K + group_size - 1) / group_size : 1;  // a K of 64 still has one group of 128
+  l.sp = 0;
+  l.cexp = round_up(static_cast<size_t>(l.groups) * N * 2, 256);
+  l.rowf = l.cexp + round_up(static_cast<size_t>(N) * 4, 256);
+  l.a = l.rowf + round_up(static_cast<size_t>(M) * 4, 256);
+  l.total = l.a + round_up(static_cast<size_t>(M) * l.npad * 2, 256);
+  return l;
+}
+
+}  // namespace
+
+size_t linear_grad_workspace(int64_t M, int64_t K, int64_t N, int group_size) {
+  return layout_of(M, K, N, group_size).total;
+}
+
+void describe_linear_grad(int64_t M, int64_t K, int64_t N, char* buf, size_t n) {
+  int tm, tb;
+  pick_tile(M, K, &tm, &tb);
+  snprintf(buf, n, "wol::grad_gemm_kernel: %d rows x %d columns (k) per workgroup, N in chunks of %d",
+           64 * tm, 128 * tb, kChunk);
+  (void)N;
+}
+
+int launch_linear_grad(const void* out_grad, const void* codes, const void* scale, int dtype, int64_t M,
+                       int64_t K, int64_t N, int bits, int group_size, void* x_grad, bool out_f32,
+                       void* workspace, hipStream_t stream) {
+  const Layout l = layout_of(M, K, N, group_size);
+  unsigned char* ws = static_cast<unsigned char*>(workspace);
+  uint16_t* sp = reinterpret_cast<uint16_t*>(ws + l.sp);
+  int* cexp = reinterpret_cast<int*>(ws + l.cexp);
+  float* rowf = reinterpret_cast<float*>(ws + l.rowf);
+  uint16_t* a = reinterpret_cast<uint16_t*>(ws + l.a);
+  const uint16_t* sc = static_cast<const uint16_t*>(scale);
+  const uint16_t* dout = static_cast<const uint16_t*>(out_grad);
+  const dim3 sgrid(static_cast<unsigned>((N + 255) / 256)), pgrid(static_cast<unsigned>(M));
+  if (dtype == WOL_DTYPE_BF16) {
+    grad_scales_kernel<WOL_DTYPE_BF16><<<sgrid, 256, 0, stream>>>(sc, static_cast<int>(l.groups), static_cast<int>(N), sp, cexp);
+    grad_prepare_kernel<WOL_DTYPE_BF16><<<pgrid, 256, 0, stream>>>(dout, cexp, static_cast<int>(N), static_cast<int>(l.npad), a, rowf);
+  } else {
+    grad_scales_kernel<WOL_DTYPE_F16><<<sgrid, 256, 0, stream>>>(sc, static_cast<int>(l.groups), static_cast<int>(N), sp, cexp);
+    grad_prepare_kernel<WOL_DTYPE_F16><<<pgrid, 256, 0, stream>>>(dout, cexp, static_cast<int>(N), static_cast<int>(l.npad), a, rowf);
+  }
+  GradParams p;
+  p.a = a;
+  p.codes = static_cast<const uint8_t*>(codes);
+  p.sp = sp;
+  p.rowf = rowf;
+  p.out = x_grad;
+  p.out_f32 = out_f32 ? 1 : 0;
+  p.M = static_cast<int>(M);
+  p.K = static_cast<int>(K);
+  p.N = static_cast<int>(N);
+  p.npad = static_cast<int>(l.npad);
+  p.gshift = group_size == 64 ? 6 : (group_size == 128 ? 7 : -1);
+  p.nbm = p.nbk = 0;
+  if (dtype == WOL_DTYPE_BF16) {
+    if (bits == 8) launch_gemm<WOL_DTYPE_BF16, 8>(p, stream); else launch_gemm<WOL_DTYPE_BF16, 4>(p, stream);
+  } else {
+    if (bits == 8) launch_gemm<WOL_DTYPE_F16, 8>(p, stream); else launch_gemm<WOL_DTYPE_F16, 4>(p, stream);
+  }
+  return check_launch();
+}
+
+}  // namespace wol

@@ -61,7 +61,8 @@ __device__ inline float sum_lane_groups(float v, bool x16, bool x32) {
 // NU > 0: every wavefront owns exactly NU units and issues all their loads at
 // once (the whole problem is in flight from the first cycle; used when K is
 // small enough).  NU == 0: a wavefront walks its share of the units with the
-// loads of the next unit in flight while it consumes the current one.
+// loads of the next units (one to three, by register budget) in flight while
+// it consumes the current one.
 //
 // TN strips (16 columns each) share one workgroup and with it every load of
 // the activations: the activation traffic out of L2, which grows with M, drops
@@ -587,7 +588,7 @@ void launch_m(const Args& a, int wk, int nu) {
 // enough that one unit per wavefront keeps every wavefront resident at once
 // (at most ~6 per SIMD on 1024 SIMDs) and the unit count per strip is a power
 // of two up to 16, each wavefront takes exactly one unit and loads it at once.
-// Otherwise wavefronts walk several units with two in flight, and WK follows
+// Otherwise wavefronts walk several units with up to three more in flight, and WK follows
 // a budget of resident wavefronts that shrinks with the row count.
 static void pick_split(int64_t M, int64_t K, int64_t N, int bits, int* wk, int* nu, int* tn) {
   int mp = 1;
@@ -632,7 +633,7 @@ void describe_linear_stream(int64_t M, int64_t K, int64_t N, int bits, int group
   while (mp < 16 && mp < M) mp *= 2;
   snprintf(buf, n, "wol::stream_kernel: %lld workgroups of %d wavefronts, %d strip(s) each, %d-row operands x %d, %s",
            static_cast<long long>((N / kStripCols + tn - 1) / tn), wk, tn, mp, static_cast<int>((M + 15) / 16),
-           nu > 0 ? "all loads of a wavefront issued at once" : "wavefronts walk their units double-buffered");
+           nu > 0 ? "all loads of a wavefront issued at once" : "wavefronts walk their units through a ring of loads");
   (void)group_size;
 }
 

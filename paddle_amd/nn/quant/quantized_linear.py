@@ -320,21 +320,39 @@ def _linear_call(fn, x, weight, bias, weight_scale, weight_dtype, group_size, ou
 
 def weight_only_linear_grad(x, weight, bias, weight_scale, out_grad, weight_dtype="int8", arch=None,
                             group_size=-1):
-    """x_grad of weight_only_linear, composed as the reference composes it
-    (paddle/phi/kernels/gpu/weight_only_linear_grad_kernel.cu:52-69): the weight
-    is dequantised to T with this library's kernel and multiplied by the
-    library GEMM (torch.matmul standing in for phi::MatmulKernel):
-    x_grad[M,K] = out_grad[M,N] . dequant(W)[K,N]^T.  The reference restricts
-    this op to per-channel scales and arch 80/86; every group size works here.
-    x is only used for its shape (no_need_buffer in the reference's backward.yaml)."""
-    algo = "weight_only_int8" if weight_dtype == "int8" else "weight_only_int4"
-    names = {torch.float16: "float16", torch.bfloat16: "bfloat16"}
-    if out_grad.dtype not in names:
-        raise ValueError("(InvalidArgument) out_grad must be float16 or bfloat16")
-    wdq = weight_dequantize(weight, weight_scale, algo=algo, out_dtype=names[out_grad.dtype],
-                            group_size=group_size)
-    g2 = out_grad.reshape(-1, out_grad.shape[-1])
-    return torch.matmul(g2, wdq.t()).reshape(x.shape)
+    """x_grad of weight_only_linear, the op's only gradient
+    (paddle/phi/kernels/gpu/weight_only_linear_grad_kernel.cu:27-72,
+    backward.yaml:3651-3661): x_grad[M,K] = out_grad[M,N] . dequant(W)[K,N]^T.
+    The reference dequantises the weight to T and calls a library GEMM, for
+    per-channel scales and arch 80/86 only; here wol_linear_grad contracts over
+    n straight from the packed codes, for every group size, without rounding
+    code * scale to T.  x is only used for its shape (no_need_buffer in the
+    reference's backward.yaml); bias gets no gradient and is ignored."""
+    if weight_dtype not in ("int8", "int4"):
+        raise ValueError("(InvalidArgument) weight_dtype must be 'int8' or 'int4', but got %r" % (weight_dtype,))
+    _check_group_size(group_size, "weight_only_linear_grad")
+    _require_gpu(out_grad, "out_grad")
+    _require_gpu(weight, "weight")
+    dt = _dtype_id(out_grad, "out_grad")
+    bits = 8 if weight_dtype == "int8" else 4
+    N = out_grad.shape[-1]
+    K = x.shape[-1]
+    if weight_scale.dtype != out_grad.dtype:
+        raise ValueError("(InvalidArgument) weight_scale and out_grad must have the same dtype")
+    g2 = out_grad.reshape(-1, N).contiguous()
+    M = g2.shape[0]
+    out = torch.empty((M, K), dtype=out_grad.dtype, device=out_grad.device)
+    if M:
+        with torch.cuda.device(out_grad.device):
+            ws_bytes = _lib.lib.wol_linear_grad_workspace(M, K, N, bits, group_size)
+            ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=out_grad.device)
+            _lib.check(
+                _lib.lib.wol_linear_grad(
+                    g2.data_ptr(), weight.data_ptr(), weight_scale.data_ptr(), dt, M, K, N, bits,
+                    group_size, out.data_ptr(), ws.data_ptr(), ws_bytes, _stream_ptr(out_grad),
+                )
+            )
+    return out.reshape(tuple(x.shape))
 
 
 class _WeightOnlyLinearFn(torch.autograd.Function):
