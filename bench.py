@@ -61,6 +61,9 @@ def _quantize(Q, w, bits, group_size):
     return Q.weight_quantize(w, algo=algo, group_size=group_size)
 
 
+EAGER = False  # --eager: every leg launches eagerly (for counter collection, which needs plain dispatches)
+
+
 def time_graph(torch, fn, launches, warm_launches=400, warm_ms=50.0, replays=REPLAYS, eager=False):
     """fn(i) enqueues launch i on the current stream.  Captures `launches`
     calls into one HIP graph, replays it untimed until both warm-up thresholds
@@ -69,7 +72,7 @@ def time_graph(torch, fn, launches, warm_launches=400, warm_ms=50.0, replays=REP
     for i in range(3):
         fn(i)
     torch.cuda.synchronize()
-    if eager:
+    if eager or EAGER:
         def run():
             for i in range(launches):
                 fn(i)
@@ -405,6 +408,8 @@ def main():
         del src, dst
 
     failures = []
+    global EAGER
+    EAGER = args.eager
 
     # ---------------- decode (the headline metric) ----------------
     c = DECODE

@@ -153,12 +153,18 @@ __device__ inline void sync_stage() {
 // 128 bytes): a lane group reads the same piece of 16 consecutive rows.
 __device__ inline int a_swizzle(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
-// The same for the weight tile, rows k of 128 bytes.  Stores of one instruction
-// go to rows k = i + 8*kb (kb = 0..3): bits 3 and 4 of k must move the
-// 32-byte window of a strip; operand reads go to 16 consecutive rows: bits 1
-// to 3 must spread over all eight pieces.
+// The same for the weight tile, rows k of 128 bytes: a linear map of the low
+// five bits of k to a 3-bit piece XOR, chosen so that no access of the kernel
+// has a bank conflict whether the LDS serves 128 or 256 bytes per cycle:
+//   * 128-bit operand reads: 8 (16) consecutive rows, the same logical piece ->
+//     8 distinct pieces (and 16 distinct piece/row-parity pairs);
+//   * the dword stores of one instruction: rows i + 8*kb + (j & 1), pieces
+//     2*strip + j/8 -> the 8 combinations of (j & 1, kb & 1, j / 8) (128 bytes
+//     per cycle: half a wavefront) and of (kb, j / 8) per row parity (256) all
+//     land in different pieces.
 __device__ inline int b_swizzle(int k) {
-  return ((k >> 1) & 1) | ((((k >> 2) ^ (k >> 4)) & 1) << 1) | (((k >> 3) & 1) << 2);
+  const int k0 = k & 1, k1 = (k >> 1) & 1, k2 = (k >> 2) & 1, k3 = (k >> 3) & 1, k4 = (k >> 4) & 1;
+  return k1 | ((k0 ^ k2 ^ k4) << 1) | ((k2 ^ k3) << 2);
 }
 
 // s_waitcnt that only bounds the number of outstanding vector-memory loads.
@@ -232,9 +238,9 @@ __global__ __launch_bounds__(512) void grad_gemm_kernel(const GradParams p) {
     const int row = 64 * ukc + 8 * kb + (j & 1);
     ulds[c] = static_cast<uint32_t>(row * 128 + ((j >> 1) & 3) * 4);
   }
-  // piece index of the lane's stores before the part of the swizzle that
-  // depends on the pair: bits 3 and 4 of k come from kb
-  const int wpiece_lane = ((kb >> 1) << 1) | ((kb & 1) << 2);
+  // the lane's part of the stores' swizzle (k = 8*kb + 2*pr + (j & 1): bits 0, 3
+  // and 4 of k are the lane's, bits 1 and 2 the pair's)
+  const int wpiece_lane = b_swizzle(8 * kb + (j & 1));
   const uint32_t xsel = (j & 1) ? 0x03020706u : 0x05040100u;  // see the trade below
   const int64_t sbytes = strip_bytes(K, BITS);
 
@@ -300,8 +306,8 @@ __global__ __launch_bounds__(512) void grad_gemm_kernel(const GradParams p) {
         const uint32_t other = static_cast<uint32_t>(
             __builtin_amdgcn_update_dpp(fresh, static_cast<int>(mine), 0xB1, 0xF, 0xF, false));
         const uint32_t d = __builtin_amdgcn_perm(other, mine, xsel);
-        // the swizzle's pair-dependent bits: bit 1 and bit 2 of k = 2*pr + (j & 1)
-        const int piece = piece0 ^ ((pr & 1) | (((pr >> 1) & 1) << 1));
+        // the swizzle is linear: the pair's part is that of k = 2*pr
+        const int piece = piece0 ^ b_swizzle(2 * pr);
         *reinterpret_cast<uint32_t*>(tile + ulds[c] + (32 * step + 2 * pr) * 128 + piece * 16) = d;
       }
     }
