@@ -171,6 +171,31 @@ def test_linear_random_shapes_all_kernels(G, oracle):
         check(G, oracle, dt, bits, g, M, K, N, bias=bool(rng.integers(2)), seed=case, **kw)
 
 
+@pytest.mark.parametrize("bits,g", [(8, -1), (4, 64)])
+def test_cpu_quantised_weight_through_repack_host(G, oracle, bits, g):
+    # The flow of a weight that never saw the GPU quantiser: quantised on the CPU
+    # (the oracle stands for the reference's CPU kernel), stored in the layout a
+    # ROCm build of that kernel emits (cpu/weight_quantize_kernel.cc:113-125),
+    # re-laid once on the host with wol_repack_host, then used by the GPU linear
+    # at one row, a few rows and a GEMM-sized batch.  Fed to the kernels without
+    # the re-layout the same bytes give numbers that are simply wrong.
+    from paddle_amd import _lib
+
+    dt, K, N = H.BF16, 512, 256
+    wb = H.make_weight(K, N, dt, seed=21)
+    oc, osc = oracle.weight_quantize(wb, dt, bits, g)
+    hip = np.ascontiguousarray(H.paddle_hip_from_q(H.q_from_canonical(oc, bits), bits)).view(np.uint8).reshape(-1)
+    packed = np.full(hip.size, 0xEE, np.uint8)
+    assert _lib.lib.wol_repack_host(hip.ctypes.data, 1, packed.ctypes.data, 2, K, N, bits) == 0
+    for M in (1, 5, 96):
+        xb = H.make_act(M, K, dt, seed=M)
+        _, wantT = oracle.linear(xb, oc, osc, None, dt, bits, g)
+        got = G.linear(xb, packed, None, osc, dt, N, bits, g)
+        assert H.rel_l2(H.bits_to_f32(got, dt), H.bits_to_f32(wantT, dt)) <= 1e-3, (bits, g, M)
+        wrong = G.linear(xb, hip, None, osc, dt, N, bits, g)
+        assert H.rel_l2(H.bits_to_f32(wrong, dt), H.bits_to_f32(wantT, dt)) > 0.1
+
+
 # The reference's own test matrix (test/quantization/test_weight_only_linear.py:
 # 62-614): dtype x weight dtype x bias x token x group size x (K, N), x ~ U[0,1),
 # compared there with a dense fp16/bf16 Linear at atol 1e-2 .. 0.13; here against
