@@ -17,7 +17,8 @@
 // never rounded to T.  fp16 is used for bfloat16 tensors as well: a bfloat16
 // product code * scale would keep 8 bits.
 //
-// Three launches:
+// Three launches (two with per-channel scales, where the first rides along
+// with the second):
 //   grad_scales_kernel   c[n] and s' (fp16 bits) from the scale tensor
 //   grad_prepare_kernel  e[m] and A, one workgroup per row of out_grad
 //   grad_gemm_kernel     the product
@@ -55,6 +56,15 @@ inline int64_t round_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
 // ---- preparation ---------------------------------------------------------
 
+// c for a column whose largest scale magnitude is mx.
+__device__ inline int column_exponent(float mx) {
+  if (!(mx > 0.0f && mx < __builtin_inff())) return 0;
+  int e;
+  (void)frexpf(mx, &e);  // mx = f * 2^e, f in [0.5, 1)
+  const int c = 8 - e;
+  return c > 120 ? 120 : (c < -120 ? -120 : c);  // fits a byte; scales below 2^-112 lose their normalisation
+}
+
 // One thread per column n: c[n] and s'[g, n] for every group g.
 template <int DT>
 __global__ __launch_bounds__(256) void grad_scales_kernel(const uint16_t* __restrict__ scale, int groups,
@@ -64,12 +74,7 @@ __global__ __launch_bounds__(256) void grad_scales_kernel(const uint16_t* __rest
   if (n >= N) return;
   float mx = 0.0f;
   for (int g = 0; g < groups; ++g) mx = fmaxf(mx, fabsf(to_f32<DT>(scale[static_cast<int64_t>(g) * N + n])));
-  int c = 0;
-  if (mx > 0.0f && mx < __builtin_inff()) {
-    int e;
-    (void)frexpf(mx, &e);  // mx = f * 2^e, f in [0.5, 1)
-    c = 8 - e;
-  }
+  const int c = column_exponent(mx);
   cexp[n] = c;
   for (int g = 0; g < groups; ++g) {
     const float s = to_f32<DT>(scale[static_cast<int64_t>(g) * N + n]);
@@ -78,23 +83,72 @@ __global__ __launch_bounds__(256) void grad_scales_kernel(const uint16_t* __rest
 }
 
 // One workgroup per row m of out_grad: e[m], A[m, :] (row length npad, zeros
-// behind column N) and rowf[m] = 2^-e[m].
-template <int DT>
+// behind column N) and rowf[m] = 2^-e[m].  The row stays in registers between
+// the two passes when it has at most kKeep * 2048 elements.
+// ONE: per-channel scales.  c[n] then follows from scale[n] alone and is
+// computed on the spot (no grad_scales_kernel launch, no c array); workgroup 0
+// also writes s'.
+template <int DT, bool ONE>
 __global__ __launch_bounds__(256) void grad_prepare_kernel(const uint16_t* __restrict__ dout,
-                                                           const int* __restrict__ cexp, int N, int npad,
+                                                           const int* __restrict__ cexp,
+                                                           const uint16_t* __restrict__ scale,
+                                                           uint16_t* __restrict__ sp, int N, int npad,
                                                            uint16_t* __restrict__ a, float* __restrict__ rowf) {
+  constexpr int kKeep = 4;
   __shared__ float red[4];
   const int m = blockIdx.x;
   const uint16_t* row = dout + static_cast<int64_t>(m) * N;
+  const bool keep = N <= kKeep * 256 * 8;
+  // the eight c of columns n0 .. n0+7
+  auto load_c = [&](int n0, int (&c)[8]) {
+    if (ONE) {
+      const u32x4 sv = *reinterpret_cast<const u32x4*>(scale + n0);
+      const uint32_t sw[4] = {sv.x, sv.y, sv.z, sv.w};
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        c[i] = column_exponent(fabsf(to_f32<DT>(static_cast<uint16_t>(sw[i / 2] >> (16 * (i % 2))))));
+      if (m == 0) {
+        uint32_t r[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float lo = ldexpf(to_f32<DT>(static_cast<uint16_t>(sw[i] & 0xFFFFu)), c[2 * i]);
+          const float hi = ldexpf(to_f32<DT>(static_cast<uint16_t>(sw[i] >> 16)), c[2 * i + 1]);
+          r[i] = static_cast<uint32_t>(f32_to_f16_rne(lo)) | (static_cast<uint32_t>(f32_to_f16_rne(hi)) << 16);
+        }
+        *reinterpret_cast<u32x4*>(sp + n0) = u32x4{r[0], r[1], r[2], r[3]};
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) c[i] = cexp[n0 + i];
+    }
+  };
+  u32x4 held[kKeep];
+  int8_t heldc[kKeep][8];
   float mx = 0.0f;
-  for (int n0 = threadIdx.x * 8; n0 < N; n0 += 256 * 8) {  // N is a multiple of 16
+  auto scan = [&](int n0, int slot) {
     const u32x4 v = *reinterpret_cast<const u32x4*>(row + n0);
+    int c[8];
+    load_c(n0, c);
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const uint16_t h = static_cast<uint16_t>(w[i / 2] >> (16 * (i % 2)));
-      mx = fmaxf(mx, ldexpf(fabsf(to_f32<DT>(h)), -cexp[n0 + i]));
+      mx = fmaxf(mx, ldexpf(fabsf(to_f32<DT>(h)), -c[i]));
     }
+    if (slot >= 0) {
+      held[slot] = v;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) heldc[slot][i] = static_cast<int8_t>(c[i]);
+    }
+  };
+  if (keep) {
+#pragma unroll
+    for (int t = 0; t < kKeep; ++t) {
+      const int n0 = (t * 256 + static_cast<int>(threadIdx.x)) * 8;
+      if (n0 < N) scan(n0, t);
+    }
+  } else {
+    for (int n0 = threadIdx.x * 8; n0 < N; n0 += 256 * 8) scan(n0, -1);  // N is a multiple of 16
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
@@ -110,21 +164,44 @@ __global__ __launch_bounds__(256) void grad_prepare_kernel(const uint16_t* __res
   }
   if (threadIdx.x == 0) rowf[m] = ldexpf(1.0f, -em);
   uint16_t* arow = a + static_cast<int64_t>(m) * npad;
-  for (int n0 = threadIdx.x * 8; n0 < npad; n0 += 256 * 8) {
-    u32x4 o = {0u, 0u, 0u, 0u};
-    if (n0 < N) {
-      const u32x4 v = *reinterpret_cast<const u32x4*>(row + n0);
-      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-      uint32_t r[4];
+  auto emit = [&](int n0, const u32x4& v, const int (&c)[8]) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    uint32_t r[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float lo = ldexpf(to_f32<DT>(static_cast<uint16_t>(w[i] & 0xFFFFu)), em - cexp[n0 + 2 * i]);
-        const float hi = ldexpf(to_f32<DT>(static_cast<uint16_t>(w[i] >> 16)), em - cexp[n0 + 2 * i + 1]);
-        r[i] = static_cast<uint32_t>(f32_to_f16_rne(lo)) | (static_cast<uint32_t>(f32_to_f16_rne(hi)) << 16);
-      }
-      o = u32x4{r[0], r[1], r[2], r[3]};
+    for (int i = 0; i < 4; ++i) {
+      const float lo = ldexpf(to_f32<DT>(static_cast<uint16_t>(w[i] & 0xFFFFu)), em - c[2 * i]);
+      const float hi = ldexpf(to_f32<DT>(static_cast<uint16_t>(w[i] >> 16)), em - c[2 * i + 1]);
+      r[i] = static_cast<uint32_t>(f32_to_f16_rne(lo)) | (static_cast<uint32_t>(f32_to_f16_rne(hi)) << 16);
     }
-    *reinterpret_cast<u32x4*>(arow + n0) = o;
+    *reinterpret_cast<u32x4*>(arow + n0) = u32x4{r[0], r[1], r[2], r[3]};
+  };
+  if (keep) {
+#pragma unroll
+    for (int t = 0; t < kKeep; ++t) {
+      const int n0 = (t * 256 + static_cast<int>(threadIdx.x)) * 8;
+      if (n0 < N) {
+        int c[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) c[i] = heldc[t][i];
+        emit(n0, held[t], c);
+      } else if (n0 < npad) {
+        *reinterpret_cast<u32x4*>(arow + n0) = u32x4{0u, 0u, 0u, 0u};
+      }
+    }
+    // padding columns beyond what the kept slots cover (npad - N < 64)
+    for (int n0 = (kKeep * 256 + static_cast<int>(threadIdx.x)) * 8; n0 < npad; n0 += 256 * 8)
+      *reinterpret_cast<u32x4*>(arow + n0) = u32x4{0u, 0u, 0u, 0u};
+  } else {
+    for (int n0 = threadIdx.x * 8; n0 < npad; n0 += 256 * 8) {
+      if (n0 < N) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(row + n0);
+        int c[8];
+        load_c(n0, c);
+        emit(n0, v, c);
+      } else {
+        *reinterpret_cast<u32x4*>(arow + n0) = u32x4{0u, 0u, 0u, 0u};
+      }
+    }
   }
 }
 
@@ -174,14 +251,15 @@ __device__ inline void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N_ & 0xF) | ((N_ >> 4) << 14) | (0x7 << 4) | (0xF << 8));
 }
 
-// AS: LDS stages of out_grad's tile (2 or 3); the weight tile has two.
-template <int DT, int BITS, int TM, int TB, int AS>
+// Two LDS stages of each tile.
+template <int DT, int BITS, int TM, int TB>
 __global__ __launch_bounds__(512) void grad_gemm_kernel(const GradParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr int NW = 8, WKW = 4;
   constexpr int BMR = 2 * TM * 32;    // rows of the output tile
   constexpr int BKC = WKW * TB * 32;  // columns (k) of the output tile
   constexpr int kABytes = BMR * 128, kBBytes = BKC * 128;
+  constexpr int AS = 2;
   constexpr int kBBase = AS * kABytes;  // the weight stages lie behind out_grad's
   constexpr int kLds = AS * kABytes + 2 * kBBytes;
   constexpr int kALoads = BMR / 64;   // 1 KiB direct-to-LDS loads per wavefront
@@ -335,58 +413,108 @@ __global__ __launch_bounds__(512) void grad_gemm_kernel(const GradParams p) {
       bf[c] = *reinterpret_cast<const u32x4*>(bt + b_off + c * 32 * 128 + (((2 * q + b) ^ b_swz) * 16));
   };
   auto chunk_of = [&](int it) { return it < niter ? it : niter - 1; };  // past the end: the last chunk again
+  auto mfmas = [&](const u32x4 (&af)[TM], const u32x4 (&bf)[TB]) {
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+      for (int c = 0; c < TB; ++c)
+        acc[a][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, af[a]),
+                                                           __builtin_bit_cast(f16x8, bf[c]), acc[a][c], 0, 0, 0);
+  };
 
-  // What is in flight.  While chunk `it` is multiplied, out_grad's tiles up to
-  // chunk it+AS-1 are on their way into LDS, the codes of chunk it+2 are on
-  // their way into registers, and the codes of chunk it+1 (loaded during the
-  // previous chunk) are converted and stored into the other weight tile.
-  // Loads past the last chunk repeat it into places nobody reads any more.
+  // Schedule.  A chunk is four slices of 16 n; operand fragments are read two
+  // slices ahead of their MFMAs, and the one workgroup barrier of a chunk sits
+  // in its middle:
+  //   first half of chunk it:   MFMAs of slices 0, 1; fragments of slices 2, 3
+  //                             are read; the codes of chunk it+1 (in registers
+  //                             since the middle of chunk it-1) are converted
+  //                             and stored into the other weight tile
+  //   middle:                   wait for out_grad's tile of chunk it+1 and for
+  //                             the stores; barrier.  Nobody reads the tiles of
+  //                             chunk it any more (their last fragments are in
+  //                             registers), so out_grad's tile of chunk it+2
+  //                             is requested into the stage of chunk it, and
+  //                             the codes of chunk it+3 into the registers
+  //                             just converted
+  //   second half:              MFMAs of slices 2, 3 while the fragments of
+  //                             slices 0, 1 of chunk it+1 are read
+  // so neither the barrier nor the LDS latency stands between two MFMAs, and
+  // two stages of each tile suffice.  Loads past the last chunk repeat it into
+  // places nobody reads any more.
+  // (With eight MFMAs per slice one slice of lead covers the LDS latency, and
+  // four sets of fragments would not fit the registers: kDeep = false reads
+  // one slice ahead and requests slice 3 just before the barrier.)
+  constexpr bool kDeep = TM * TB < 8;
   Raw raw[2];
+  u32x4 af[kDeep ? 4 : 2][TM], bf[kDeep ? 4 : 2][TB];  // kDeep: the fragments of slice q live in af[q], bf[q]
   issue_a(0);
   load_units(0, raw[0]);
-  if (AS == 3) issue_a(1);
+  issue_a(1);
   load_units(chunk_of(1), raw[1]);
 #pragma unroll
   for (int q = 0; q < 4; ++q) store_quarter(smem + kBBase, raw[0], q / 2, q % 2);
-  // chunk 0 has landed: everything but the loads of chunk 1
-  wait_vmcnt<(AS == 3 ? kALoads : 0) + kCLoads>();
+  load_units(chunk_of(2), raw[0]);
+  wait_vmcnt<0>();
   __builtin_amdgcn_s_waitcnt(0x0070 | (0xF << 0) | (3 << 14));  // lgkmcnt(0)
   __builtin_amdgcn_s_barrier();
+  read_frags(smem, smem + kBBase, af[0], bf[0], 0);
+  if (kDeep) read_frags(smem, smem + kBBase, af[1], bf[1], 1);
 
-  auto chunk = [&](int it, Raw& spare, const Raw& ready) {
-    const unsigned char* at = smem + (it % AS) * kABytes;
+  // conv: the codes of chunk it+1; refilled with those of chunk it+3
+  auto chunk = [&](int it, Raw& conv) {
+    const unsigned char* at = smem + (it & 1) * kABytes;
     const unsigned char* bt = smem + kBBase + (it & 1) * kBBytes;
-    unsigned char* bnext = smem + kBBase + ((it + 1) & 1) * kBBytes;
-    // `spare` held chunk it (converted during the previous chunk)
-    issue_a(it + AS - 1);  // with three stages: the stage last read for chunk it-1
-    load_units(chunk_of(it + 2), spare);
-    __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of everything below
-    u32x4 af[2][TM], bf[2][TB];
-    read_frags(at, bt, af[0], bf[0], 0);
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      if (q < 3) read_frags(at, bt, af[(q + 1) & 1], bf[(q + 1) & 1], q + 1);
-#pragma unroll
-      for (int a = 0; a < TM; ++a)
-#pragma unroll
-        for (int c = 0; c < TB; ++c)
-          acc[a][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, af[q & 1][a]),
-                                                             __builtin_bit_cast(f16x8, bf[q & 1][c]),
-                                                             acc[a][c], 0, 0, 0);
-      // a quarter of the next chunk's weight is converted in the shadow of the matrix pipe
-      store_quarter(bnext, ready, q / 2, q % 2);
+    const unsigned char* an = smem + ((it + 1) & 1) * kABytes;
+    unsigned char* bn = smem + kBBase + ((it + 1) & 1) * kBBytes;
+    if (kDeep) {
+      read_frags(at, bt, af[2], bf[2], 2);
+      mfmas(af[0], bf[0]);
+      store_quarter(bn, conv, 0, 0);
+      store_quarter(bn, conv, 0, 1);
+      read_frags(at, bt, af[3], bf[3], 3);
+      mfmas(af[1], bf[1]);
+      store_quarter(bn, conv, 1, 0);
+      store_quarter(bn, conv, 1, 1);
+    } else {
+      read_frags(at, bt, af[1], bf[1], 1);
+      mfmas(af[0], bf[0]);
+      store_quarter(bn, conv, 0, 0);
+      store_quarter(bn, conv, 0, 1);
+      __builtin_amdgcn_sched_barrier(0);
+      read_frags(at, bt, af[0], bf[0], 2);
+      mfmas(af[1], bf[1]);
+      store_quarter(bn, conv, 1, 0);
+      store_quarter(bn, conv, 1, 1);
+      __builtin_amdgcn_sched_barrier(0);
+      read_frags(at, bt, af[1], bf[1], 3);
     }
-    // out_grad's tile of chunk it+1 has landed (loads issued since may still fly),
-    // this wavefront's stores are done, then the workgroup meets
-    wait_vmcnt<(AS == 3 ? kALoads : 0) + kCLoads>();
+    __builtin_amdgcn_sched_barrier(0);
+    // out_grad's tile of chunk it+1 has landed (the codes requested with it may
+    // still fly), this wavefront's stores and fragment reads are done
+    wait_vmcnt<kCLoads>();
     __builtin_amdgcn_s_waitcnt(0x0070 | (0xF << 0) | (3 << 14));  // lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
+    issue_a(it + 2);
+    load_units(chunk_of(it + 3), conv);
+    __builtin_amdgcn_sched_barrier(0);
+    if (kDeep) {
+      read_frags(an, bn, af[0], bf[0], 0);
+      mfmas(af[2], bf[2]);
+      read_frags(an, bn, af[1], bf[1], 1);
+      mfmas(af[3], bf[3]);
+    } else {
+      mfmas(af[0], bf[0]);
+      __builtin_amdgcn_sched_barrier(0);
+      read_frags(an, bn, af[0], bf[0], 0);
+      mfmas(af[1], bf[1]);
+    }
   };
   for (int it = 0; it < niter; it += 2) {
-    chunk(it, raw[0], raw[1]);
-    if (it + 1 < niter) chunk(it + 1, raw[1], raw[0]);
+    chunk(it, raw[1]);
+    if (it + 1 < niter) chunk(it + 1, raw[0]);
   }
   wait_vmcnt<0>();
+  __builtin_amdgcn_s_waitcnt(0x0070 | (0xF << 0) | (3 << 14));  // the fragments read ahead have arrived
   __builtin_amdgcn_s_barrier();  // the spare loads are done and every wavefront has stopped reading
 
   // ---- epilogue: 2^-e[m], cast, 32-row slabs leave through LDS as 16-byte stores
@@ -439,14 +567,14 @@ __global__ __launch_bounds__(512) void grad_gemm_kernel(const GradParams p) {
 #endif
 }
 
-template <int DT, int BITS, int TM, int TB, int AS>
+template <int DT, int BITS, int TM, int TB>
 void launch_cfg(const GradParams& p0, hipStream_t stream) {
   GradParams p = p0;
   constexpr int BMR = 2 * TM * 32, BKC = 4 * TB * 32;
   p.nbm = (p.M + BMR - 1) / BMR;
   p.nbk = (p.K + BKC - 1) / BKC;
-  const size_t lds = static_cast<size_t>(AS * BMR + 2 * BKC) * 128;
-  auto kern = grad_gemm_kernel<DT, BITS, TM, TB, AS>;
+  const size_t lds = static_cast<size_t>(2 * BMR + 2 * BKC) * 128;
+  auto kern = grad_gemm_kernel<DT, BITS, TM, TB>;
   // more than 64 KiB of LDS must be allowed once per device
   static std::atomic<uint32_t> done{0};
   int dev = 0;
@@ -477,10 +605,10 @@ template <int DT, int BITS>
 void launch_gemm(const GradParams& p, hipStream_t stream) {
   int tm, tb;
   pick_tile(p.M, p.K, &tm, &tb);
-  if (tm == 4 && tb == 2) launch_cfg<DT, BITS, 4, 2, 2>(p, stream);
-  else if (tm == 4) launch_cfg<DT, BITS, 4, 1, 3>(p, stream);
-  else if (tb == 2) launch_cfg<DT, BITS, 2, 2, 3>(p, stream);
-  else launch_cfg<DT, BITS, 2, 1, 3>(p, stream);
+  if (tm == 4 && tb == 2) launch_cfg<DT, BITS, 4, 2>(p, stream);
+  else if (tm == 4) launch_cfg<DT, BITS, 4, 1>(p, stream);
+  else if (tb == 2) launch_cfg<DT, BITS, 2, 2>(p, stream);
+  else launch_cfg<DT, BITS, 2, 1>(p, stream);
 }
 
 struct Layout {
@@ -526,12 +654,22 @@ int launch_linear_grad(const void* out_grad, const void* codes, const void* scal
   const uint16_t* sc = static_cast<const uint16_t*>(scale);
   const uint16_t* dout = static_cast<const uint16_t*>(out_grad);
   const dim3 sgrid(static_cast<unsigned>((N + 255) / 256)), pgrid(static_cast<unsigned>(M));
+  const int n32 = static_cast<int>(N), np32 = static_cast<int>(l.npad);
+  const bool one = l.groups == 1;  // per-channel: the scale preparation rides along with the rows
   if (dtype == WOL_DTYPE_BF16) {
-    grad_scales_kernel<WOL_DTYPE_BF16><<<sgrid, 256, 0, stream>>>(sc, static_cast<int>(l.groups), static_cast<int>(N), sp, cexp);
-    grad_prepare_kernel<WOL_DTYPE_BF16><<<pgrid, 256, 0, stream>>>(dout, cexp, static_cast<int>(N), static_cast<int>(l.npad), a, rowf);
+    if (one) {
+      grad_prepare_kernel<WOL_DTYPE_BF16, true><<<pgrid, 256, 0, stream>>>(dout, cexp, sc, sp, n32, np32, a, rowf);
+    } else {
+      grad_scales_kernel<WOL_DTYPE_BF16><<<sgrid, 256, 0, stream>>>(sc, static_cast<int>(l.groups), n32, sp, cexp);
+      grad_prepare_kernel<WOL_DTYPE_BF16, false><<<pgrid, 256, 0, stream>>>(dout, cexp, sc, sp, n32, np32, a, rowf);
+    }
   } else {
-    grad_scales_kernel<WOL_DTYPE_F16><<<sgrid, 256, 0, stream>>>(sc, static_cast<int>(l.groups), static_cast<int>(N), sp, cexp);
-    grad_prepare_kernel<WOL_DTYPE_F16><<<pgrid, 256, 0, stream>>>(dout, cexp, static_cast<int>(N), static_cast<int>(l.npad), a, rowf);
+    if (one) {
+      grad_prepare_kernel<WOL_DTYPE_F16, true><<<pgrid, 256, 0, stream>>>(dout, cexp, sc, sp, n32, np32, a, rowf);
+    } else {
+      grad_scales_kernel<WOL_DTYPE_F16><<<sgrid, 256, 0, stream>>>(sc, static_cast<int>(l.groups), n32, sp, cexp);
+      grad_prepare_kernel<WOL_DTYPE_F16, false><<<pgrid, 256, 0, stream>>>(dout, cexp, sc, sp, n32, np32, a, rowf);
+    }
   }
   GradParams p;
   p.a = a;
