@@ -30,6 +30,10 @@
  *     multiary.cc:5495-5575); the PHI glue turns a non-zero status into
  *     PADDLE_THROW(InvalidArgument / External).
  *   - Thread-safe and re-entrant: no mutable global state.
+ *   - WOL_LOG=1 in the environment makes wol_linear, wol_linear_fused and
+ *     wol_linear_grad write one line per call to stderr (the problem and the
+ *     kernel taken), the way the reference's VLOG lines name the GEMV/GEMM
+ *     branch (gpu/weight_only_linear_kernel.cu:60-200).  Read once per process.
  */
 #ifndef WOL_C_API_H_
 #define WOL_C_API_H_

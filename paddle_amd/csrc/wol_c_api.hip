@@ -4,6 +4,8 @@
 #include <atomic>
 #include <cstring>
 
+#include <stdlib.h>
+
 #include "wol_common.h"
 #include "wol_diag.h"
 
@@ -117,6 +119,16 @@ int resolve_kernel(int kernel, int64_t M, int64_t K, int64_t N, int bits, int gr
   return use_stream(M, K, N, bits, have_ws) ? WOL_KERNEL_STREAM : WOL_KERNEL_GEMM;
 }
 
+// WOL_LOG=1 in the environment: every compute call writes one line to stderr
+// (entry point, problem, the kernel taken).  Read once.
+bool log_enabled() {
+  static const bool on = [] {
+    const char* e = getenv("WOL_LOG");
+    return e != nullptr && e[0] != '\0' && e[0] != '0';
+  }();
+  return on;
+}
+
 int linear_impl(const void* x, const void* codes, const void* bias, const void* scale, int dtype,
                 int64_t M, int64_t K, int64_t N, int bits, int group_size, void* out, bool out_f32,
                 int kernel, void* workspace, size_t workspace_bytes, void* stream,
@@ -138,6 +150,12 @@ int linear_impl(const void* x, const void* codes, const void* bias, const void* 
   if (workspace == nullptr || !aligned16(workspace)) workspace_bytes = 0;  // optional: only speeds up
   const bool have_ws = workspace_bytes / sizeof(float) / 2 >= static_cast<size_t>(M) * static_cast<size_t>(N);
   const int which = resolve_kernel(kernel, M, K, N, bits, group_size, have_ws);
+  if (log_enabled())
+    fprintf(stderr, "[wol] linear M=%lld K=%lld N=%lld int%d group=%d %s%s%s act=%d -> %s kernel\n",
+            static_cast<long long>(M), static_cast<long long>(K), static_cast<long long>(N), bits, group_size,
+            dtype == WOL_DTYPE_BF16 ? "bf16" : "f16", bias != nullptr ? " bias" : "",
+            fuse.pre_scale != nullptr ? " pre_scale" : "", fuse.act,
+            which == WOL_KERNEL_BATCH ? "batch" : (which == WOL_KERNEL_STREAM ? "stream" : "gemm"));
   if (which == WOL_KERNEL_BATCH)
     return wol::launch_linear_batch(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out,
                                     out_f32, s, fuse);
@@ -362,6 +380,10 @@ int linear_grad_impl(const void* out_grad, const void* codes, const void* scale,
     return WOL_ERR_WORKSPACE;
   if (!aligned16(workspace)) return WOL_ERR_ALIGNMENT;
   if (const int dv = require_gfx950(); dv != WOL_OK) return dv;
+  if (log_enabled())
+    fprintf(stderr, "[wol] linear_grad M=%lld K=%lld N=%lld int%d group=%d %s\n", static_cast<long long>(M),
+            static_cast<long long>(K), static_cast<long long>(N), bits, group_size,
+            dtype == WOL_DTYPE_BF16 ? "bf16" : "f16");
   return wol::launch_linear_grad(out_grad, codes, scale, dtype, M, K, N, bits, group_size, x_grad, out_f32,
                                  workspace, static_cast<hipStream_t>(stream));
 }

@@ -284,6 +284,50 @@ def test_baseline_config_5_int8_group64(G, oracle, shape):
     check(G, oracle, H.BF16, 8, 64, M, K, N if M < 64 else N, bias=False, seed=1234)
 
 
+def test_baseline_config_5_as_a_sequence(device, oracle):
+    # Configuration 5 the way it runs: the four linears of consecutive decoder
+    # layers (int8, group 64, bf16, full K and N, every layer its own weights)
+    # as a decode step at 8 rows, then one prefill chunk of 1024 rows, then the
+    # decode step again, all enqueued back to back on one stream.  Every output
+    # is checked against the oracle on its first columns (the quantiser and the
+    # linear are column-wise, so a column slice of the oracle is exact), and the
+    # two decode steps must agree bit for bit: nothing carries over between calls.
+    import torch
+    from paddle_amd.nn import quant as Q
+
+    dt, g, cols = H.BF16, 64, 128
+    shapes = [(4096, 12288), (4096, 4096), (4096, 22016), (11008, 4096)]
+    gen = torch.Generator(device="cuda").manual_seed(55)
+    layers = []
+    for layer in range(2):
+        for K, N in shapes:
+            w = (torch.randn(K, N, device="cuda", generator=gen) * 0.02).to(torch.bfloat16)
+            codes, scale = Q.weight_quantize(w, algo="weight_only_int8", group_size=g)
+            layers.append((K, N, H.torch_to_bits(w[:, :cols].contiguous()), codes, scale))
+            del w
+    xs = {(M, K): (torch.randn(M, K, device="cuda", generator=gen)).to(torch.bfloat16)
+          for M in (8, 1024) for K in (4096, 11008)}
+
+    def step(M):
+        return [Q.weight_only_linear(xs[(M, K)], codes, None, scale, "int8", None, g) for K, N, _, codes, scale in layers]
+
+    d1 = step(8)
+    pf = step(1024)
+    d2 = step(8)
+    torch.cuda.synchronize()
+    for i, (K, N, wb, codes, scale) in enumerate(layers):
+        oc, osc = oracle.weight_quantize(wb, dt, 8, g)
+        assert np.array_equal(H.torch_to_bits(scale[:, :cols].contiguous()), osc)
+        for M, outs in ((8, d1), (1024, pf)):
+            rows = 64 if M > 64 else M  # the oracle is scalar code
+            xb = H.torch_to_bits(xs[(M, K)][:rows].contiguous())
+            _, wantT = oracle.linear(xb, oc, osc, None, dt, 8, g)
+            got = H.bits_to_f32(H.torch_to_bits(outs[i][:rows, :cols].contiguous()), dt)
+            err = H.rel_l2(got, H.bits_to_f32(wantT, dt))
+            assert err <= TOL, (err, i, M, K, N)
+        assert torch.equal(d1[i], d2[i]), (i, K, N)
+
+
 # ---- full-size properties (no oracle needed: size-independent identities) ----
 def _full_size_properties(dt, bits, g, M, K, N, outliers=0.0):
     import torch
@@ -489,3 +533,29 @@ def test_gemm_partial_last_round_split(G, oracle, dt, bits, g, M, K, N):
     rows = np.r_[0:3, M - 3:M]
     r32, _ = oracle.linear(xb[rows], oc, osc, bb, dt, bits, g)
     assert H.rel_l2(split32[rows], r32) < 2e-5
+
+
+def test_call_log_names_the_kernel(device):
+    # WOL_LOG=1: one line per call on stderr with the problem and the kernel taken
+    # (read once per process, hence a child process)
+    import os
+    import subprocess
+    import sys
+
+    code = (
+        "import torch\n"
+        "from paddle_amd.nn import quant as Q\n"
+        "w = (torch.randn(2048, 8192, device='cuda') * 0.02).to(torch.bfloat16)\n"
+        "c, s = Q.weight_quantize(w, algo='weight_only_int8')\n"
+        "for M in (1, 8, 300):\n"
+        "    Q.weight_only_linear(torch.randn(M, 2048, device='cuda').to(torch.bfloat16), c, None, s, 'int8')\n"
+        "torch.cuda.synchronize()\n"
+    )
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-c", code], env=dict(os.environ, WOL_LOG="1", PYTHONPATH=root),
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [ln for ln in r.stderr.splitlines() if ln.startswith("[wol] linear ")]
+    assert len(lines) == 3
+    assert "M=1 K=2048 N=8192 int8" in lines[0] and lines[0].endswith("-> stream kernel")
+    assert lines[1].endswith("-> batch kernel") and lines[2].endswith("-> gemm kernel")
