@@ -415,6 +415,60 @@ def test_calls_replay_correctly_from_a_hip_graph(device):
             assert torch.equal(a, b), rep
 
 
+def test_fused_grad_moe_and_batched_decode_replay_from_a_hip_graph(device):
+    # the same for the batched decode kernel, the fused linear (pre-scale folded
+    # into the loads, gelu, swiglu through its pass), weight_only_linear_grad
+    # (its prepare launches and the GEMM) and the MoE expert FFN (table built on
+    # the device): replayed three times with eager work in between
+    import torch
+    from paddle_amd.nn import quant as Q
+    from paddle_amd.nn.quant import quantized_linear as QL
+
+    dev = torch.device("cuda:0")
+    K, N = 2048, 8192
+    gen = torch.Generator(device="cuda").manual_seed(4)
+    w = (torch.randn(K, N, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+    codes, scale = Q.weight_quantize(w, algo="weight_only_int8", group_size=64)
+    c4, s4 = Q.weight_quantize(w, algo="weight_only_int4", group_size=-1)
+    xs = {M: torch.randn(M, K, device=dev, generator=gen).to(torch.bfloat16) for M in (1, 8, 200)}
+    pre = (0.5 + torch.rand(K, device=dev, generator=gen)).to(torch.bfloat16)
+    gos = {M: torch.randn(M, N, device=dev, generator=gen).to(torch.bfloat16) for M in (8, 300)}
+    E, hidden, inter = 4, 256, 512
+    w1 = (torch.randn(E, hidden, inter, device=dev, generator=gen) * 0.05).to(torch.bfloat16)
+    w2 = (torch.randn(E, inter // 2, hidden, device=dev, generator=gen) * 0.05).to(torch.bfloat16)
+    q1, s1 = Q.moe_quantize_experts(w1)
+    q2, s2 = Q.moe_quantize_experts(w2)
+    tokens = torch.randn(300, hidden, device=dev, generator=gen).to(torch.bfloat16)
+    cum = torch.tensor([40, 40, 171, 300], dtype=torch.int64, device=dev)
+
+    def work():
+        outs = [Q.weight_only_linear(xs[8], codes, None, scale, "int8", None, 64)]  # batched decode kernel
+        for M, x in xs.items():
+            outs.append(Q.weight_only_linear_fused(x, codes, None, scale, "int8", 64, pre_scale=pre, act="gelu"))
+            outs.append(Q.weight_only_linear_fused(x, c4, None, s4, "int4", -1, pre_scale=None, act="swiglu"))
+        for M, go in gos.items():
+            x_like = torch.empty((M, K), dtype=go.dtype, device="meta")
+            outs.append(QL.weight_only_linear_grad(x_like, codes, None, scale, go, "int8", None, 64))
+            outs.append(QL.weight_only_linear_grad(x_like, c4, None, s4, go, "int4", None, -1))
+        outs.append(Q.moe_ffn(tokens, cum, q1, q2, None, s1, s2, "weight_only_int8"))
+        return outs
+
+    eager = [t.clone() for t in work()]
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        captured = work()
+    for rep in range(3):
+        for t in captured:
+            t.zero_()
+        _ = work()  # eager work between the replays
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for i, (a, b) in enumerate(zip(eager, captured)):
+            assert torch.equal(a, b), (rep, i)
+
+
 def test_weight_larger_than_2_gib(device):
     # byte offsets beyond 2^31: a 8192 x 327680 int8 weight (2.7 GB of codes).
     # One-hot activations must read back the dequantised rows, also at the far
