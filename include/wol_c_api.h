@@ -166,9 +166,12 @@ size_t wol_linear_workspace(int64_t M, int64_t K, int64_t N, int bits,
  * fp32 accumulation, one round-to-nearest-even cast to T at the end.
  * codes must be in GFX950 layout.  bias may be NULL.
  * scale: [N] T (group_size -1) or [ceil(K/g),N] T, as wol_quantize wrote it.
- * M <= 16 takes a streaming (HBM-bound) kernel, M > 64 the MFMA GEMM, and in
- * between whichever a cost model of the two predicts to be faster; the
- * reference's split is M <= 3 (gpu/weight_only_linear_kernel.cu:60-61).
+ * M <= 16 takes a decode (HBM-bound) kernel -- the batched one, which fetches
+ * the activations once per workgroup, where it applies (2 to 16 rows, K =
+ * 2048/4096/8192, at least two 16-column strips per CU), else the streaming
+ * one --, M > 64 the MFMA GEMM, and in between the streaming kernel or the
+ * GEMM, whichever a cost model predicts to be faster; the reference's split
+ * is M <= 3 (gpu/weight_only_linear_kernel.cu:60-61).
  * x, codes and scale must be 16-byte aligned.
  */
 int wol_linear(const void* x, const void* codes, const void* bias,

@@ -59,7 +59,9 @@ bool layout_ok(int layout) {
 // the weights best, but every 16-column strip re-reads its activations from
 // L2; the MFMA GEMM shares them through LDS at the price of a second launch
 // that adds the K runs.  Up to 16 rows the streaming kernel won every shape
-// measured (K and N from 4096 to 28672, both bit widths); from 17 to 64 rows
+// measured against the GEMM (K and N from 4096 to 28672, both bit widths; the
+// batched decode kernel, where it applies, is chosen before either, see
+// use_batch); from 17 to 64 rows
 // the cheaper of the two by a linear cost model runs (microseconds, least
 // squares over those measurements on MI355X; it picks the slower kernel in 2
 // of 96 cases, by 16 %).

@@ -559,7 +559,7 @@ void launch_wk(const Args& a, int wk, int nu) {
     else launch_one<DT, BITS, MP, MT, 1, 1>(a);
   } else {
     // 16 wavefronts (1024 threads) leave 128 registers each: enough for the
-    // double-buffered units of 2 to 8 rows, not for the others
+    // ring of units of 2 to 8 rows (and of one row of int4), not for the others
     if constexpr ((MP >= 2 && MP <= 8) || (MP == 1 && BITS == 4)) {
       if (wk >= 16) { launch_one<DT, BITS, MP, MT, 16, 0>(a); return; }
     }

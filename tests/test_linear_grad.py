@@ -186,3 +186,55 @@ def test_linear_grad_argument_checks():
     assert L.wol_linear_grad(None, None, None, 0, 4, 65, 16, 8, -1, None, None, 0, None) == 5
     assert L.wol_linear_grad(None, None, None, 0, 0, 64, 16, 8, -1, None, None, 0, None) == 0  # nothing to do
     assert L.wol_linear_grad(None, None, None, 0, 4, 64, 16, 8, -1, None, None, 0, None) == 1
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", [(2048, 4096, 4096, 8, -1, H.BF16), (8192, 4096, 4096, 4, 64, H.BF16),
+                                  (512, 8192, 8192, 4, 128, H.F16), (1000, 11008, 4096, 8, 64, H.F16)])
+def test_linear_grad_full_size_is_the_adjoint_of_the_linear(device, case):
+    # at the benchmark's sizes, where the oracle would take minutes: for any x and
+    # g, <linear(x), g> = <x, linear_grad(g)> (both sides through the fp32
+    # outputs of the two kernels, summed in float64).  A wrong tile, a dropped
+    # chunk of N or a mis-indexed scale group breaks the identity; the fp16
+    # rounding of code * scale in the grad kernel leaves about 1e-4.
+    import torch
+    from paddle_amd import _lib
+    from paddle_amd.nn import quant as Q
+
+    M, K, N, bits, g, dt = case
+    tdt = H.torch_dtype(dt)
+    gen = torch.Generator(device="cuda").manual_seed(M + K)
+    w = (torch.randn(K, N, device="cuda", generator=gen) * 0.02).to(tdt)
+    codes, scale = Q.weight_quantize(w, algo="weight_only_int8" if bits == 8 else "weight_only_int4", group_size=g)
+    del w
+    x = torch.randn(M, K, device="cuda", generator=gen).to(tdt)
+    go = torch.randn(M, N, device="cuda", generator=gen).to(tdt)
+    L = _lib.lib
+    y32 = torch.empty(M, N, device="cuda", dtype=torch.float32)
+    wsb = L.wol_linear_workspace(M, K, N, bits, g)
+    ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device="cuda")
+    _lib.check(L.wol_linear_f32(x.data_ptr(), codes.data_ptr(), None, scale.data_ptr(), dt, M, K, N, bits, g,
+                                y32.data_ptr(), ws.data_ptr() if wsb else None, wsb, None))
+    gx32 = torch.empty(M, K, device="cuda", dtype=torch.float32)
+    gsb = L.wol_linear_grad_workspace(M, K, N, bits, g)
+    gws = torch.empty(gsb, dtype=torch.uint8, device="cuda")
+    _lib.check(L.wol_linear_grad_f32(go.data_ptr(), codes.data_ptr(), scale.data_ptr(), dt, M, K, N, bits, g,
+                                     gx32.data_ptr(), gws.data_ptr(), gsb, None))
+    torch.cuda.synchronize()
+    # row by row (every row of the batch has its own normaliser in the grad
+    # kernel), measured against the size of the terms: the inner products
+    # themselves are sums of random signs and may come out near zero
+    lhs = (y32.double() * go.double()).sum(dim=1)
+    rhs = (x.double() * gx32.double()).sum(dim=1)
+    size = y32.double().norm(dim=1) * go.double().norm(dim=1)
+    rel = ((lhs - rhs).abs() / size).max().item()
+    print("adjoint mismatch", case, rel, flush=True)
+    # the grad kernel's 1.7e-4 per element averages down by sqrt(N) in the inner
+    # product (measured 3e-6 .. 1e-5); one missing chunk of 64 columns would read 2e-3
+    assert rel <= 1e-4, rel
+    # and the T output is the cast of the fp32 one
+    gxT = torch.empty(M, K, device="cuda", dtype=tdt)
+    _lib.check(L.wol_linear_grad(go.data_ptr(), codes.data_ptr(), scale.data_ptr(), dt, M, K, N, bits, g,
+                                 gxT.data_ptr(), gws.data_ptr(), gsb, None))
+    torch.cuda.synchronize()
+    assert torch.equal(gxT, gx32.to(tdt))
