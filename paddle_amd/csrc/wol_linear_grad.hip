@@ -48,6 +48,7 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4v __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 constexpr int kChunk = 64;  // n per step of the contraction
@@ -217,6 +218,8 @@ struct GradParams {
   int M, K, N, npad;
   int gshift;            // log2(group size), -1: one scale row
   int nbm, nbk;          // output tiles along m and k
+  int nsplit, chunks_per_split;  // N is cut into nsplit runs of chunks, one workgroup each
+  float* partial;        // nsplit > 1: [nsplit][M][K] sums (times 2^-e[m]) of the runs
 };
 
 // Every load (direct-to-LDS ones included) and LDS store of the wavefront has
@@ -271,11 +274,15 @@ __global__ __launch_bounds__(512) void grad_gemm_kernel(const GradParams p) {
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WKW, wk = wave % WKW;
   const int j = lane & 15, kb = lane >> 4, b = lane >> 5, r32 = lane & 31;
-  const int bm = blockIdx.x % p.nbm, bk = blockIdx.x / p.nbm;
+  const int ntiles = p.nbm * p.nbk;
+  const int split = blockIdx.x / ntiles, tile = blockIdx.x - split * ntiles;
+  const int bm = tile % p.nbm, bk = tile / p.nbm;
   const int m0 = bm * BMR, k0 = bk * BKC;
   const int M = p.M, K = p.K, N = p.N;
   const int nstrips = N / kStripCols;
-  const int niter = p.npad / kChunk;
+  // this workgroup's run of chunks
+  const int cbase = split * p.chunks_per_split;
+  const int niter = (p.npad / kChunk - cbase) < p.chunks_per_split ? (p.npad / kChunk - cbase) : p.chunks_per_split;
 
   // ---- out_grad's tile: sources of this lane's direct-to-LDS loads
   const uint16_t* asrc[kALoads];
@@ -347,7 +354,7 @@ __global__ __launch_bounds__(512) void grad_gemm_kernel(const GradParams p) {
   // last one is fetched again (into a stage nobody reads any more)
   auto issue_a = [&](int it) {
     unsigned char* stage = smem + (it % AS) * kABytes;
-    const int src = it < niter ? it : niter - 1;
+    const int src = cbase + (it < niter ? it : niter - 1);
 #pragma unroll
     for (int c = 0; c < kALoads; ++c)
       __builtin_amdgcn_global_load_lds(asrc[c] + src * kChunk, (lds_ptr_t)(stage + (c * NW + wave) * 1024), 16, 0, 0);
@@ -412,7 +419,7 @@ __global__ __launch_bounds__(512) void grad_gemm_kernel(const GradParams p) {
     for (int c = 0; c < TB; ++c)
       bf[c] = *reinterpret_cast<const u32x4*>(bt + b_off + c * 32 * 128 + (((2 * q + b) ^ b_swz) * 16));
   };
-  auto chunk_of = [&](int it) { return it < niter ? it : niter - 1; };  // past the end: the last chunk again
+  auto chunk_of = [&](int it) { return cbase + (it < niter ? it : niter - 1); };  // past the end: the last chunk again
   auto mfmas = [&](const u32x4 (&af)[TM], const u32x4 (&bf)[TB]) {
 #pragma unroll
     for (int a = 0; a < TM; ++a)
@@ -448,7 +455,7 @@ __global__ __launch_bounds__(512) void grad_gemm_kernel(const GradParams p) {
   Raw raw[2];
   u32x4 af[kDeep ? 4 : 2][TM], bf[kDeep ? 4 : 2][TB];  // kDeep: the fragments of slice q live in af[q], bf[q]
   issue_a(0);
-  load_units(0, raw[0]);
+  load_units(chunk_of(0), raw[0]);
   issue_a(1);
   load_units(chunk_of(1), raw[1]);
 #pragma unroll
@@ -520,8 +527,8 @@ __global__ __launch_bounds__(512) void grad_gemm_kernel(const GradParams p) {
   // ---- epilogue: 2^-e[m], cast, 32-row slabs leave through LDS as 16-byte stores
   // accumulator element r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its block
   const int col0 = k0 + wk * TB * 32;
-  if (p.out_f32) {  // verification mode: the sums before the cast, plain stores
-    float* outf = static_cast<float*>(p.out);
+  if (p.out_f32 || p.nsplit > 1) {  // fp32 results (verification mode) or the sums of this run: plain stores
+    float* outf = p.nsplit > 1 ? p.partial + static_cast<int64_t>(split) * M * K : static_cast<float*>(p.out);
 #pragma unroll
     for (int a = 0; a < TM; ++a)
 #pragma unroll
@@ -567,6 +574,34 @@ __global__ __launch_bounds__(512) void grad_gemm_kernel(const GradParams p) {
 #endif
 }
 
+// out[i] = T(sum over the runs of part[run][i]) (or the fp32 sum), eight elements per thread.
+template <int DT>
+__global__ __launch_bounds__(256) void reduce_runs_kernel(const float* __restrict__ part, int runs, int64_t total,
+                                                          void* __restrict__ out, int out_f32) {
+  const int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 8;  // total is a multiple of 64
+  if (i >= total) return;
+  float v[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = 0.0f;
+  for (int r = 0; r < runs; ++r) {  // in run order: the result does not depend on timing
+    const float* src = part + static_cast<int64_t>(r) * total + i;
+    const f32x4v a = *reinterpret_cast<const f32x4v*>(src), b2 = *reinterpret_cast<const f32x4v*>(src + 4);
+    v[0] += a.x; v[1] += a.y; v[2] += a.z; v[3] += a.w;
+    v[4] += b2.x; v[5] += b2.y; v[6] += b2.z; v[7] += b2.w;
+  }
+  if (out_f32) {
+    float* o = static_cast<float*>(out) + i;
+    *reinterpret_cast<f32x4v*>(o) = f32x4v{v[0], v[1], v[2], v[3]};
+    *reinterpret_cast<f32x4v*>(o + 4) = f32x4v{v[4], v[5], v[6], v[7]};
+  } else {
+    uint32_t r[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      r[e] = static_cast<uint32_t>(cast_out<DT>(v[2 * e])) | (static_cast<uint32_t>(cast_out<DT>(v[2 * e + 1])) << 16);
+    *reinterpret_cast<u32x4*>(static_cast<uint16_t*>(out) + i) = u32x4{r[0], r[1], r[2], r[3]};
+  }
+}
+
 template <int DT, int BITS, int TM, int TB>
 void launch_cfg(const GradParams& p0, hipStream_t stream) {
   GradParams p = p0;
@@ -585,7 +620,22 @@ void launch_cfg(const GradParams& p0, hipStream_t stream) {
                               static_cast<int>(lds));
     done.fetch_or(bit, std::memory_order_release);
   }
-  kern<<<dim3(static_cast<unsigned>(p.nbm * p.nbk)), dim3(512), lds, stream>>>(p);
+  // Few tiles: N is cut into runs so that the CUs fill (a chunk costs a workgroup
+  // about the same time whatever the tile, so a run of half the chunks takes
+  // half as long); the runs' fp32 sums meet in reduce_runs_kernel.
+  const int tiles = p.nbm * p.nbk, chunks = p.npad / kChunk;
+  int ns = 1;
+  if (p.partial != nullptr) {
+    while (ns < 4 && tiles * ns * 2 <= 256 && chunks / (ns * 2) >= 8) ns *= 2;
+  }
+  p.chunks_per_split = (chunks + ns - 1) / ns;
+  p.nsplit = (chunks + p.chunks_per_split - 1) / p.chunks_per_split;
+  kern<<<dim3(static_cast<unsigned>(tiles * p.nsplit)), dim3(512), lds, stream>>>(p);
+  if (p.nsplit > 1) {
+    const int64_t total = static_cast<int64_t>(p.M) * p.K;
+    reduce_runs_kernel<DT><<<dim3(static_cast<unsigned>((total / 8 + 255) / 256)), dim3(256), 0, stream>>>(
+        p.partial, p.nsplit, total, p.out, p.out_f32);
+  }
 }
 
 // Tile choice.  Every element of the weight is converted once per row tile, so
@@ -612,9 +662,17 @@ void launch_gemm(const GradParams& p, hipStream_t stream) {
 }
 
 struct Layout {
-  size_t sp, cexp, rowf, a, total;
+  size_t sp, cexp, rowf, a, partial, total;
   int64_t npad, groups;
 };
+
+// Runs of N the GEMM may use for a problem (the scratch is sized for it).
+int max_runs(int64_t M, int64_t K) {
+  int tm, tb;
+  pick_tile(M, K, &tm, &tb);
+  const int64_t tiles = ((M + 64 * tm - 1) / (64 * tm)) * ((K + 128 * tb - 1) / (128 * tb));
+  return tiles * 2 <= 256 ? (tiles * 4 <= 256 ? 4 : 2) : 1;
+}
 
 Layout layout_of(int64_t M, int64_t K, int64_t N, int group_size) {
   Layout l;
@@ -624,7 +682,9 @@ Layout layout_of(int64_t M, int64_t K, int64_t N, int group_size) {
   l.cexp = round_up(static_cast<size_t>(l.groups) * N * 2, 256);
   l.rowf = l.cexp + round_up(static_cast<size_t>(N) * 4, 256);
   l.a = l.rowf + round_up(static_cast<size_t>(M) * 4, 256);
-  l.total = l.a + round_up(static_cast<size_t>(M) * l.npad * 2, 256);
+  l.partial = l.a + round_up(static_cast<size_t>(M) * l.npad * 2, 256);
+  const int runs = max_runs(M, K);
+  l.total = l.partial + (runs > 1 ? round_up(static_cast<size_t>(runs) * M * K * 4, 256) : 0);
   return l;
 }
 
@@ -637,9 +697,12 @@ size_t linear_grad_workspace(int64_t M, int64_t K, int64_t N, int group_size) {
 void describe_linear_grad(int64_t M, int64_t K, int64_t N, char* buf, size_t n) {
   int tm, tb;
   pick_tile(M, K, &tm, &tb);
-  snprintf(buf, n, "wol::grad_gemm_kernel: %d rows x %d columns (k) per workgroup, N in chunks of %d",
-           64 * tm, 128 * tb, kChunk);
-  (void)N;
+  const int64_t tiles = ((M + 64 * tm - 1) / (64 * tm)) * ((K + 128 * tb - 1) / (128 * tb));
+  const int64_t chunks = round_up(N, kChunk) / kChunk;
+  int ns = 1;
+  while (ns < 4 && tiles * ns * 2 <= 256 && chunks / (ns * 2) >= 8) ns *= 2;
+  snprintf(buf, n, "wol::grad_gemm_kernel: %d rows x %d columns (k) per workgroup, N in chunks of %d%s",
+           64 * tm, 128 * tb, kChunk, ns == 1 ? "" : (ns == 2 ? ", in 2 runs + reduce_runs_kernel" : ", in 4 runs + reduce_runs_kernel"));
 }
 
 int launch_linear_grad(const void* out_grad, const void* codes, const void* scale, int dtype, int64_t M,
@@ -684,6 +747,9 @@ int launch_linear_grad(const void* out_grad, const void* codes, const void* scal
   p.npad = static_cast<int>(l.npad);
   p.gshift = group_size == 64 ? 6 : (group_size == 128 ? 7 : -1);
   p.nbm = p.nbk = 0;
+  p.nsplit = 1;
+  p.chunks_per_split = 0;
+  p.partial = max_runs(M, K) > 1 ? reinterpret_cast<float*>(ws + l.partial) : nullptr;
   if (dtype == WOL_DTYPE_BF16) {
     if (bits == 8) launch_gemm<WOL_DTYPE_BF16, 8>(p, stream); else launch_gemm<WOL_DTYPE_BF16, 4>(p, stream);
   } else {

@@ -88,8 +88,10 @@ def _case(oracle, dt, bits, g, M, K, N, seed=0, gstd=1.0):
 
 # every tile shape of the kernel (by the number of output tiles), N that is and
 # is not a multiple of the 64-column chunk, M off the tile height, K off the
-# tile width and, for int4, a K that ends in a half tile
-SHAPES = [(24, 512, 256), (1, 64, 16), (130, 192, 48), (300, 1088, 144), (1000, 2048, 512), (2100, 4096, 320)]
+# tile width and, for int4, a K that ends in a half tile; the last two have few
+# tiles and a long N, which the kernel cuts into four and two runs
+SHAPES = [(24, 512, 256), (1, 64, 16), (130, 192, 48), (300, 1088, 144), (1000, 2048, 512), (2100, 4096, 320),
+          (100, 256, 2048), (500, 512, 1040)]
 
 
 @pytest.mark.gpu
