@@ -235,7 +235,9 @@ int wol_linear_fused(const void* x, const void* pre_scale, const void* codes,
  * the sums are kept in fp32.  No bias and no activations are involved (x is
  * no_need_buffer in the reference).
  * codes: GFX950 layout.  scale: as for wol_linear.  The workspace holds the
- * scaled out_grad and scales; wol_linear_grad_workspace() bytes are required.
+ * scaled out_grad and scales (and, for M <= 512 or so, the sums of the runs N
+ * is cut into); wol_linear_grad_workspace() bytes are required.  out_grad,
+ * codes, scale, x_grad and the workspace must be 16-byte aligned.
  */
 size_t wol_linear_grad_workspace(int64_t M, int64_t K, int64_t N, int bits,
                                  int group_size);

@@ -377,7 +377,7 @@ int linear_grad_impl(const void* out_grad, const void* codes, const void* scale,
   if (M < 0 || M > (int64_t{1} << 24)) return WOL_ERR_BAD_SHAPE;
   if (M == 0) return WOL_OK;
   if (out_grad == nullptr || codes == nullptr || scale == nullptr || x_grad == nullptr) return WOL_ERR_NULL_POINTER;
-  if (!aligned16(out_grad) || !aligned16(codes) || !aligned16(x_grad)) return WOL_ERR_ALIGNMENT;
+  if (!aligned16(out_grad) || !aligned16(codes) || !aligned16(scale) || !aligned16(x_grad)) return WOL_ERR_ALIGNMENT;
   if (workspace == nullptr || workspace_bytes < wol::linear_grad_workspace(M, K, N, group_size))
     return WOL_ERR_WORKSPACE;
   if (!aligned16(workspace)) return WOL_ERR_ALIGNMENT;
