@@ -974,51 +974,62 @@ inline int plan_big_columns(int M, int N) {
 }
 
 // Rows up to which the small-M configurations (one row block of 32 or 64
-// rows, 256 columns, K split across workgroups) are used.  They run two
-// stages deep instead of three: the smaller LDS footprint lets a third (32
-// rows) or second (64 rows, int4) workgroup share the CU, which hides more
+// rows, K split across workgroups) are used.  They run two stages deep
+// instead of three: the smaller LDS footprint lets a third (32 rows, and
+// int8) or second (64 rows, int4) workgroup share the CU, which hides more
 // latency than the third stage did.
 constexpr int kSkinnyMaxM = 64;
 
-// Split of K for the small-M configurations: the number of runs that
-// minimises rounds-of-workgroups x (k tiles per run + fixed cost), at most 16
-// runs of at least 4 k tiles, and no more than the scratch buffer allows.
-// cols: columns per workgroup (256 or 512).
-inline int plan_split(int M, int K, int N, int bits, int cols, size_t lds, size_t ws_bytes) {
+// How a small-M problem is cut up.  A workgroup takes 256 columns, or 512
+// (two 32-column blocks per wavefront: half the activation bytes out of L2
+// and half the A-fragment reads out of LDS per MFMA, for twice the weight
+// bytes per k tile), and K is split into runs: at most 16, of at least 4 k
+// tiles, and no more than the scratch buffer holds.  Of all such pairs the one
+// with the lowest estimated time is taken.  The estimate, in k-tile times of a
+// 256-column workgroup:
+//   ceil(workgroups / CUs) x (tiles per run + 8) x (1.3 if 512 columns)
+//     + runs x M x N / 300000
+// The workgroups of a CU share its load path, so what counts is how many
+// the fullest CU gets, not how many are resident; the 8 is a workgroup's
+// start (the first tile's latency) and end (writing the partial sums); the
+// last term is the traffic of the partial sums, which every run writes and
+// the reduction reads.  The three constants are fitted to three sweeps, on
+// three machines, over every admissible pair on 160 problems (4096 <= K, N <=
+// 28672; 17, 32, 48, 64 rows; int4 and int8, with and without groups),
+// scoring a pair by the slowest of its three times: launches with more
+// workgroups than CUs but fewer than resident slots vary by up to 30 %
+// between machines, launches of at most one workgroup per CU by 3 %.  The
+// choice is 1.8 % slower than the best pair on average and 14 % at worst; the
+// rule it replaces (width by N and K alone, rounds by resident slots, no
+// traffic term) was 9.6 % and 29 % off.  int4 with group size 64 and 64-row
+// tiles does not fit the registers at 512 columns.
+struct SkinnyPlan {
+  bool wide;  // 512 columns per workgroup instead of 256
+  int ns;     // K runs
+};
+inline SkinnyPlan plan_skinny(int M, int K, int N, int bits, int group, size_t ws_bytes) {
   const int tk = bits == 8 ? 64 : 128, tiles = K / tk;
-  const int nbx = (N + cols - 1) / cols;
-  const int per_cu = static_cast<int>((160 * 1024) / lds) > 0 ? static_cast<int>((160 * 1024) / lds) : 1;
-  const int slots = num_cus() * per_cu;
+  const int cus = num_cus();
   const size_t per_run = static_cast<size_t>(M) * N * sizeof(float);
-  int best = 1;
-  int64_t best_cost = INT64_MAX;
-  for (int ns = 1; ns <= 16; ++ns) {
-    const int tps = (tiles + ns - 1) / ns;
-    const int eff = (tiles + tps - 1) / tps;
-    if (eff != ns || (ns > 1 && tps < 4)) continue;
-    if (ns > 1 && per_run * ns > ws_bytes) continue;
-    const int64_t rounds = (static_cast<int64_t>(nbx) * ns + slots - 1) / slots;
-    const int64_t cost = rounds * (tps + 2) * 8 + ns;  // the last term prefers fewer runs on ties
-    if (cost < best_cost) { best_cost = cost; best = ns; }
+  const double traffic = static_cast<double>(M) * N / 300000.0;
+  SkinnyPlan best{false, 1};
+  double best_cost = 1e300;
+  for (int wide = 0; wide < 2; ++wide) {
+    if (wide && bits == 4 && group == 64 && M > 32) continue;
+    const int cols = wide ? 512 : 256;
+    const int64_t nbx = (N + cols - 1) / cols;
+    for (int ns = 1; ns <= 16; ++ns) {
+      const int tps = (tiles + ns - 1) / ns;
+      const int eff = (tiles + tps - 1) / tps;
+      if (eff != ns || (ns > 1 && tps < 4)) continue;
+      if (ns > 1 && per_run * ns > ws_bytes) continue;
+      const int64_t rounds = (nbx * ns + cus - 1) / cus;
+      const double cost = static_cast<double>(rounds) * (tps + 8) * (wide ? 1.3 : 1.0) +
+                          (ns > 1 ? ns * traffic : 0.0) + 1e-6 * ns;  // the last term prefers fewer runs on ties
+      if (cost < best_cost) { best_cost = cost; best = SkinnyPlan{wide != 0, ns}; }
+    }
   }
   return best;
-}
-
-// The small-M configurations take 256 columns per workgroup, or 512 (two
-// 32-column blocks per wavefront): half the activation bytes out of L2 and
-// half the A-fragment reads out of LDS per MFMA (each workgroup fetches its
-// rows of x for its K run, which at 64 rows of int4 equals its weight
-// bytes).  Worth it while K runs can still make at least one workgroup per
-// CU; measured -13..-21 % at N >= 12288, +5..+20 % at N <= 4096 or K = 4096
-// int4 at N = 11008.  int4 with group size 64 and 64-row tiles does not fit
-// the registers at 512 columns.
-inline bool skinny_wide(int M, int K, int N, int bits, int group, size_t ws_bytes) {
-  if (bits == 4 && group == 64 && M > 32) return false;
-  const int tk = bits == 8 ? 64 : 128, tiles = K / tk;
-  int max_runs = tiles / 4 < 16 ? (tiles / 4 < 1 ? 1 : tiles / 4) : 16;
-  const size_t fit = ws_bytes / sizeof(float) / (static_cast<size_t>(M) * N);  // runs the scratch holds
-  if (fit < static_cast<size_t>(max_runs)) max_runs = fit < 1 ? 1 : static_cast<int>(fit);
-  return ((N + 511) / 512) * max_runs >= num_cus();
 }
 
 // Tile of the configuration launch_fast gives the columns that do not get
@@ -1065,26 +1076,13 @@ inline TailPlan plan_tail(int M, int K, int ncols, int bm, int bn, int tk, size_
   return {full, ns};
 }
 
-template <int BITS>
-size_t skinny_lds(int M, bool wide) {  // with group scales (the larger footprint)
-  if (BITS == 4 && M <= 32)
-    return wide ? dma_lds_bytes<4, 64, 1, 8, 1, 2, 2>() : dma_lds_bytes<4, 64, 1, 8, 1, 1, 2>();
-  return wide ? dma_lds_bytes<BITS, 64, 1, 8, 2, 2, 2>() : dma_lds_bytes<BITS, 64, 1, 8, 2, 1, 2>();
-}
-
-// K runs of the small-M configurations for a problem
-inline int plan_skinny(int M, int K, int N, int bits, int group, size_t ws_bytes, bool* wide) {
-  *wide = skinny_wide(M, K, N, bits, group, ws_bytes);
-  const size_t lds = bits == 8 ? skinny_lds<8>(M, *wide) : skinny_lds<4>(M, *wide);
-  return plan_split(M, K, N, bits, *wide ? 512 : 256, lds, ws_bytes);
-}
-
 template <int DT, int BITS, int G>
 void launch_fast(const Args& a) {
   const int nstrips = a.N / kStripCols;
   if (a.M <= kSkinnyMaxM) {
-    bool wide = false;
-    const int ns = plan_skinny(a.M, a.K, a.N, BITS, G, a.ws != nullptr ? a.ws_bytes : 0, &wide);
+    const SkinnyPlan sp = plan_skinny(a.M, a.K, a.N, BITS, G, a.ws != nullptr ? a.ws_bytes : 0);
+    const bool wide = sp.wide;
+    const int ns = sp.ns;
     if constexpr (BITS == 4) {
       if (a.M <= 32) {
         if (wide) launch_dma<DT, BITS, G, true, 1, 8, 1, 2, 2>(a, 0, nstrips, ns);
@@ -1231,9 +1229,8 @@ size_t linear_gemm_workspace(int64_t M, int64_t K, int64_t N, int bits, int grou
     const TailPlan t = plan_tail(static_cast<int>(M), static_cast<int>(K), ncols, bm, bn, tk, SIZE_MAX);
     return t.ns > 1 ? static_cast<size_t>(t.ns) * M * (ncols - t.full_tiles * bn) * sizeof(float) : 0;
   }
-  bool wide = false;
   const int ns = plan_skinny(static_cast<int>(M), static_cast<int>(K), static_cast<int>(N), bits,
-                             group_size > 0 ? group_size : 0, SIZE_MAX, &wide);
+                             group_size > 0 ? group_size : 0, SIZE_MAX).ns;
   return ns > 1 ? static_cast<size_t>(ns) * M * N * sizeof(float) : 0;
 }
 
@@ -1246,8 +1243,9 @@ void describe_linear_gemm(int64_t M, int64_t K, int64_t N, int bits, int group_s
     return;
   }
   if (M <= kSkinnyMaxM) {
-    bool wide = false;
-    const int ns = plan_skinny(static_cast<int>(M), static_cast<int>(K), static_cast<int>(N), bits, g, ws_bytes, &wide);
+    const SkinnyPlan sp = plan_skinny(static_cast<int>(M), static_cast<int>(K), static_cast<int>(N), bits, g, ws_bytes);
+    const bool wide = sp.wide;
+    const int ns = sp.ns;
     snprintf(buf, n, "wol::gemm_dma_kernel: %d rows x %d columns per workgroup, K in %d run(s)%s",
              bits == 4 && M <= 32 ? 32 : 64, wide ? 512 : 256, ns, ns > 1 ? " + reduce_partials_kernel" : "");
     return;
