@@ -294,10 +294,15 @@ enum wol_kernel {
   WOL_KERNEL_STREAM = 1, /* the streaming kernel (a workgroup per 16 columns);
                             M <= 64 only                                        */
   WOL_KERNEL_GEMM = 2,   /* the MFMA GEMM                                       */
-  WOL_KERNEL_BATCH = 3   /* the batched decode kernel (a workgroup per CU, the
+  WOL_KERNEL_BATCH = 3,  /* the batched decode kernel (a workgroup per CU, the
                             activations fetched once per workgroup); M <= 16
                             and K = 2048 or 4096 (8192 for int4 with group_size
                             -1 or 128) only                                     */
+  WOL_KERNEL_BATCH_SPLIT = 4 /* the same kernel with K cut into runs across
+                            workgroups, the runs' sums added by a second
+                            kernel; M <= 32, K at least 16 whole weight tiles
+                            (128 k for int4, 64 k for int8); needs the
+                            workspace wol_linear_workspace_for reports        */
 };
 
 /*

@@ -132,7 +132,7 @@ _ARG_ERRORS = {1, 2, 3, 4, 5, 6, 7, 8, 9}
 ACT_NONE, ACT_GELU, ACT_SWIGLU = 0, 1, 2
 
 # wol_kernel
-KERNEL_AUTO, KERNEL_STREAM, KERNEL_GEMM, KERNEL_BATCH = 0, 1, 2, 3
+KERNEL_AUTO, KERNEL_STREAM, KERNEL_GEMM, KERNEL_BATCH, KERNEL_BATCH_SPLIT = 0, 1, 2, 3, 4
 
 
 def check(status):

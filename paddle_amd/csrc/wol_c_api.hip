@@ -112,13 +112,53 @@ bool use_batch(int64_t M, int64_t K, int64_t N, int bits, int group_size) {
   return (M == 3 || M == 4) ? per_cu >= 5 : per_cu >= 2;
 }
 
+// The batched decode kernel with K cut into runs across workgroups (two
+// launches: the runs, then their sum) against whatever the rules above would
+// take.  Measured on MI355X over 18 shapes (K, N from 2048 to 28672, also the
+// ones that are not powers of two), both bit widths, 2 to 32 rows:
+//  * up to 16 rows it wins where the streaming kernel is at its worst -- 10
+//    rows and more (the activation reads of a workgroup per strip weigh in),
+//    a K the one-launch batched kernel is not built for, and strips that
+//    leave the CUs a ragged last round (N / 16 / CUs is 1.1 or more below
+//    its ceiling: N = 5120 ... 7168 on 256 CUs), by 10 to 49 %; int4 with
+//    K >= 14336 from 12 rows on also with whole rounds (9 to 18 %);
+//  * from 17 to 32 rows (two 16-row operands) it beats the better of the
+//    streaming kernel and the MFMA GEMM on int8 weights of 20 MB and more by
+//    5 to 20 %, and on int4 weights of 10 to 34 MB by up to 17 %.
+// Elsewhere the second launch (3 us) costs more than the split gains.
+// ws_bytes: the caller's scratch.
+bool use_batch_split(int64_t M, int64_t K, int64_t N, int bits, int group_size, size_t ws_bytes) {
+  if (M < 2 || !wol::linear_batch_split_supports(M, K, bits, group_size)) return false;
+  if (ws_bytes < wol::linear_batch_split_workspace(M, K, N, bits, group_size)) return false;
+  const double w = static_cast<double>(K) * N * bits / 8.0 * 1e-6;  // weight MB
+  if (M > 16) return bits == 4 ? (w >= 10.0 && w <= 34.0) : w >= 20.0;
+  const int64_t cus = wol::linear_batch_cus(), nstrips = N / wol::kStripCols;
+  if (M < 10 || nstrips > 2 * cus || wol::linear_batch_supports(M, K, bits, group_size)) return false;
+  const double rounds = static_cast<double>(nstrips) / cus;
+  const double ragged = static_cast<double>((nstrips + cus - 1) / cus) / rounds;
+  if (ragged >= 1.1) return true;
+  return bits == 4 && M >= 12 && K >= 14336;
+}
+
 // kernel: a wol_kernel; AUTO resolves by M and the cost model.  Returns the
-// wol_kernel that runs.
+// wol_kernel that runs.  ws_bytes: the caller's scratch (SIZE_MAX: as much as
+// any kernel asks for).
 int resolve_kernel(int kernel, int64_t M, int64_t K, int64_t N, int bits, int group_size,
-                   bool have_ws = true) {
+                   size_t ws_bytes = SIZE_MAX) {
   if (kernel != WOL_KERNEL_AUTO) return kernel;
+  if (use_batch_split(M, K, N, bits, group_size, ws_bytes)) return WOL_KERNEL_BATCH_SPLIT;
   if (use_batch(M, K, N, bits, group_size)) return WOL_KERNEL_BATCH;
+  const bool have_ws = ws_bytes / sizeof(float) / 2 >= static_cast<size_t>(M) * static_cast<size_t>(N);
   return use_stream(M, K, N, bits, have_ws) ? WOL_KERNEL_STREAM : WOL_KERNEL_GEMM;
+}
+
+const char* kernel_name(int which) {
+  switch (which) {
+    case WOL_KERNEL_BATCH: return "batch";
+    case WOL_KERNEL_BATCH_SPLIT: return "batch (K split)";
+    case WOL_KERNEL_STREAM: return "stream";
+    default: return "gemm";
+  }
 }
 
 // WOL_LOG=1 in the environment: every compute call writes one line to stderr
@@ -139,10 +179,13 @@ int linear_impl(const void* x, const void* codes, const void* bias, const void* 
   if (rc != WOL_OK) return rc;
   if (M < 0 || M > (int64_t{1} << 24)) return WOL_ERR_BAD_SHAPE;
   if (kernel != WOL_KERNEL_AUTO && kernel != WOL_KERNEL_STREAM && kernel != WOL_KERNEL_GEMM &&
-      kernel != WOL_KERNEL_BATCH)
+      kernel != WOL_KERNEL_BATCH && kernel != WOL_KERNEL_BATCH_SPLIT)
     return WOL_ERR_BAD_SHAPE;
   if (kernel == WOL_KERNEL_STREAM && M > kStreamMaxM) return WOL_ERR_BAD_SHAPE;
   if (kernel == WOL_KERNEL_BATCH && M > 0 && !wol::linear_batch_supports(M, K, bits, group_size)) return WOL_ERR_BAD_SHAPE;
+  if (kernel == WOL_KERNEL_BATCH_SPLIT && M > 0 &&
+      (!wol::linear_batch_split_supports(M, K, bits, group_size) || fuse.pre_scale != nullptr))
+    return WOL_ERR_BAD_SHAPE;
   if (M == 0) return WOL_OK;  // empty batch: nothing to write
   if (x == nullptr || codes == nullptr || scale == nullptr || out == nullptr)
     return WOL_ERR_NULL_POINTER;
@@ -150,14 +193,18 @@ int linear_impl(const void* x, const void* codes, const void* bias, const void* 
   if (const int dv = require_gfx950(); dv != WOL_OK) return dv;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (workspace == nullptr || !aligned16(workspace)) workspace_bytes = 0;  // optional: only speeds up
-  const bool have_ws = workspace_bytes / sizeof(float) / 2 >= static_cast<size_t>(M) * static_cast<size_t>(N);
-  const int which = resolve_kernel(kernel, M, K, N, bits, group_size, have_ws);
+  int which = resolve_kernel(kernel, M, K, N, bits, group_size, workspace_bytes);
+  if (which == WOL_KERNEL_BATCH_SPLIT && kernel == WOL_KERNEL_AUTO && fuse.pre_scale != nullptr)
+    which = resolve_kernel(kernel, M, K, N, bits, group_size, 0);  // that kernel applies no pre-scale
   if (log_enabled())
     fprintf(stderr, "[wol] linear M=%lld K=%lld N=%lld int%d group=%d %s%s%s act=%d -> %s kernel\n",
             static_cast<long long>(M), static_cast<long long>(K), static_cast<long long>(N), bits, group_size,
             dtype == WOL_DTYPE_BF16 ? "bf16" : "f16", bias != nullptr ? " bias" : "",
             fuse.pre_scale != nullptr ? " pre_scale" : "", fuse.act,
-            which == WOL_KERNEL_BATCH ? "batch" : (which == WOL_KERNEL_STREAM ? "stream" : "gemm"));
+            kernel_name(which));
+  if (which == WOL_KERNEL_BATCH_SPLIT)
+    return wol::launch_linear_batch_split(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out,
+                                          out_f32, workspace, workspace_bytes, s, fuse);
   if (which == WOL_KERNEL_BATCH)
     return wol::launch_linear_batch(x, codes, bias, scale, dtype, M, K, N, bits, group_size, out,
                                     out_f32, s, fuse);
@@ -263,7 +310,9 @@ size_t wol_linear_workspace_for(int64_t M, int64_t K, int64_t N, int bits, int g
                                 int kernel) {
   if (check_problem(WOL_DTYPE_F16, K, N, bits, group_size) != WOL_OK || M <= 0) return 0;
   if (kernel == WOL_KERNEL_STREAM && M > kStreamMaxM) return 0;
-  if (resolve_kernel(kernel, M, K, N, bits, group_size) != WOL_KERNEL_GEMM) return 0;  // partial sums stay on chip
+  const int which = resolve_kernel(kernel, M, K, N, bits, group_size);
+  if (which == WOL_KERNEL_BATCH_SPLIT) return wol::linear_batch_split_workspace(M, K, N, bits, group_size);
+  if (which != WOL_KERNEL_GEMM) return 0;  // partial sums stay on chip
   return wol::linear_gemm_workspace(M, K, N, bits, group_size);
 }
 
@@ -295,7 +344,8 @@ struct FusedPlan {
 FusedPlan plan_fused(int64_t M, int64_t K, int64_t N, int bits, int group_size, bool has_pre, int act) {
   FusedPlan f{};
   const size_t lws = wol_linear_workspace(M, K, N, bits, group_size);
-  const int which = resolve_kernel(WOL_KERNEL_AUTO, M, K, N, bits, group_size, true);
+  // a call with activation scales never takes the K-split batched kernel
+  const int which = resolve_kernel(WOL_KERNEL_AUTO, M, K, N, bits, group_size, has_pre ? 0 : SIZE_MAX);
   const bool fused_pre = (which == WOL_KERNEL_BATCH && wol::linear_batch_fuses_pre_scale(K, bits, group_size)) ||
                          (which == WOL_KERNEL_STREAM && M == 1);
   f.prepass = has_pre && !fused_pre;
@@ -562,9 +612,10 @@ int wol_linear_plan(int64_t M, int64_t K, int64_t N, int bits, int group_size, s
   const int rc = check_problem(WOL_DTYPE_F16, K, N, bits, group_size);
   if (rc != WOL_OK) return rc;
   if (M <= 0 || M > (int64_t{1} << 24)) return WOL_ERR_BAD_SHAPE;
-  const bool have_ws = workspace_bytes / sizeof(float) / 2 >= static_cast<size_t>(M) * static_cast<size_t>(N);
-  const int which = resolve_kernel(WOL_KERNEL_AUTO, M, K, N, bits, group_size, have_ws);
-  if (which == WOL_KERNEL_BATCH) {
+  const int which = resolve_kernel(WOL_KERNEL_AUTO, M, K, N, bits, group_size, workspace_bytes);
+  if (which == WOL_KERNEL_BATCH_SPLIT) {
+    wol::describe_linear_batch_split(M, K, N, bits, group_size, buf, buf_bytes);
+  } else if (which == WOL_KERNEL_BATCH) {
     int grid = 1, tpw = 1;
     wol::plan_linear_batch(K, N, bits, &grid, &tpw);
     snprintf(buf, buf_bytes, "wol::batch_kernel: %d workgroups of 16 wavefronts, %lld or %lld strips each, "

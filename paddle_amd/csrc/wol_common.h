@@ -277,6 +277,21 @@ void plan_linear_batch(int64_t K, int64_t N, int bits, int* grid, int* tpw);
 int launch_linear_batch(const void* x, const void* codes, const void* bias, const void* scale,
                         int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
                         void* out, bool out_f32, hipStream_t stream, const Fuse& f = Fuse());
+// The batched decode kernel with K cut into runs across workgroups (up to 32
+// rows, any K of at least 16 whole weight tiles): the runs' fp32 sums go
+// through ws (linear_batch_split_workspace bytes) and launch_reduce_partials
+// adds them.  It applies no Fuse::pre_scale.
+bool linear_batch_split_supports(int64_t M, int64_t K, int bits, int group_size);
+size_t linear_batch_split_workspace(int64_t M, int64_t K, int64_t N, int bits, int group_size);
+int launch_linear_batch_split(const void* x, const void* codes, const void* bias, const void* scale,
+                              int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
+                              void* out, bool out_f32, void* ws, size_t ws_bytes, hipStream_t stream,
+                              const Fuse& f = Fuse());
+void describe_linear_batch_split(int64_t M, int64_t K, int64_t N, int bits, int group_size, char* buf, size_t n);
+// out[m, n] = T(act(sum over the runs of part[run][m][n] + bias[n])): the second
+// kernel of every K-split launch (wol_linear_gemm.hip).  N % 4 == 0.
+int launch_reduce_partials(const float* part, int nsplit, const void* bias, int dtype, void* out,
+                           bool out_f32, int64_t M, int64_t N, int act, hipStream_t stream);
 // One-line descriptions of what the launchers would run for a problem.
 void describe_linear_stream(int64_t M, int64_t K, int64_t N, int bits, int group_size, char* buf, size_t n);
 void describe_linear_gemm(int64_t M, int64_t K, int64_t N, int bits, int group_size, size_t ws_bytes,

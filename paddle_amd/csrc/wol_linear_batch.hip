@@ -61,7 +61,7 @@ __device__ inline f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
 }
 
 constexpr int kBatchWaves = 16;
-constexpr int kBatchRun = 7;  // strips whose partial sums (16 KiB each) share the LDS
+constexpr int kBatchRun = 7;  // strips whose partial sums (16 KiB each per 16 rows) share the LDS
 
 struct BatchParams {
   const uint16_t* x;
@@ -75,6 +75,11 @@ struct BatchParams {
   int strips_q, strips_r;  // strips per workgroup: N / 16 = grid * strips_q + strips_r
   const uint16_t* pre;     // [K] per-channel scales of the activations, or null
   int act;                 // WOL_ACT_NONE or WOL_ACT_GELU
+  // K cut into runs across workgroups (SPLIT): workgroup b takes run b % nseg
+  // of strip set b / nseg and leaves its scaled fp32 sums in ws[run][M][N]
+  int nseg;
+  int ntiles;              // K / tile depth
+  float* ws;
 };
 
 // G: 0 per-channel, else the group size.  TPW: weight tiles (1 KiB, 64 or 128
@@ -86,7 +91,15 @@ struct BatchParams {
 // IT: tiles per item, D: items in the ring (a multiple of TPW / IT).
 // PRE: the activations are multiplied by p.pre (each product rounded to T as
 // apply_per_channel_scale rounds it) once, in the registers they stay in.
-template <int DT, int BITS, int G, int TPW, int IT, int D, bool PRE>
+// MT: 16-row operands (M <= 16 * MT); every dequantised B fragment feeds MT
+// MFMAs.
+// SPLIT: K is cut into p.nseg runs of 16 * TPW tiles across workgroups, the
+// last of which may reach past K: a wavefront's tiles past the end have zero
+// activations and fetch nothing.  The sums of a run go to p.ws and a second
+// kernel adds the runs (bias and activation function there).  This is what
+// serves any K made of whole tiles, and what keeps x down to K / nseg per CU
+// when the strips are few.
+template <int DT, int BITS, int G, int TPW, int IT, int D, bool PRE, int MT, bool SPLIT>
 __global__ __launch_bounds__(kBatchWaves * 64) void batch_kernel(const BatchParams p) {
   constexpr int WK = kBatchWaves;
   constexpr int TK = BITS == 8 ? 64 : 128;   // k per 1 KiB weight tile
@@ -98,8 +111,9 @@ __global__ __launch_bounds__(kBatchWaves * 64) void batch_kernel(const BatchPara
   constexpr int CPT = TK / CK;               // chains per tile
   constexpr int SPC = SPT / CPT;             // k steps per chain
   constexpr int NS = G == 0 ? 1 : IT * CPT;  // group scales per item and lane
-  constexpr bool kKeepCancel = TPW * SPT <= 8 && TPW * CPT <= 4;  // cancelling terms computed once and kept
-                                                               // where 32 registers of A leave 16 for them
+  constexpr bool kKeepCancel = MT * TPW * SPT <= 8 && MT * TPW * CPT <= 4;  // cancelling terms computed once and kept
+                                                                         // where 32 registers of A leave 16 for them
+  static_assert(!(PRE && (SPLIT || MT > 1)), "the fused activation scales exist for the one-run, 16-row form");
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
   const int lane = threadIdx.x & 63;
@@ -107,10 +121,12 @@ __global__ __launch_bounds__(kBatchWaves * 64) void batch_kernel(const BatchPara
   const int j = lane & 15, kb = lane >> 4;
   const int K = p.K, N = p.N, M = p.M;
   // this workgroup's strips; this wavefront's tiles are t0 .. t0 + TPW - 1 of each
-  const int bid = static_cast<int>(blockIdx.x);
+  const int seg = SPLIT ? static_cast<int>(blockIdx.x) % p.nseg : 0;
+  const int bid = SPLIT ? static_cast<int>(blockIdx.x) / p.nseg : static_cast<int>(blockIdx.x);
   const int s0 = bid * p.strips_q + (bid < p.strips_r ? bid : p.strips_r);
   const int s1 = s0 + p.strips_q + (bid < p.strips_r ? 1 : 0);
-  const int t0 = wave * TPW;
+  const int t0 = (seg * WK + wave) * TPW;
+  const int ntiles = p.ntiles;
   const int64_t sbytes = strip_bytes(K, BITS);
 
   uint32_t magic = Dequant<DT, BITS>::kMagic;
@@ -123,13 +139,25 @@ __global__ __launch_bounds__(kBatchWaves * 64) void batch_kernel(const BatchPara
   // its cycles per active lane: at 4 rows the fragments cost a quarter of what
   // 16 rows cost); the other rows hold whatever the registers held (rows of an MFMA result do
   // not mix) and are never stored.
-  const uint16_t* xrow = p.x + static_cast<int64_t>(j < M ? j : 0) * K + t0 * TK + 8 * kb;
-  u32x4 A[TPW * SPT];
+  u32x4 A[MT][TPW * SPT];
 #pragma unroll
-  for (int s = 0; s < TPW * SPT; ++s) asm volatile("" : "=v"(A[s]));  // any value will do in the rows past M
-  if (j < M) {
+  for (int mt = 0; mt < MT; ++mt) {
+    const int row = mt * 16 + j;
+    const uint16_t* xrow = p.x + static_cast<int64_t>(row < M ? row : 0) * K + t0 * TK + 8 * kb;
 #pragma unroll
-    for (int s = 0; s < TPW * SPT; ++s) A[s] = *reinterpret_cast<const u32x4*>(xrow + s * 32);
+    for (int s = 0; s < TPW * SPT; ++s) asm volatile("" : "=v"(A[mt][s]));  // any value will do in the rows past M
+    if (SPLIT) {
+      // tiles past the end of K: zero activations in every lane, so that what
+      // the weight registers of such a tile hold (zeros) never counts
+#pragma unroll
+      for (int s = 0; s < TPW * SPT; ++s)
+        if (t0 + s / SPT >= ntiles) A[mt][s] = u32x4{0u, 0u, 0u, 0u};
+    }
+    if (row < M) {
+#pragma unroll
+      for (int s = 0; s < TPW * SPT; ++s)
+        if (!SPLIT || t0 + s / SPT < ntiles) A[mt][s] = *reinterpret_cast<const u32x4*>(xrow + s * 32);
+    }
   }
   // The activation scales of the wavefront's k (the same for every row): lane
   // 4 * s + kb holds the eight scales that go with A[s] in lane group kb, one
@@ -150,17 +178,20 @@ __global__ __launch_bounds__(kBatchWaves * 64) void batch_kernel(const BatchPara
     if (G != 0) {  // the item's group scales travel with it (past the last item: the last strip's again)
 #pragma unroll
       for (int q = 0; q < NS; ++q) {
-        const int k0 = (t0 + part * IT) * TK + q * CK;
+        int k0 = (t0 + part * IT) * TK + q * CK;
+        if (SPLIT) k0 = k0 < K ? k0 : K - CK;  // a tile past K: any scale that exists (it meets zeros)
         sc[q] = p.scale[static_cast<int64_t>(k0 >> p.gshift) * N + strip * kStripCols + j];
       }
     }
     const int soff = real ? strip_of_run * static_cast<int>(sbytes) + part * IT * 1024 : 0x7FFF0000;
 #pragma unroll
-    for (int i = 0; i < IT; ++i)
-      w[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off + soff + i * 1024, 0, 0));
+    for (int i = 0; i < IT; ++i) {
+      const int off = !SPLIT || t0 + part * IT + i < ntiles ? soff : 0x7FFF0000;
+      w[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off + off + i * 1024, 0, 0));
+    }
   };
 
-  f32x4 ccs[kKeepCancel ? TPW * CPT : 1];  // the cancelling term of every chain of the wavefront's run
+  f32x4 ccs[MT][kKeepCancel ? TPW * CPT : 1];  // the cancelling term of every chain of the wavefront's run
   bool have_cc = false;
   // the per-channel scales (first row of the scale tensor) and the bias behind
   // bounded descriptors, for the staging loads
@@ -169,13 +200,14 @@ __global__ __launch_bounds__(kBatchWaves * 64) void batch_kernel(const BatchPara
   const __amdgpu_buffer_rsrc_t bias_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<uint16_t*>(p.bias != nullptr ? p.bias : p.scale), 0, N * 2, 0x00020000);
 
-  for (int sr = s0; sr < s1; sr += kBatchRun) {
-    const int cnt = s1 - sr < kBatchRun ? s1 - sr : kBatchRun;  // strips of this run
+  constexpr int kRun = kBatchRun / MT;  // strips whose partial sums share the LDS
+  for (int sr = s0; sr < s1; sr += kRun) {
+    const int cnt = s1 - sr < kRun ? s1 - sr : kRun;  // strips of this run
     const int nitems = cnt * P;  // item it: strip sr + it / P, part it % P
 
     const int ncols = cnt * kStripCols;
-    float* red = reinterpret_cast<float*>(smem);                          // [cnt][WK][4][64]
-    uint16_t* lsc = reinterpret_cast<uint16_t*>(smem + cnt * WK * 1024);  // [ncols] per-channel scales
+    float* red = reinterpret_cast<float*>(smem);                               // [cnt][WK][MT * 4][64]
+    uint16_t* lsc = reinterpret_cast<uint16_t*>(smem + cnt * WK * MT * 1024);  // [ncols] per-channel scales
     uint16_t* lbi = lsc + ncols;                                          // [ncols] bias
 
     // What the end of the run needs -- per-channel scales and bias of its
@@ -210,20 +242,24 @@ __global__ __launch_bounds__(kBatchWaves * 64) void batch_kernel(const BatchPara
         ps.y = __builtin_amdgcn_ds_bpermute(src, PS.y);
         ps.z = __builtin_amdgcn_ds_bpermute(src, PS.z);
         ps.w = __builtin_amdgcn_ds_bpermute(src, PS.w);
-        A[s] = prescale_frag<DT>(A[s], ps);
+        A[0][s] = prescale_frag<DT>(A[0][s], ps);
       }
     }
     if (kKeepCancel && !have_cc) {
 #pragma unroll
-      for (int c = 0; c < TPW * CPT; ++c) {
-        f32x4 cc = {0.f, 0.f, 0.f, 0.f};
+      for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int s = 0; s < SPC; ++s) cc = mfma16<DT>(A[c * SPC + s], cancel, cc);
-        ccs[c] = cc;
-      }
+        for (int c = 0; c < TPW * CPT; ++c) {
+          f32x4 cc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int s = 0; s < SPC; ++s) cc = mfma16<DT>(A[mt][c * SPC + s], cancel, cc);
+          ccs[mt][c] = cc;
+        }
     }
     have_cc = true;
-    f32x4 tot = {0.f, 0.f, 0.f, 0.f};
+    f32x4 tot[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) tot[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
     for (int base = 0; base < nitems; base += D) {
 #pragma unroll
       for (int d = 0; d < D; ++d) {
@@ -237,33 +273,44 @@ __global__ __launch_bounds__(kBatchWaves * 64) void batch_kernel(const BatchPara
 #pragma unroll
             for (int ch = 0; ch < CPT; ++ch) {
               const int a0 = ((part * IT + i) * CPT + ch) * SPC;  // first A fragment of the chain
-              f32x4 acc;
-              if (kKeepCancel) {
-                acc = ccs[(part * IT + i) * CPT + ch];
-              } else {
-                acc = f32x4{0.f, 0.f, 0.f, 0.f};
+              f32x4 acc[MT];
 #pragma unroll
-                for (int s = 0; s < SPC; ++s) acc = mfma16<DT>(A[a0 + s], cancel, acc);
+              for (int mt = 0; mt < MT; ++mt) {
+                if (kKeepCancel) {
+                  acc[mt] = ccs[mt][(part * IT + i) * CPT + ch];
+                } else {
+                  acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                  for (int s = 0; s < SPC; ++s) acc[mt] = mfma16<DT>(A[mt][a0 + s], cancel, acc[mt]);
+                }
               }
 #pragma unroll
               for (int s = 0; s < SPC; ++s) {
                 const u32x4 b = Dequant<DT, BITS>::run(&w4[(ch * SPC + s) * kDw], magic);
-                acc = mfma16<DT>(A[a0 + s], b, acc);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) acc[mt] = mfma16<DT>(A[mt][a0 + s], b, acc[mt]);
               }
               if (G != 0) {
                 const float sc = to_f32<DT>(S[d][i * CPT + ch]);
 #pragma unroll
-                for (int r = 0; r < 4; ++r) tot[r] = fmaf(acc[r], sc, tot[r]);
+                for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                  for (int r = 0; r < 4; ++r) tot[mt][r] = fmaf(acc[mt][r], sc, tot[mt][r]);
               } else {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) tot[r] += acc[r];
+                for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                  for (int r = 0; r < 4; ++r) tot[mt][r] += acc[mt][r];
               }
             }
           }
           if (part == P - 1) {  // the strip is complete for this wavefront
 #pragma unroll
-            for (int r = 0; r < 4; ++r) red[((sl * WK + wave) * 4 + r) * 64 + lane] = tot[r];
-            tot = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+              for (int r = 0; r < 4; ++r) red[((sl * WK + wave) * MT * 4 + mt * 4 + r) * 64 + lane] = tot[mt][r];
+              tot[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
           }
         }
         // the slot is free: refill it with the item D places further on (if there is one)
@@ -277,18 +324,23 @@ __global__ __launch_bounds__(kBatchWaves * 64) void batch_kernel(const BatchPara
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
       const int e = threadIdx.x + q * WK * 64;
-      if (e < cnt * 256) {
-        const int sl = e >> 8, r = (e >> 6) & 3, l = e & 63;
+      if (e < cnt * MT * 256) {
+        // e = ((strip of the run * MT + mt) * 4 + r) * 64 + lane of the MFMA result
+        const int sl = e / (MT * 256), rr = (e >> 6) % (MT * 4), l = e & 63;
         float s = 0.0f;
 #pragma unroll
-        for (int w = 0; w < WK; ++w) s += red[((sl * WK + w) * 4 + r) * 64 + l];
-        const int m = 4 * (l >> 4) + r;
+        for (int w = 0; w < WK; ++w) s += red[((sl * WK + w) * MT * 4 + rr) * 64 + l];
+        const int m = (rr >> 2) * 16 + 4 * (l >> 4) + (rr & 3);
         if (m < M) {
           const int cl = sl * kStripCols + (l & 15);
           const float ep_scale = G == 0 ? to_f32<DT>(lsc[cl]) : 1.0f;
+          const int64_t o = static_cast<int64_t>(m) * N + (sr + sl) * kStripCols + (l & 15);
+          if (SPLIT) {
+            p.ws[static_cast<int64_t>(seg) * M * N + o] = s * ep_scale;
+            continue;
+          }
           const float ep_bias = p.bias != nullptr ? to_f32<DT>(lbi[cl]) : 0.0f;
           s = act_apply(s * ep_scale + ep_bias, p.act);
-          const int64_t o = static_cast<int64_t>(m) * N + (sr + sl) * kStripCols + (l & 15);
           if (p.out_f32)
             static_cast<float*>(p.out)[o] = s;
           else
@@ -307,7 +359,7 @@ __global__ __launch_bounds__(kBatchWaves * 64) void batch_kernel(const BatchPara
 #pragma unroll
       for (int q = 0; q < NS; ++q) asm volatile("" ::"v"(S[d][q]));
     }
-    if (sr + kBatchRun < s1) __syncthreads();  // the next run overwrites the partial sums
+    if (sr + kRun < s1) __syncthreads();  // the next run overwrites the partial sums
   }
 }
 
@@ -315,6 +367,7 @@ struct Args {
   const void* x; const void* codes; const void* bias; const void* scale; void* out;
   int M, K, N, gshift, out_f32; hipStream_t stream;
   const void* pre; int act;
+  int nseg; float* ws;  // K runs across workgroups and where their sums go (nseg = 1: none)
 };
 
 inline int num_cus() {
@@ -338,20 +391,20 @@ inline void allow_lds(const void* kern, size_t lds, std::atomic<uint32_t>& done)
   done.fetch_or(bit, std::memory_order_release);
 }
 
-// LDS of a launch: partial sums, scales and bias of the longest run of strips
-inline size_t batch_lds(int64_t K, int64_t N, int group_size, int grid) {
+// LDS of a launch: partial sums, scales and bias of the longest run of strips.
+// sets: strip sets (workgroups, or workgroups / K runs); mt: 16-row operands.
+inline size_t batch_lds(int64_t N, int sets, int mt) {
   const int64_t nstrips = N / kStripCols;
-  int64_t per_wg = (nstrips + grid - 1) / grid;
-  if (per_wg > kBatchRun) per_wg = kBatchRun;
-  (void)K;
-  (void)group_size;
-  return static_cast<size_t>(per_wg * kBatchWaves * 1024 + 2 * per_wg * kStripCols * 2);
+  int64_t per_wg = (nstrips + sets - 1) / sets;
+  if (per_wg > kBatchRun / mt) per_wg = kBatchRun / mt;
+  return static_cast<size_t>(per_wg * kBatchWaves * mt * 1024 + 2 * per_wg * kStripCols * 2);
 }
 
-template <int DT, int BITS, int G, int TPW, int IT, int D, bool PRE>
+// grid: strip sets; with SPLIT every set is worked on by a.nseg workgroups
+template <int DT, int BITS, int G, int TPW, int IT, int D, bool PRE, int MT = 1, bool SPLIT = false>
 void launch_pre(const Args& a, int grid) {
-  const size_t lds = batch_lds(a.K, a.N, G, grid);
-  auto kern = batch_kernel<DT, BITS, G, TPW, IT, D, PRE>;
+  const size_t lds = batch_lds(a.N, grid, MT);
+  auto kern = batch_kernel<DT, BITS, G, TPW, IT, D, PRE, MT, SPLIT>;
   static std::atomic<uint32_t> configured{0};  // per instantiation
   allow_lds(reinterpret_cast<const void*>(kern), 160 * 1024, configured);
   BatchParams p;
@@ -367,7 +420,10 @@ void launch_pre(const Args& a, int grid) {
   p.strips_r = a.N / kStripCols % grid;
   p.pre = PRE ? static_cast<const uint16_t*>(a.pre) : nullptr;
   p.act = a.act;
-  kern<<<dim3(static_cast<unsigned>(grid)), dim3(kBatchWaves * 64), lds, a.stream>>>(p);
+  p.nseg = SPLIT ? a.nseg : 1;
+  p.ntiles = a.K / (BITS == 8 ? 64 : 128);
+  p.ws = a.ws;
+  kern<<<dim3(static_cast<unsigned>(grid * p.nseg)), dim3(kBatchWaves * 64), lds, a.stream>>>(p);
 }
 
 // The fused activation scales are built where the registers allow: A
@@ -410,6 +466,37 @@ void launch_g(const Args& a, int grid, int tpw) {
   else launch_cfg<DT, BITS, 128>(a, grid, tpw);
 }
 
+// The K-split form.  k2: a wavefront's run is 256 k long (two int4 tiles,
+// four int8 tiles) instead of 128; the items and ring depths are those of the
+// one-run form with the same run.  Up to 16 rows, or up to 32 as two 16-row
+// operands -- those with the short run only: 64 registers of A fragments
+// leave no room for the ring.
+template <int DT, int BITS, int G, int MT>
+void launch_split_cfg(const Args& a, int sets, bool k2) {
+  if constexpr (MT == 1) {
+    if (k2) {
+      if constexpr (BITS == 4) launch_pre<DT, 4, G, 2, 2, 3, false, 1, true>(a, sets);
+      else launch_pre<DT, 8, G, 4, 4, 2, false, 1, true>(a, sets);
+      return;
+    }
+  }
+  if constexpr (BITS == 4) launch_pre<DT, 4, G, 1, 1, 4, false, MT, true>(a, sets);
+  else launch_pre<DT, 8, G, 2, 2, 3, false, MT, true>(a, sets);
+}
+
+template <int DT, int BITS>
+void launch_split_g(const Args& a, int sets, bool k2) {
+  if (a.M <= 16) {
+    if (a.gshift < 0) launch_split_cfg<DT, BITS, 0, 1>(a, sets, k2);
+    else if (a.gshift == 6) launch_split_cfg<DT, BITS, 64, 1>(a, sets, k2);
+    else launch_split_cfg<DT, BITS, 128, 1>(a, sets, k2);
+  } else {
+    if (a.gshift < 0) launch_split_cfg<DT, BITS, 0, 2>(a, sets, k2);
+    else if (a.gshift == 6) launch_split_cfg<DT, BITS, 64, 2>(a, sets, k2);
+    else launch_split_cfg<DT, BITS, 128, 2>(a, sets, k2);
+  }
+}
+
 }  // namespace
 
 // K must split into the same number of whole weight tiles for each of the 16
@@ -446,13 +533,81 @@ int launch_linear_batch(const void* x, const void* codes, const void* bias, cons
   plan_linear_batch(K, N, bits, &grid, &tpw);
   const Args a{x, codes, bias, scale, out, static_cast<int>(M), static_cast<int>(K),
                static_cast<int>(N), gshift, out_f32 ? 1 : 0, stream,
-               linear_batch_fuses_pre_scale(K, bits, group_size) ? f.pre_scale : nullptr, f.act};
+               linear_batch_fuses_pre_scale(K, bits, group_size) ? f.pre_scale : nullptr, f.act, 1, nullptr};
   if (dtype == WOL_DTYPE_BF16) {
     if (bits == 8) launch_g<WOL_DTYPE_BF16, 8>(a, grid, tpw); else launch_g<WOL_DTYPE_BF16, 4>(a, grid, tpw);
   } else {
     if (bits == 8) launch_g<WOL_DTYPE_F16, 8>(a, grid, tpw); else launch_g<WOL_DTYPE_F16, 4>(a, grid, tpw);
   }
   return check_launch();
+}
+
+// The K-split form takes up to 32 rows and any K made of at least 16 whole
+// weight tiles (128 k for int4, 64 k for int8).
+bool linear_batch_split_supports(int64_t M, int64_t K, int bits, int group_size) {
+  (void)group_size;
+  const int64_t tk = bits == 8 ? 64 : 128;
+  return M >= 1 && M <= 32 && K % tk == 0 && K / tk >= 16;
+}
+
+// How the K-split form cuts a problem: k2 (256 k per wavefront and run
+// instead of 128), the number of runs and the number of strip sets (each set
+// is worked on by one workgroup per run; sets x runs is about the CU count).
+// The longer run halves the partial sums and doubles the activations a
+// workgroup holds: measured faster from seven short runs on (K >= 13824 for
+// int4), slower below.  Two 16-row operands leave registers for the short run
+// only.
+void plan_linear_batch_split(int64_t M, int64_t K, int64_t N, int bits, int group_size, bool* k2,
+                             int* nseg, int* sets) {
+  (void)group_size;
+  const int64_t tk = bits == 8 ? 64 : 128, tiles = K / tk;
+  const int64_t nstrips = N / kStripCols;
+  const int cus = num_cus();
+  const int64_t per_run_short = kBatchWaves * (128 / tk);
+  *k2 = M <= 16 && (tiles + per_run_short - 1) / per_run_short >= 7;
+  const int64_t per_run = *k2 ? 2 * per_run_short : per_run_short;
+  *nseg = static_cast<int>((tiles + per_run - 1) / per_run);
+  int64_t v = cus / *nseg;
+  if (v < 1) v = 1;
+  *sets = static_cast<int>(v < nstrips ? v : nstrips);
+}
+
+size_t linear_batch_split_workspace(int64_t M, int64_t K, int64_t N, int bits, int group_size) {
+  if (!linear_batch_split_supports(M, K, bits, group_size)) return 0;
+  bool k2 = false;
+  int nseg = 1, sets = 1;
+  plan_linear_batch_split(M, K, N, bits, group_size, &k2, &nseg, &sets);
+  return static_cast<size_t>(nseg) * M * N * sizeof(float);
+}
+
+void describe_linear_batch_split(int64_t M, int64_t K, int64_t N, int bits, int group_size, char* buf, size_t n) {
+  bool k2 = false;
+  int nseg = 1, sets = 1;
+  plan_linear_batch_split(M, K, N, bits, group_size, &k2, &nseg, &sets);
+  snprintf(buf, n, "wol::batch_kernel: %d strip sets x %d K runs of %d k, %d-row operands x %d + reduce_partials_kernel",
+           sets, nseg, kBatchWaves * (k2 ? 256 : 128), 16, M > 16 ? 2 : 1);
+}
+
+// ws: nseg x M x N floats (linear_batch_split_workspace).  No fused pre-scale.
+int launch_linear_batch_split(const void* x, const void* codes, const void* bias, const void* scale,
+                              int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
+                              void* out, bool out_f32, void* ws, size_t ws_bytes, hipStream_t stream,
+                              const Fuse& f) {
+  if (!linear_batch_split_supports(M, K, bits, group_size) || f.pre_scale != nullptr) return WOL_ERR_BAD_SHAPE;
+  if (ws == nullptr || ws_bytes < linear_batch_split_workspace(M, K, N, bits, group_size)) return WOL_ERR_WORKSPACE;
+  const int gshift = group_size == 64 ? 6 : (group_size == 128 ? 7 : -1);
+  bool k2 = false;
+  int nseg = 1, sets = 1;
+  plan_linear_batch_split(M, K, N, bits, group_size, &k2, &nseg, &sets);
+  const Args a{x, codes, nullptr, scale, nullptr, static_cast<int>(M), static_cast<int>(K),
+               static_cast<int>(N), gshift, 0, stream, nullptr, WOL_ACT_NONE, nseg, static_cast<float*>(ws)};
+  if (dtype == WOL_DTYPE_BF16) {
+    if (bits == 8) launch_split_g<WOL_DTYPE_BF16, 8>(a, sets, k2); else launch_split_g<WOL_DTYPE_BF16, 4>(a, sets, k2);
+  } else {
+    if (bits == 8) launch_split_g<WOL_DTYPE_F16, 8>(a, sets, k2); else launch_split_g<WOL_DTYPE_F16, 4>(a, sets, k2);
+  }
+  if (const int rc = check_launch(); rc != WOL_OK) return rc;
+  return launch_reduce_partials(static_cast<const float*>(ws), nseg, bias, dtype, out, out_f32, M, N, f.act, stream);
 }
 
 }  // namespace wol

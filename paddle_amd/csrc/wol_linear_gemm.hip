@@ -1218,6 +1218,21 @@ void launch_cfg(const Args& a) {
 
 }  // namespace
 
+int launch_reduce_partials(const float* part, int nsplit, const void* bias, int dtype, void* out,
+                           bool out_f32, int64_t M, int64_t N, int act, hipStream_t stream) {
+  const int64_t total = M * N;
+  const dim3 grid(static_cast<unsigned>((total / 4 + 255) / 256)), block(256);
+  if (dtype == WOL_DTYPE_BF16)
+    reduce_partials_kernel<WOL_DTYPE_BF16><<<grid, block, 0, stream>>>(
+        part, nsplit, static_cast<const uint16_t*>(bias), out, out_f32 ? 1 : 0, total, static_cast<int>(N), 0,
+        static_cast<int>(N), act);
+  else
+    reduce_partials_kernel<WOL_DTYPE_F16><<<grid, block, 0, stream>>>(
+        part, nsplit, static_cast<const uint16_t*>(bias), out, out_f32 ? 1 : 0, total, static_cast<int>(N), 0,
+        static_cast<int>(N), act);
+  return check_launch();
+}
+
 size_t linear_gemm_workspace(int64_t M, int64_t K, int64_t N, int bits, int group_size) {
   const int tk = bits == 8 ? 64 : 128;
   if (K % tk != 0 || K / tk < 2) return 0;

@@ -58,7 +58,8 @@ def quantize_llm_int8(w_bits, dt, g, layout=1):
 def linear(x_bits, codes_u8, bias_bits, scale_bits, dt, N, bits, g, f32=False, no_workspace=False,
            kernel=None, ws_bytes=None):
     """codes_u8 in gfx950 layout.  Returns fp32 numpy [M,N] (f32=True) or T bits.
-    kernel pins the streaming (1) or GEMM (2) kernel through wol_linear_on;
+    kernel pins a wol_kernel (streaming 1, GEMM 2, batched 3, batched with K
+    runs 4) through wol_linear_on;
     ws_bytes overrides the size of the scratch buffer handed in."""
     x = H.bits_to_torch(x_bits, dt, DEV)
     M, K = x.shape
@@ -85,6 +86,15 @@ def linear(x_bits, codes_u8, bias_bits, scale_bits, dt, N, bits, g, f32=False, n
         _lib.check(_lib.lib.wol_linear_on(*args, 1 if f32 else 0, kernel, *tail))
     torch.cuda.synchronize()
     return out.cpu().numpy() if f32 else H.torch_to_bits(out)
+
+
+def linear_plan(M, K, N, bits, g, ws_bytes):
+    """What wol_linear would launch for the problem, given ws_bytes of scratch."""
+    import ctypes
+
+    buf = ctypes.create_string_buffer(512)
+    _lib.check(_lib.lib.wol_linear_plan(M, K, N, bits, g, ws_bytes, buf, 512))
+    return buf.value.decode()
 
 
 def llm_int8_linear(x_bits, w_nk, bias_bits, wscale, threshold, dt, stages=False):

@@ -82,7 +82,53 @@ def test_linear_batch_kernel_pinned(G, oracle, dt, bits, g):
         check(G, oracle, dt, bits, g, 4, 1024, 256, seed=1, kernel=KERNEL_BATCH)
 
 
-@pytest.mark.parametrize("kernel", [KERNEL_STREAM, KERNEL_BATCH, KERNEL_GEMM])
+KERNEL_BATCH_SPLIT = 4
+
+
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("g", [-1, 64, 128])
+def test_linear_batch_split_kernel_pinned(G, oracle, dt, bits, g):
+    # the batched decode kernel with K cut into runs across workgroups: K that
+    # fills its runs exactly (2048, 4096), K whose last run is mostly past the
+    # end (one tile more than a run; 11008), K long enough for the 256-k runs
+    # (14336); fewer strips than strip sets, more strips per set than one LDS
+    # run holds; N that is 16 mod 32; 1 to 16 rows and the two-operand form up
+    # to 32
+    tk = 64 if bits == 8 else 128
+    shapes = [(2048, 1024), (2048 + tk, 4128), (4096, 272), (11008, 528), (14336, 272), (2048, 48), (2048, 36880)]
+    for K, N in shapes:
+        for M in ((1, 2, 5, 16, 17, 24, 32) if K * N < 5e6 else ((3, 16, 31) if K * N < 5e7 else (7, 20))):
+            print("case", dt, bits, g, K, N, M, flush=True)
+            check(G, oracle, dt, bits, g, M, K, N, bias=(M % 2 == 1), seed=M, kernel=KERNEL_BATCH_SPLIT)
+    # refused: more than 32 rows, fewer than 16 weight tiles, a K that ends in
+    # half a tile (int4), scratch that is too small
+    with pytest.raises(ValueError):
+        check(G, oracle, dt, bits, g, 33, 2048, 256, seed=1, kernel=KERNEL_BATCH_SPLIT)
+    with pytest.raises(ValueError):
+        check(G, oracle, dt, bits, g, 4, 15 * tk, 256, seed=1, kernel=KERNEL_BATCH_SPLIT)
+    if bits == 4:
+        with pytest.raises(ValueError):
+            check(G, oracle, dt, bits, g, 4, 2048 + 64, 256, seed=1, kernel=KERNEL_BATCH_SPLIT)
+    with pytest.raises(ValueError):
+        check(G, oracle, dt, bits, g, 4, 4096, 256, seed=1, kernel=KERNEL_BATCH_SPLIT, ws_bytes=4 * 256 * 4)
+
+
+def test_linear_takes_the_split_batch_kernel_where_it_is_measured_faster(G, oracle):
+    # the dispatcher's choice (named by wol_linear_plan), with and without the
+    # scratch that kernel needs, and the same call checked against the oracle
+    big = 1 << 30
+    assert "K runs" in G.linear_plan(12, 13824, 5120, 4, 128, big)       # ragged last round of strips
+    assert "K runs" in G.linear_plan(16, 14336, 4096, 4, -1, big)        # int4, long K
+    assert "K runs" in G.linear_plan(24, 4096, 11008, 8, 64, big)        # two 16-row operands, int8
+    assert "K runs" not in G.linear_plan(12, 13824, 5120, 4, 128, 0)     # no scratch: one of the others
+    assert "K runs" not in G.linear_plan(4, 13824, 5120, 4, 128, big)    # few rows: the streaming kernel
+    assert "K runs" not in G.linear_plan(12, 4096, 11008, 4, 128, big)   # the one-launch batched kernel
+    check(G, oracle, H.BF16, 4, 128, 12, 6144, 384 * 16, seed=2)
+    check(G, oracle, H.F16, 8, 64, 24, 4096, 5120, seed=3)
+
+
+@pytest.mark.parametrize("kernel", [KERNEL_STREAM, KERNEL_BATCH, KERNEL_BATCH_SPLIT, KERNEL_GEMM])
 @pytest.mark.parametrize("dt", [H.F16, H.BF16])
 def test_linear_int4_offset_cancellation_with_biased_activations(G, oracle, dt, kernel):
     # activations that are all positive (what follows a gelu or a relu) make the

@@ -70,11 +70,16 @@ def test_workspace_queries(lib):
     # 384 tiles: the 256 of the whole round run as they are, the other 128 (4096 columns) in two K runs
     assert L.wol_linear_workspace(1024, 4096, 12288, 8, 64) == 2 * 1024 * 4096 * 4
     # small M on the GEMM: whole fp32 [M, N] partial buffers, at most 16 of them
-    for M, K, N, bits, g in [(64, 8192, 28672, 4, 128), (32, 4096, 11008, 4, -1), (24, 8192, 28672, 4, 128)]:
+    for M, K, N, bits, g in [(64, 8192, 28672, 4, 128), (48, 4096, 11008, 4, -1), (24, 8192, 28672, 4, 128)]:
         need = L.wol_linear_workspace(M, K, N, bits, g)
         assert need == L.wol_linear_workspace_for(M, K, N, bits, g, lib.KERNEL_GEMM)
         assert need % (M * N * 4) == 0 and 2 <= need // (M * N * 4) <= 16, (M, K, N, need)
-    assert L.wol_linear_workspace(16, 8192, 28672, 4, 128) == 0  # up to 16 rows: always the streaming kernel
+    # the batched kernel with K runs: one fp32 [M, N] buffer per run (K / 2048, or K / 4096 from 13824 on)
+    assert L.wol_linear_workspace(32, 4096, 11008, 4, -1) == 2 * 32 * 11008 * 4
+    assert L.wol_linear_workspace(12, 13824, 5120, 4, 128) == 4 * 12 * 5120 * 4
+    assert L.wol_linear_workspace_for(4, 4096, 4096, 8, 64, lib.KERNEL_BATCH_SPLIT) == 2 * 4 * 4096 * 4
+    assert L.wol_linear_workspace_for(33, 4096, 4096, 8, 64, lib.KERNEL_BATCH_SPLIT) == 0  # not built for 33 rows
+    assert L.wol_linear_workspace(16, 8192, 28672, 4, 128) == 0  # the one-launch batched kernel
     assert L.wol_linear_workspace_for(16, 8192, 28672, 4, 128, lib.KERNEL_GEMM) > 0
     assert L.wol_linear_workspace_for(16, 4096, 11008, 4, 128, lib.KERNEL_STREAM) == 0
     assert L.wol_linear_workspace_for(16, 4160, 11008, 4, 128, lib.KERNEL_GEMM) == 0  # K not a multiple of the k tile
