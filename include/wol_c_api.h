@@ -170,8 +170,10 @@ size_t wol_linear_workspace(int64_t M, int64_t K, int64_t N, int bits,
  * the activations once per workgroup, where it applies (2 to 16 rows, K =
  * 2048/4096/8192, at least two 16-column strips per CU), else the streaming
  * one --, M > 64 the MFMA GEMM, and in between the streaming kernel or the
- * GEMM, whichever a cost model predicts to be faster; the reference's split
- * is M <= 3 (gpu/weight_only_linear_kernel.cu:60-61).
+ * GEMM, whichever a cost model predicts to be faster.  Where the workspace
+ * allows and it is measured faster (10 to 32 rows on some shapes), the
+ * batched kernel with K cut into runs across workgroups runs instead.  The
+ * reference's split is M <= 3 (gpu/weight_only_linear_kernel.cu:60-61).
  * x, codes and scale must be 16-byte aligned.
  */
 int wol_linear(const void* x, const void* codes, const void* bias,
