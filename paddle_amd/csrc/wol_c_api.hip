@@ -121,7 +121,8 @@ bool use_batch(int64_t M, int64_t K, int64_t N, int bits, int group_size) {
 //    a K the one-launch batched kernel is not built for, and strips that
 //    leave the CUs a ragged last round (N / 16 / CUs is 1.1 or more below
 //    its ceiling: N = 5120 ... 7168 on 256 CUs), by 10 to 49 %; int4 with
-//    K >= 14336 from 12 rows on also with whole rounds (9 to 18 %);
+//    K >= 14336 from 12 rows on also with whole rounds (9 to 18 %), and with
+//    K >= 11008 at 16 rows (4 to 13 %);
 //  * from 17 to 32 rows (two 16-row operands) it beats the better of the
 //    streaming kernel and the MFMA GEMM on int8 weights of 20 MB and more by
 //    5 to 20 %, and on int4 weights of 10 to 34 MB by up to 17 %.
@@ -137,7 +138,7 @@ bool use_batch_split(int64_t M, int64_t K, int64_t N, int bits, int group_size, 
   const double rounds = static_cast<double>(nstrips) / cus;
   const double ragged = static_cast<double>((nstrips + cus - 1) / cus) / rounds;
   if (ragged >= 1.1) return true;
-  return bits == 4 && M >= 12 && K >= 14336;
+  return bits == 4 && ((M >= 12 && K >= 14336) || (M >= 16 && K >= 11008));
 }
 
 // kernel: a wol_kernel; AUTO resolves by M and the cost model.  Returns the
