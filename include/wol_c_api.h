@@ -168,7 +168,7 @@ size_t wol_linear_workspace(int64_t M, int64_t K, int64_t N, int bits,
  * scale: [N] T (group_size -1) or [ceil(K/g),N] T, as wol_quantize wrote it.
  * M <= 16 takes a decode (HBM-bound) kernel -- the batched one, which fetches
  * the activations once per workgroup, where it applies (2 to 16 rows, K =
- * 2048/4096/8192, at least two 16-column strips per CU), else the streaming
+ * 2048/4096/8192, at least 2.5 16-column strips per CU), else the streaming
  * one --, M > 64 the MFMA GEMM, and in between the streaming kernel or the
  * GEMM, whichever a cost model predicts to be faster.  Where the workspace
  * allows and it is measured faster (10 to 32 rows on some shapes), the

@@ -100,16 +100,19 @@ bool use_stream(int64_t M, int64_t K, int64_t N, int bits, bool have_ws) {
 
 // The batched decode kernel (a workgroup per CU that owns N / 16 / CUs strips
 // and fetches the activations once for all of them) against the streaming
-// kernel (a workgroup per strip): measured on MI355X over K = 4096 and 8192,
-// N from 4096 to 28672, both bit widths, it wins from two strips per CU on
-// when the streaming kernel's activation reads weigh in -- 5 rows and more
-// (16-row and 8-row operands) and 2 rows (whose operands share the least) --
-// and for 3 and 4 rows from five strips per CU on; with one strip per CU the
-// streaming kernel has the shorter critical path at every row count.
+// kernel (a workgroup per strip): measured on MI355X over K = 2048, 4096 and
+// 8192, N from 4096 to 28672, both bit widths, it wins from 2.5 strips per CU
+// on when the streaming kernel's activation reads weigh in -- 5 rows and more
+// (16-row and 8-row operands) -- by up to 30 %; for 3 and 4 rows from 3.5
+// strips per CU on, for 2 rows from 2.5 (int4) or 5 (int8).  With exactly two
+// strips per CU (N = 8192 on 256 CUs) and with one the streaming kernel has
+// the shorter critical path at every row count (by 2 to 40 %).
 bool use_batch(int64_t M, int64_t K, int64_t N, int bits, int group_size) {
   if (M < 2 || M > 16 || !wol::linear_batch_supports(M, K, bits, group_size)) return false;
-  const int64_t per_cu = N / wol::kStripCols / wol::linear_batch_cus();
-  return (M == 3 || M == 4) ? per_cu >= 5 : per_cu >= 2;
+  const double per_cu = static_cast<double>(N / wol::kStripCols) / wol::linear_batch_cus();
+  if (M == 3 || M == 4) return per_cu >= 3.5;
+  if (M == 2) return per_cu >= (bits == 4 ? 2.5 : 5.0);
+  return per_cu >= 2.5;
 }
 
 // The batched decode kernel with K cut into runs across workgroups (two
