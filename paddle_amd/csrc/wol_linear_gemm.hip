@@ -21,6 +21,7 @@
 #include "wol_dequant.h"
 
 #include <climits>
+#include <type_traits>
 
 namespace wol {
 namespace {
@@ -806,20 +807,27 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(
   if (i >= total) return;
   const int64_t o = i / ncols * N + col0 + i % ncols;  // position in out
   f32x4 s = {0.f, 0.f, 0.f, 0.f};
-  for (int r0 = 0; r0 < nsplit; r0 += 4) {  // four loads in flight, added in run order
-    f32x4 v[4];
+  // W loads in flight at a time (past the last run: the last run again, not
+  // added), added in run order: one trip to memory for up to W runs
+  auto add_runs = [&](auto width) {
+    constexpr int W = decltype(width)::value;
+    for (int r0 = 0; r0 < nsplit; r0 += W) {
+      f32x4 v[W];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int r = r0 + u < nsplit ? r0 + u : nsplit - 1;
-      v[u] = *reinterpret_cast<const f32x4*>(part + r * total + i);
-    }
-#pragma unroll
-    for (int u = 0; u < 4; ++u)
-      if (r0 + u < nsplit) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) s[e] += v[u][e];
+      for (int u = 0; u < W; ++u) {
+        const int r = r0 + u < nsplit ? r0 + u : nsplit - 1;
+        v[u] = *reinterpret_cast<const f32x4*>(part + r * total + i);
       }
-  }
+#pragma unroll
+      for (int u = 0; u < W; ++u)
+        if (r0 + u < nsplit) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) s[e] += v[u][e];
+        }
+    }
+  };
+  if (nsplit <= 4) add_runs(std::integral_constant<int, 4>());
+  else add_runs(std::integral_constant<int, 8>());
   if (bias != nullptr) {
     const int n = col0 + static_cast<int>(i % ncols);
 #pragma unroll

@@ -661,7 +661,7 @@ def test_call_log_names_the_kernel(device):
     code = (
         "import torch\n"
         "from paddle_amd.nn import quant as Q\n"
-        "w = (torch.randn(2048, 8192, device='cuda') * 0.02).to(torch.bfloat16)\n"
+        "w = (torch.randn(2048, 12288, device='cuda') * 0.02).to(torch.bfloat16)\n"
         "c, s = Q.weight_quantize(w, algo='weight_only_int8')\n"
         "for M in (1, 8, 300):\n"
         "    Q.weight_only_linear(torch.randn(M, 2048, device='cuda').to(torch.bfloat16), c, None, s, 'int8')\n"
@@ -673,7 +673,7 @@ def test_call_log_names_the_kernel(device):
     assert r.returncode == 0, r.stderr[-2000:]
     lines = [ln for ln in r.stderr.splitlines() if ln.startswith("[wol] linear ")]
     assert len(lines) == 3
-    assert "M=1 K=2048 N=8192 int8" in lines[0] and lines[0].endswith("-> stream kernel")
+    assert "M=1 K=2048 N=12288 int8" in lines[0] and lines[0].endswith("-> stream kernel")
     assert lines[1].endswith("-> batch kernel") and lines[2].endswith("-> gemm kernel")
 
 

@@ -77,7 +77,7 @@ def _fused(x_bits, pre_bits, packed, bias_bits, scale_bits, dt, N, bits, g, act)
 # rows x (K, N): one row (streaming kernel), a small batch on a K and N the
 # batched decode kernel takes, and row counts / shapes that go to the streaming
 # kernel with several rows and to the GEMM
-SHAPES = [(1, 512, 256), (1, 4096, 1024), (8, 2048, 8192), (5, 4096, 8704), (3, 512, 256), (40, 1024, 512),
+SHAPES = [(1, 512, 256), (1, 4096, 1024), (8, 2048, 12288), (5, 4096, 10272), (3, 512, 256), (40, 1024, 512),
           (100, 512, 1024)]
 
 
