@@ -63,8 +63,12 @@ bool layout_ok(int layout) {
 // batched decode kernel, where it applies, is chosen before either, see
 // use_batch); from 17 to 64 rows
 // the cheaper of the two by a linear cost model runs (microseconds, least
-// squares over those measurements on MI355X; it picks the slower kernel in 2
-// of 96 cases, by 16 %).
+// squares of the relative error over 648 measurements on MI355X: 18 shapes
+// with K, N from 2048 to 28672, four weight formats, nine row counts; the
+// streaming kernel only where K is a power of two -- elsewhere its wavefronts
+// walk their units instead of loading them at once and the GEMM won every
+// case.  The choice costs 0.2 % of the total time of those cases against
+// always taking the faster kernel, 23 % in the worst case).
 constexpr int64_t kStreamMaxM = 64;
 constexpr int64_t kStreamAlwaysM = 16;
 
@@ -82,7 +86,7 @@ bool use_stream(int64_t M, int64_t K, int64_t N, int bits, bool have_ws) {
   // 16-row operands they are padded to (padding rows repeat the last row)
   const double a = static_cast<double>(N / 16) * M * K * 2.0 * 1e-6;
   const double a_pad = static_cast<double>(N / 16) * ((M + 15) / 16 * 16) * K * 2.0 * 1e-6;
-  const double t_stream = 3.0 + 0.0132 * w + 0.0829 * a + 0.0296 * a_pad;
+  const double t_stream = 2.908 + 0.0305 * w + 0.0914 * a + 0.0238 * a_pad;
   // two launches; K runs of a few k tiles each; fp32 partial sums written and
   // read back (M * N); MFMA work of the 32- or 64-row tile
   const double tile_rows = bits == 4 && M <= 32 ? 32.0 : 64.0;
@@ -93,8 +97,9 @@ bool use_stream(int64_t M, int64_t K, int64_t N, int bits, bool have_ws) {
     const double rounds = static_cast<double>((N / 256 + 511) / 512);  // two workgroups fit a CU
     return t_stream <= 3.0 + tiles * (bits == 4 && M > 32 ? 1.17 : 0.75) * rounds;
   }
-  const double t_gemm = 11.2 + (bits == 8 ? 0.035 : 0.0014) * w + 7.04 * (M * N * 1e-6) +
-                        2.184 * (tile_rows * N * K * 1e-9);
+  if ((K & (K - 1)) != 0) return false;
+  const double t_gemm = 10.232 + (bits == 8 ? 0.0622 : 0.0445) * w + 2.047 * (M * N * 1e-6) +
+                        2.2896 * (tile_rows * N * K * 1e-9);
   return t_stream <= t_gemm;
 }
 
