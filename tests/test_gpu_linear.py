@@ -478,7 +478,8 @@ def test_calls_replay_correctly_from_a_hip_graph(device):
 
 
 def test_fused_grad_moe_and_batched_decode_replay_from_a_hip_graph(device):
-    # the same for the batched decode kernel, the fused linear (pre-scale folded
+    # the same for the batched decode kernel (in one launch, and with K runs and
+    # the kernel that adds them), the fused linear (pre-scale folded
     # into the loads, gelu, swiglu through its pass), weight_only_linear_grad
     # (its prepare launches and the GEMM) and the MoE expert FFN (table built on
     # the device): replayed three times with eager work in between
@@ -487,12 +488,13 @@ def test_fused_grad_moe_and_batched_decode_replay_from_a_hip_graph(device):
     from paddle_amd.nn.quant import quantized_linear as QL
 
     dev = torch.device("cuda:0")
-    K, N = 2048, 8192
+    K, N = 2048, 12288
     gen = torch.Generator(device="cuda").manual_seed(4)
     w = (torch.randn(K, N, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
     codes, scale = Q.weight_quantize(w, algo="weight_only_int8", group_size=64)
     c4, s4 = Q.weight_quantize(w, algo="weight_only_int4", group_size=-1)
     xs = {M: torch.randn(M, K, device=dev, generator=gen).to(torch.bfloat16) for M in (1, 8, 200)}
+    x24 = torch.randn(24, K, device=dev, generator=gen).to(torch.bfloat16)
     pre = (0.5 + torch.rand(K, device=dev, generator=gen)).to(torch.bfloat16)
     gos = {M: torch.randn(M, N, device=dev, generator=gen).to(torch.bfloat16) for M in (8, 300)}
     E, hidden, inter = 4, 256, 512
@@ -505,6 +507,7 @@ def test_fused_grad_moe_and_batched_decode_replay_from_a_hip_graph(device):
 
     def work():
         outs = [Q.weight_only_linear(xs[8], codes, None, scale, "int8", None, 64)]  # batched decode kernel
+        outs.append(Q.weight_only_linear(x24, codes, None, scale, "int8", None, 64))  # the same with K runs + reduce
         for M, x in xs.items():
             outs.append(Q.weight_only_linear_fused(x, codes, None, scale, "int8", 64, pre_scale=pre, act="gelu"))
             outs.append(Q.weight_only_linear_fused(x, c4, None, s4, "int4", -1, pre_scale=None, act="swiglu"))
