@@ -290,6 +290,70 @@ def bench_linear_grad(torch, np, Q, _lib, H, dev, quick, failures):
             "rows": rows, "rel_l2_vs_oracle": err, "parity_sample": "first 4 rows of the M=2048 result"}
 
 
+def bench_moe_ffn(torch, np, Q, H, dev, quick, failures):
+    """moe_ffn on weight-only int8 experts of Mixtral-8x7B's size (8 experts,
+    hidden 4096, fc1 width 2 x 14336 for swiglu, bf16): a prefill-like call
+    (4096 rows in expert order, 512 per expert; MFMA-bound) and a decode-like
+    one (128 rows, 16 per expert; bound by the 1.4 GB of expert weights every
+    call streams).  Two rows of one expert are checked against the oracle (the
+    oracle's linear, swiglu on its rounded output, the oracle's linear)."""
+    E, hidden, inter = 8, 4096, 28672
+    bf16, dt = torch.bfloat16, H.BF16
+    q1, s1, q2, s2 = [], [], [], []
+    for e in range(E):
+        c, s = _quantize(Q, _device_weight(torch, hidden, inter, bf16, 500 + e, dev), 8, -1)
+        q1.append(c); s1.append(s)
+        c, s = _quantize(Q, _device_weight(torch, inter // 2, hidden, bf16, 600 + e, dev), 8, -1)
+        q2.append(c); s2.append(s)
+    q1, s1, q2, s2 = torch.stack(q1), torch.stack(s1), torch.stack(q2), torch.stack(s2)
+    wbytes = E * (hidden * inter + inter // 2 * hidden)
+    rows_out = []
+    sample = None
+    for rows in ((4096,) if quick else (4096, 128)):
+        gen = torch.Generator(device=dev)
+        gen.manual_seed(rows)
+        x = torch.randn((rows, hidden), generator=gen, device=dev, dtype=torch.float32).to(bf16)
+        cum = torch.arange(1, E + 1, device=dev, dtype=torch.int64) * (rows // E)
+        holder = {}
+
+        def step(_i):
+            holder["out"] = Q.moe_ffn(x, cum, q1, q2, None, s1, s2, "weight_only_int8")
+
+        n = 2 if rows >= 1024 else 4
+        med, mn = time_graph(torch, step, n, warm_launches=8, warm_ms=30.0, replays=5)
+        t = med / n
+        flops = 2.0 * rows * hidden * inter + 2.0 * rows * (inter // 2) * hidden
+        entry = {"rows": rows, "rows_per_expert": rows // E, "ms": round(t * 1e3, 4), "ms_min": round(mn / n * 1e3, 4)}
+        if rows >= 1024:
+            tf = flops / t / 1e12
+            entry.update({"bound": "mfma", "achieved": round(tf, 1), "unit": "TFLOP/s",
+                          "frac": round(tf / MFMA_BF16_PEAK_TF, 4)})
+        else:
+            gbs = wbytes / t / 1e9
+            entry.update({"bound": "hbm", "achieved": round(gbs, 1), "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4)})
+        rows_out.append(entry)
+        if rows == 4096:
+            step(0)
+            torch.cuda.synchronize()
+            e_s, r0 = 3, 3 * (rows // E)  # two rows of expert 3
+            sample = (H.torch_to_bits(x[r0:r0 + 2]), H.torch_to_bits(holder["out"][r0:r0 + 2]), e_s)
+    xb, got, e_s = sample
+    O = H.O
+    c1, sc1 = O.weight_quantize(H.torch_to_bits(_device_weight(torch, hidden, inter, bf16, 500 + e_s, dev)), dt, 8, -1)
+    c2, sc2 = O.weight_quantize(H.torch_to_bits(_device_weight(torch, inter // 2, hidden, bf16, 600 + e_s, dev)), dt, 8, -1)
+    _, fc1 = O.linear(xb, c1, sc1, None, dt, 8, -1)
+    _, act = O.activation(H.bits_to_f32(fc1, dt), O.ACT_SWIGLU, dt)
+    _, want = O.linear(act, c2, sc2, None, dt, 8, -1)
+    err = H.rel_l2(H.bits_to_f32(got, dt), H.bits_to_f32(want, dt))
+    if err > REL_L2_BAR:
+        failures.append("moe_ffn output differs from the oracle")
+    return {"workload": "moe_ffn, 8 experts, hidden 4096, fc1 width 28672 (swiglu to 14336), int8 per-channel, bf16; "
+                        "rows in expert order, the same number per expert",
+            "launches_per_call": "tile table, grouped GEMM, swiglu pass, grouped GEMM",
+            "weight_bytes": wbytes, "rows": rows_out, "rel_l2_vs_oracle": err,
+            "parity_sample": "two rows of expert 3 of the 4096-row call"}
+
+
 def _plan_grad(_lib, M, K, N):
     import ctypes
     buf = ctypes.create_string_buffer(256)
@@ -514,13 +578,15 @@ def main():
         }
 
     # ---------------- every BASELINE configuration ----------------
-    configs = stack = grad = None
+    configs = stack = grad = moe = None
     if not args.no_configs:
         del copies, scales
         torch.cuda.empty_cache()
         configs = bench_configs(torch, Q, _lib, dev, args.quick)
         stack = bench_decoder_stack(torch, Q, _lib, dev, args.quick)
         grad = bench_linear_grad(torch, np, Q, _lib, H, dev, args.quick, failures)
+        torch.cuda.empty_cache()
+        moe = bench_moe_ffn(torch, np, Q, H, dev, args.quick, failures)
 
     # ---------------- parity of what was measured, against the oracle ----------------
     O = H.O
@@ -632,6 +698,7 @@ def main():
         "configs": configs,
         "decoder_stack": stack,
         "linear_grad": grad,
+        "moe_ffn": moe,
         "llm_int8": llm,
         "cpu_baseline": cpu,
         "parity": parity,
