@@ -1175,17 +1175,27 @@ __global__ __launch_bounds__(256) void moe_plan_kernel(const int64_t* __restrict
   }
 }
 
-constexpr int kMoeTileRows = 128;
+// Rows of a grouped launch's tiles, by the average number of rows per expert
+// (the host knows the total only; the per-expert counts stay on the device):
+// 128 x 256 tiles, or the small-M configurations' 64 x 256 (32 x 256 for int4)
+// when the experts have few rows each -- a decode step of a mixture of
+// experts -- where the large tile would do up to eight times the MFMA work
+// and hold one workgroup per CU where three fit.
+inline int moe_tile_rows(int64_t rows, int num_experts, int bits) {
+  const int64_t avg = rows / (num_experts > 0 ? num_experts : 1);
+  if (avg <= 32 && bits == 4) return 32;
+  if (avg <= 64) return 64;
+  return 128;
+}
 
-// One grouped GEMM: every expert's rows against that expert's weights, 128 x
-// 256 tiles, per-channel scales, out [rows, N] T.
-template <int DT, int BITS>
-void launch_moe_gemm(const void* x, const int* table, int max_tiles, const void* codes, const void* bias,
-                     const void* scale, int64_t K, int64_t N, void* out, hipStream_t stream) {
-  constexpr bool kOffs = BITS == 4 && DT == WOL_DTYPE_BF16;  // as the ungrouped launch chooses
-  constexpr int WM = 2, WN = 4, TM = 2, TN = 2, BN = WN * TN * 32;
-  constexpr size_t lds = dma_lds_bytes<BITS, 0, WM, WN, TM, TN, 3>();
-  auto kern = gemm_dma_kernel<DT, BITS, 0, kOffs, WM, WN, TM, TN, 3>;
+// One grouped GEMM: every expert's rows against that expert's weights, tiles
+// of WM * TM * 32 rows x 256 columns, per-channel scales, out [rows, N] T.
+template <int DT, int BITS, bool OFFS, int WM, int WN, int TM, int TN, int STAGES>
+void launch_moe_gemm_cfg(const void* x, const int* table, int max_tiles, const void* codes, const void* bias,
+                         const void* scale, int64_t K, int64_t N, void* out, hipStream_t stream) {
+  constexpr int BN = WN * TN * 32;
+  constexpr size_t lds = dma_lds_bytes<BITS, 0, WM, WN, TM, TN, STAGES>();
+  auto kern = gemm_dma_kernel<DT, BITS, 0, OFFS, WM, WN, TM, TN, STAGES>;
   static std::atomic<uint32_t> configured{0};
   allow_lds(reinterpret_cast<const void*>(kern), lds, configured);
   DmaParams p;
@@ -1194,7 +1204,7 @@ void launch_moe_gemm(const void* x, const int* table, int max_tiles, const void*
   p.bias = static_cast<const uint16_t*>(bias);
   p.scale = static_cast<const uint16_t*>(scale);
   p.out = out;
-  p.M = kMoeTileRows; p.K = static_cast<int>(K); p.N = static_cast<int>(N);
+  p.M = WM * TM * 32; p.K = static_cast<int>(K); p.N = static_cast<int>(N);
   p.out_f32 = 0;
   p.strip_lo = 0; p.strip_hi = static_cast<int>(N / kStripCols);
   p.nbx = static_cast<int>((N + BN - 1) / BN);
@@ -1206,6 +1216,23 @@ void launch_moe_gemm(const void* x, const int* table, int max_tiles, const void*
   p.moe_table = table;
   p.moe_codes_stride = K * N * BITS / 8;
   kern<<<dim3(static_cast<unsigned>(p.nbx * p.nby)), dim3(64 * WM * WN), lds, stream>>>(p);
+}
+
+// bm: the tile rows the table was built for (moe_tile_rows)
+template <int DT, int BITS>
+void launch_moe_gemm(const void* x, const int* table, int max_tiles, int bm, const void* codes, const void* bias,
+                     const void* scale, int64_t K, int64_t N, void* out, hipStream_t stream) {
+  constexpr bool kOffs = BITS == 4 && DT == WOL_DTYPE_BF16;  // as the ungrouped launch chooses
+  if constexpr (BITS == 4) {
+    if (bm == 32) {
+      launch_moe_gemm_cfg<DT, 4, true, 1, 8, 1, 1, 2>(x, table, max_tiles, codes, bias, scale, K, N, out, stream);
+      return;
+    }
+  }
+  if (bm == 64)
+    launch_moe_gemm_cfg<DT, BITS, false, 1, 8, 2, 1, 2>(x, table, max_tiles, codes, bias, scale, K, N, out, stream);
+  else
+    launch_moe_gemm_cfg<DT, BITS, kOffs, 2, 4, 2, 2, 3>(x, table, max_tiles, codes, bias, scale, K, N, out, stream);
 }
 
 template <int DT, int BITS>
@@ -1308,12 +1335,15 @@ int launch_linear_gemm(const void* x, const void* codes, const void* bias, const
 // Scratch: [row-tile table][fc1 output rows x inter T][activation rows x inter/2 T]
 static size_t moe_up(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
 
-int moe_max_tiles(int64_t rows, int num_experts) {
-  return static_cast<int>((rows + kMoeTileRows - 1) / kMoeTileRows) + num_experts;
+// Entries of the row-tile table for tiles of bm rows: every expert may end in
+// a partial tile.
+static int moe_max_tiles(int64_t rows, int num_experts, int bm) {
+  return static_cast<int>((rows + bm - 1) / bm) + num_experts;
 }
 
 size_t moe_ffn_workspace(int64_t rows, int64_t inter, int num_experts) {
-  return moe_up(static_cast<size_t>(moe_max_tiles(rows, num_experts)) * sizeof(MoeTile)) +
+  // (the table at its longest: 32-row tiles)
+  return moe_up(static_cast<size_t>(moe_max_tiles(rows, num_experts, 32)) * sizeof(MoeTile)) +
          moe_up(static_cast<size_t>(rows) * inter * 2) + moe_up(static_cast<size_t>(rows) * (inter / 2) * 2);
 }
 
@@ -1322,18 +1352,19 @@ int launch_moe_ffn(const void* x, const int64_t* rows_before_expert, const void*
                    const void* ffn2_scale, int dtype, int64_t rows, int64_t hidden, int64_t inter,
                    int num_experts, int bits, void* out, void* workspace, hipStream_t stream) {
   unsigned char* ws = static_cast<unsigned char*>(workspace);
-  const int max_tiles = moe_max_tiles(rows, num_experts);
+  const int bm = moe_tile_rows(rows, num_experts, bits);
+  const int max_tiles = moe_max_tiles(rows, num_experts, bm);
   MoeTile* table = reinterpret_cast<MoeTile*>(ws);
-  unsigned char* fc1 = ws + moe_up(static_cast<size_t>(max_tiles) * sizeof(MoeTile));
+  unsigned char* fc1 = ws + moe_up(static_cast<size_t>(moe_max_tiles(rows, num_experts, 32)) * sizeof(MoeTile));
   unsigned char* act = fc1 + moe_up(static_cast<size_t>(rows) * inter * 2);
-  moe_plan_kernel<<<dim3(1), dim3(256), 0, stream>>>(rows_before_expert, num_experts, kMoeTileRows, max_tiles, table);
+  moe_plan_kernel<<<dim3(1), dim3(256), 0, stream>>>(rows_before_expert, num_experts, bm, max_tiles, table);
   const int* tb = reinterpret_cast<const int*>(table);
 #define WOL_MOE(DT, B)                                                                                        \
   do {                                                                                                        \
-    launch_moe_gemm<DT, B>(x, tb, max_tiles, ffn1_codes, ffn1_bias, ffn1_scale, hidden, inter, fc1, stream);  \
+    launch_moe_gemm<DT, B>(x, tb, max_tiles, bm, ffn1_codes, ffn1_bias, ffn1_scale, hidden, inter, fc1, stream);  \
     const int rc = launch_swiglu_t(fc1, dtype, rows, inter, act, stream);                                     \
     if (rc != WOL_OK) return rc;                                                                              \
-    launch_moe_gemm<DT, B>(act, tb, max_tiles, ffn2_codes, nullptr, ffn2_scale, inter / 2, hidden, out, stream); \
+    launch_moe_gemm<DT, B>(act, tb, max_tiles, bm, ffn2_codes, nullptr, ffn2_scale, inter / 2, hidden, out, stream); \
   } while (0)
   if (dtype == WOL_DTYPE_BF16) {
     if (bits == 8) WOL_MOE(WOL_DTYPE_BF16, 8); else WOL_MOE(WOL_DTYPE_BF16, 4);

@@ -28,15 +28,21 @@ def _oracle_moe(oracle, xb, cum, w1b, b1b, w2b, dt, bits):
     return out
 
 
+# rows per expert: none, a few, exactly one tile, a tile and a bit, many, none at
+# the end (128-row tiles); few rows per expert, with whole and partial tiles
+# and one expert far above the average (64-row tiles; 32-row tiles for int4);
+# an average of 38 rows (64-row tiles for both bit widths)
+ROWS_PER_EXPERT = [[0, 5, 128, 131, 300, 0], [0, 5, 33, 64, 1, 17], [40, 64, 0, 70, 3, 50], [2, 1, 150, 0, 3, 4]]
+
+
 @pytest.mark.parametrize("dt", [H.F16, H.BF16])
 @pytest.mark.parametrize("bits", [8, 4])
-def test_moe_ffn_against_oracle(device, oracle, dt, bits):
+@pytest.mark.parametrize("per", ROWS_PER_EXPERT)
+def test_moe_ffn_against_oracle(device, oracle, dt, bits, per):
     import torch
     from paddle_amd.nn import quant as Q
 
     hidden, inter, E = 256, 512, 6
-    # rows per expert: none, a few, exactly one tile, a tile and a bit, many, none at the end
-    per = [0, 5, 128, 131, 300, 0]
     cum = np.cumsum(per).astype(np.int64)
     rows = int(cum[-1]) + 3  # three rows that belong to no expert
     rng = np.random.default_rng(5)
