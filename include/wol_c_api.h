@@ -274,12 +274,15 @@ int wol_linear_grad_f32(const void* out_grad, const void* codes,
  * (GFX950 layout, per-channel scales): ffn1_weight [E] x (K = hidden,
  * N = inter), ffn1_scale [E, inter] T, ffn1_bias [E, inter] T or NULL,
  * ffn2_weight [E] x (K = inter/2, N = hidden), ffn2_scale [E, hidden] T.
- * Each of the two products is ONE grouped launch (128 x 256 tiles looked up
- * in a row-tile table that a one-workgroup kernel derives from
- * token_nums_per_expert); the swiglu between them is an element-wise pass.
+ * Each of the two products is ONE grouped launch (tiles looked up in a
+ * row-tile table that a one-workgroup kernel derives from
+ * token_nums_per_expert: 128 x 256, or 64 x 256 / 32 x 256 when rows /
+ * num_experts is at most 64 / 32, in which case the second product may run
+ * with K cut into runs and a kernel that adds them); the swiglu between them
+ * is an element-wise pass.
  * Requires hidden % 128 == 0, inter % 256 == 0, num_experts <= 1024; the
- * workspace (wol_moe_ffn_workspace bytes, 16-byte aligned) holds the table and
- * the two intermediate tensors.
+ * workspace (wol_moe_ffn_workspace bytes, 16-byte aligned) holds the table,
+ * the two intermediate tensors and the runs' sums.
  */
 size_t wol_moe_ffn_workspace(int64_t rows, int64_t hidden, int64_t inter,
                              int num_experts);

@@ -477,7 +477,7 @@ int check_moe(int64_t rows, int64_t hidden, int64_t inter, int num_experts) {
 
 size_t wol_moe_ffn_workspace(int64_t rows, int64_t hidden, int64_t inter, int num_experts) {
   if (check_moe(rows, hidden, inter, num_experts) != WOL_OK || rows == 0) return 0;
-  return wol::moe_ffn_workspace(rows, inter, num_experts);
+  return wol::moe_ffn_workspace(rows, hidden, inter, num_experts);
 }
 
 int wol_moe_ffn(const void* permute_input, const int64_t* token_nums_per_expert, const void* ffn1_weight,
@@ -495,7 +495,7 @@ int wol_moe_ffn(const void* permute_input, const int64_t* token_nums_per_expert,
   if (!aligned16(permute_input) || !aligned16(ffn1_weight) || !aligned16(ffn2_weight) || !aligned16(ffn1_scale) ||
       !aligned16(ffn2_scale) || !aligned16(ffn_out))
     return WOL_ERR_ALIGNMENT;
-  if (workspace == nullptr || workspace_bytes < wol::moe_ffn_workspace(rows, inter, num_experts))
+  if (workspace == nullptr || workspace_bytes < wol::moe_ffn_workspace(rows, hidden, inter, num_experts))
     return WOL_ERR_WORKSPACE;
   if (!aligned16(workspace)) return WOL_ERR_ALIGNMENT;
   if (const int dv = require_gfx950(); dv != WOL_OK) return dv;

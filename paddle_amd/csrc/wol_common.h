@@ -313,7 +313,7 @@ int launch_mfma_ceiling(const void* operands, int workgroups, int iters, float* 
 int launch_prescale(const void* x, const void* scales, int dtype, int64_t rows, int64_t cols,
                     void* out, hipStream_t stream);
 int launch_swiglu_t(const void* in, int dtype, int64_t M, int64_t N, void* out, hipStream_t stream);
-size_t moe_ffn_workspace(int64_t rows, int64_t inter, int num_experts);
+size_t moe_ffn_workspace(int64_t rows, int64_t hidden, int64_t inter, int num_experts);
 int launch_moe_ffn(const void* x, const int64_t* rows_before_expert, const void* ffn1_codes,
                    const void* ffn1_bias, const void* ffn1_scale, const void* ffn2_codes,
                    const void* ffn2_scale, int dtype, int64_t rows, int64_t hidden, int64_t inter,

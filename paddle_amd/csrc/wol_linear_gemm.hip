@@ -391,6 +391,7 @@ struct DmaParams {
   // bias (consecutive tensors, the strides below apart).  Null: one problem.
   const int* moe_table;
   int64_t moe_codes_stride;     // bytes between two experts' packed weights
+  int moe_rows;                 // rows of the whole grouped problem (the partial sums' row count)
 };
 
 // One entry of the row-tile table of a grouped launch.
@@ -486,7 +487,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
     const MoeTile t = reinterpret_cast<const MoeTile*>(p.moe_table)[by];
     if (t.expert < 0) return;
     x += static_cast<int64_t>(t.row0) * K;
-    outp = static_cast<uint16_t*>(outp) + static_cast<int64_t>(t.row0) * N;
+    if (p.nsplit > 1) outp = static_cast<float*>(outp) + static_cast<int64_t>(t.row0) * N;  // partial sums
+    else outp = static_cast<uint16_t*>(outp) + static_cast<int64_t>(t.row0) * N;
     codes += static_cast<int64_t>(t.expert) * p.moe_codes_stride;
     scale += static_cast<int64_t>(t.expert) * N;
     if (bias != nullptr) bias += static_cast<int64_t>(t.expert) * N;
@@ -753,7 +755,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
     // partial sums are kept compact: row length = the columns of this launch
     const int64_t ld = p.nsplit > 1 ? static_cast<int64_t>(p.strip_hi - p.strip_lo) * kStripCols : N;
     const int ncol0 = p.nsplit > 1 ? p.strip_lo * kStripCols : 0;
-    float* outf = static_cast<float*>(outp) + (p.nsplit > 1 ? static_cast<int64_t>(split) * M * ld : 0);
+    const int64_t run_rows = p.moe_table != nullptr ? p.moe_rows : M;  // rows of one run's partial sums
+    float* outf = static_cast<float*>(outp) + (p.nsplit > 1 ? static_cast<int64_t>(split) * run_rows * ld : 0);
 #pragma unroll
     for (int a = 0; a < TM; ++a)
 #pragma unroll
@@ -798,13 +801,16 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
 }
 
 // out[m, col0 + c] = T( sum over the runs of part[run][m][c] + bias[col0 + c] ) for the ncols
-// columns from col0 on; four columns per thread; total = M * ncols
+// columns from col0 on; four columns per thread; total = M * ncols.  valid_rows (may be null):
+// rows from *valid_rows on were never computed and are left alone.
 template <int DT>
 __global__ __launch_bounds__(256) void reduce_partials_kernel(
     const float* __restrict__ part, int nsplit, const uint16_t* __restrict__ bias,
-    void* __restrict__ out, int out_f32, int64_t total, int N, int col0, int ncols, int act) {
+    void* __restrict__ out, int out_f32, int64_t total, int N, int col0, int ncols, int act,
+    const int64_t* __restrict__ valid_rows = nullptr) {
   const int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
   if (i >= total) return;
+  if (valid_rows != nullptr && i / ncols >= *valid_rows) return;
   const int64_t o = i / ncols * N + col0 + i % ncols;  // position in out
   f32x4 s = {0.f, 0.f, 0.f, 0.f};
   // W loads in flight at a time (past the last run: the last run again, not
@@ -943,6 +949,7 @@ void launch_dma(const Args& a, int strip_lo, int strip_hi, int nsplit) {
   p.act = a.act;
   p.moe_table = nullptr;
   p.moe_codes_stride = 0;
+  p.moe_rows = 0;
   kern<<<dim3(static_cast<unsigned>(p.nbx * p.nby * p.nsplit)), dim3(64 * WM * WN), lds, a.stream>>>(p);
   if (nsplit > 1) {
     const int64_t total = static_cast<int64_t>(a.M) * ncols;
@@ -1188,11 +1195,25 @@ inline int moe_tile_rows(int64_t rows, int num_experts, int bits) {
   return 128;
 }
 
+// What a grouped launch needs besides the problem: the row-tile table, and
+// for K runs (ns > 1; bias must be null, the runs' sums have no expert) the
+// scratch for ns x rows x N floats and the device word that holds the number
+// of rows that belong to an expert.
+struct MoeLaunch {
+  const int* table;
+  int max_tiles, bm, ns;
+  int64_t rows;
+  float* partial;
+  const int64_t* valid_rows;
+};
+
 // One grouped GEMM: every expert's rows against that expert's weights, tiles
 // of WM * TM * 32 rows x 256 columns, per-channel scales, out [rows, N] T.
 template <int DT, int BITS, bool OFFS, int WM, int WN, int TM, int TN, int STAGES>
-void launch_moe_gemm_cfg(const void* x, const int* table, int max_tiles, const void* codes, const void* bias,
+void launch_moe_gemm_cfg(const void* x, const MoeLaunch& ml, const void* codes, const void* bias,
                          const void* scale, int64_t K, int64_t N, void* out, hipStream_t stream) {
+  const int* table = ml.table;
+  const int max_tiles = ml.max_tiles;
   constexpr int BN = WN * TN * 32;
   constexpr size_t lds = dma_lds_bytes<BITS, 0, WM, WN, TM, TN, STAGES>();
   auto kern = gemm_dma_kernel<DT, BITS, 0, OFFS, WM, WN, TM, TN, STAGES>;
@@ -1203,37 +1224,59 @@ void launch_moe_gemm_cfg(const void* x, const int* table, int max_tiles, const v
   p.codes = static_cast<const uint8_t*>(codes);
   p.bias = static_cast<const uint16_t*>(bias);
   p.scale = static_cast<const uint16_t*>(scale);
-  p.out = out;
+  const int tiles = static_cast<int>(K / (BITS == 8 ? 64 : 128));
+  const int ns = bias == nullptr && ml.partial != nullptr ? ml.ns : 1;
   p.M = WM * TM * 32; p.K = static_cast<int>(K); p.N = static_cast<int>(N);
   p.out_f32 = 0;
   p.strip_lo = 0; p.strip_hi = static_cast<int>(N / kStripCols);
   p.nbx = static_cast<int>((N + BN - 1) / BN);
   p.nby = max_tiles;
-  p.nsplit = 1;
-  p.tiles_per_split = static_cast<int>(K / (BITS == 8 ? 64 : 128));
+  p.tiles_per_split = (tiles + ns - 1) / ns;
+  p.nsplit = (tiles + p.tiles_per_split - 1) / p.tiles_per_split;
+  p.out = p.nsplit > 1 ? static_cast<void*>(ml.partial) : out;
   p.xcd_rows = 0;
   p.act = WOL_ACT_NONE;
   p.moe_table = table;
   p.moe_codes_stride = K * N * BITS / 8;
-  kern<<<dim3(static_cast<unsigned>(p.nbx * p.nby)), dim3(64 * WM * WN), lds, stream>>>(p);
+  p.moe_rows = static_cast<int>(ml.rows);
+  kern<<<dim3(static_cast<unsigned>(p.nbx * p.nby * p.nsplit)), dim3(64 * WM * WN), lds, stream>>>(p);
+  if (p.nsplit > 1) {
+    const int64_t total = ml.rows * N;
+    reduce_partials_kernel<DT><<<dim3(static_cast<unsigned>((total / 4 + 255) / 256)), dim3(256), 0, stream>>>(
+        ml.partial, p.nsplit, nullptr, out, 0, total, static_cast<int>(N), 0, static_cast<int>(N), WOL_ACT_NONE,
+        ml.valid_rows);
+  }
 }
 
-// bm: the tile rows the table was built for (moe_tile_rows)
+// ml.bm: the tile rows the table was built for (moe_tile_rows)
 template <int DT, int BITS>
-void launch_moe_gemm(const void* x, const int* table, int max_tiles, int bm, const void* codes, const void* bias,
+void launch_moe_gemm(const void* x, const MoeLaunch& ml, const void* codes, const void* bias,
                      const void* scale, int64_t K, int64_t N, void* out, hipStream_t stream) {
   constexpr bool kOffs = BITS == 4 && DT == WOL_DTYPE_BF16;  // as the ungrouped launch chooses
   if constexpr (BITS == 4) {
-    if (bm == 32) {
-      launch_moe_gemm_cfg<DT, 4, true, 1, 8, 1, 1, 2>(x, table, max_tiles, codes, bias, scale, K, N, out, stream);
+    if (ml.bm == 32) {
+      launch_moe_gemm_cfg<DT, 4, true, 1, 8, 1, 1, 2>(x, ml, codes, bias, scale, K, N, out, stream);
       return;
     }
   }
-  if (bm == 64)
-    launch_moe_gemm_cfg<DT, BITS, false, 1, 8, 2, 1, 2>(x, table, max_tiles, codes, bias, scale, K, N, out, stream);
+  if (ml.bm == 64)
+    launch_moe_gemm_cfg<DT, BITS, false, 1, 8, 2, 1, 2>(x, ml, codes, bias, scale, K, N, out, stream);
   else
-    launch_moe_gemm_cfg<DT, BITS, kOffs, 2, 4, 2, 2, 3>(x, table, max_tiles, codes, bias, scale, K, N, out, stream);
+    launch_moe_gemm_cfg<DT, BITS, kOffs, 2, 4, 2, 2, 3>(x, ml, codes, bias, scale, K, N, out, stream);
 }
+
+// K runs of a grouped launch with small tiles: as many as bring the workgroups
+// (column tiles x row tiles x runs) to the CU count, at most 4, each of at
+// least 8 k tiles.  The large tile is not split.
+inline int moe_runs(int64_t K, int64_t N, int bits, int bm, int max_tiles) {
+  if (bm >= 128) return 1;
+  const int64_t tiles = K / (bits == 8 ? 64 : 128), wgs = (N + 255) / 256 * max_tiles;
+  int ns = static_cast<int>((num_cus() + wgs - 1) / wgs);
+  ns = ns > 4 ? 4 : ns;
+  while (ns > 1 && tiles / ns < 8) --ns;
+  return ns < 1 ? 1 : ns;
+}
+constexpr int kMoeMaxRuns = 4;
 
 template <int DT, int BITS>
 void launch_cfg(const Args& a) {
@@ -1332,7 +1375,6 @@ int launch_linear_gemm(const void* x, const void* codes, const void* bias, const
 }
 
 // ---- mixture-of-experts FFN ---------------------------------------------------
-// Scratch: [row-tile table][fc1 output rows x inter T][activation rows x inter/2 T]
 static size_t moe_up(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
 
 // Entries of the row-tile table for tiles of bm rows: every expert may end in
@@ -1341,10 +1383,14 @@ static int moe_max_tiles(int64_t rows, int num_experts, int bm) {
   return static_cast<int>((rows + bm - 1) / bm) + num_experts;
 }
 
-size_t moe_ffn_workspace(int64_t rows, int64_t inter, int num_experts) {
-  // (the table at its longest: 32-row tiles)
+// Scratch: [row-tile table][fc1 output rows x inter T][activation rows x inter/2 T]
+// [fp32 sums of the second GEMM's K runs, rows x hidden each, when the tiles are small]
+size_t moe_ffn_workspace(int64_t rows, int64_t hidden, int64_t inter, int num_experts) {
+  // (the table at its longest: 32-row tiles; the runs' sums whenever either bit width would use small tiles)
+  const bool small = moe_tile_rows(rows, num_experts, 4) < 128;
   return moe_up(static_cast<size_t>(moe_max_tiles(rows, num_experts, 32)) * sizeof(MoeTile)) +
-         moe_up(static_cast<size_t>(rows) * inter * 2) + moe_up(static_cast<size_t>(rows) * (inter / 2) * 2);
+         moe_up(static_cast<size_t>(rows) * inter * 2) + moe_up(static_cast<size_t>(rows) * (inter / 2) * 2) +
+         (small ? moe_up(static_cast<size_t>(kMoeMaxRuns) * rows * hidden * sizeof(float)) : 0);
 }
 
 int launch_moe_ffn(const void* x, const int64_t* rows_before_expert, const void* ffn1_codes,
@@ -1357,14 +1403,18 @@ int launch_moe_ffn(const void* x, const int64_t* rows_before_expert, const void*
   MoeTile* table = reinterpret_cast<MoeTile*>(ws);
   unsigned char* fc1 = ws + moe_up(static_cast<size_t>(moe_max_tiles(rows, num_experts, 32)) * sizeof(MoeTile));
   unsigned char* act = fc1 + moe_up(static_cast<size_t>(rows) * inter * 2);
+  float* partial = reinterpret_cast<float*>(act + moe_up(static_cast<size_t>(rows) * (inter / 2) * 2));
+  // the second GEMM has hidden / 256 column tiles only: K (= inter / 2) in runs when the tiles are small
+  const MoeLaunch l1{reinterpret_cast<const int*>(table), max_tiles, bm, 1, rows, nullptr, nullptr};
+  const MoeLaunch l2{reinterpret_cast<const int*>(table), max_tiles, bm, moe_runs(inter / 2, hidden, bits, bm, max_tiles),
+                     rows, bm < 128 ? partial : nullptr, rows_before_expert + (num_experts - 1)};
   moe_plan_kernel<<<dim3(1), dim3(256), 0, stream>>>(rows_before_expert, num_experts, bm, max_tiles, table);
-  const int* tb = reinterpret_cast<const int*>(table);
 #define WOL_MOE(DT, B)                                                                                        \
   do {                                                                                                        \
-    launch_moe_gemm<DT, B>(x, tb, max_tiles, bm, ffn1_codes, ffn1_bias, ffn1_scale, hidden, inter, fc1, stream);  \
+    launch_moe_gemm<DT, B>(x, l1, ffn1_codes, ffn1_bias, ffn1_scale, hidden, inter, fc1, stream);  \
     const int rc = launch_swiglu_t(fc1, dtype, rows, inter, act, stream);                                     \
     if (rc != WOL_OK) return rc;                                                                              \
-    launch_moe_gemm<DT, B>(act, tb, max_tiles, bm, ffn2_codes, nullptr, ffn2_scale, inter / 2, hidden, out, stream); \
+    launch_moe_gemm<DT, B>(act, l2, ffn2_codes, nullptr, ffn2_scale, inter / 2, hidden, out, stream); \
   } while (0)
   if (dtype == WOL_DTYPE_BF16) {
     if (bits == 8) WOL_MOE(WOL_DTYPE_BF16, 8); else WOL_MOE(WOL_DTYPE_BF16, 4);
