@@ -1188,10 +1188,14 @@ __global__ __launch_bounds__(256) void moe_plan_kernel(const int64_t* __restrict
 // when the experts have few rows each -- a decode step of a mixture of
 // experts -- where the large tile would do up to eight times the MFMA work
 // and hold one workgroup per CU where three fit.
+// From 512 rows per expert on, int8 takes the 256 x 256 tile of the ungrouped
+// prefill launch (more MFMAs per dequantised fragment; a partial last tile per
+// expert then weighs little).
 inline int moe_tile_rows(int64_t rows, int num_experts, int bits) {
   const int64_t avg = rows / (num_experts > 0 ? num_experts : 1);
   if (avg <= 32 && bits == 4) return 32;
   if (avg <= 64) return 64;
+  if (avg >= 512 && bits == 8) return 256;
   return 128;
 }
 
@@ -1256,6 +1260,12 @@ void launch_moe_gemm(const void* x, const MoeLaunch& ml, const void* codes, cons
   if constexpr (BITS == 4) {
     if (ml.bm == 32) {
       launch_moe_gemm_cfg<DT, 4, true, 1, 8, 1, 1, 2>(x, ml, codes, bias, scale, K, N, out, stream);
+      return;
+    }
+  }
+  if constexpr (BITS == 8) {
+    if (ml.bm == 256) {
+      launch_moe_gemm_cfg<DT, 8, false, 2, 4, 4, 2, 3>(x, ml, codes, bias, scale, K, N, out, stream);
       return;
     }
   }

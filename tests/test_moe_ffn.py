@@ -31,13 +31,14 @@ def _oracle_moe(oracle, xb, cum, w1b, b1b, w2b, dt, bits):
 # rows per expert: none, a few, exactly one tile, a tile and a bit, many, none at
 # the end (128-row tiles); few rows per expert, with whole and partial tiles
 # and one expert far above the average (64-row tiles; 32-row tiles for int4);
-# an average of 38 rows (64-row tiles for both bit widths)
-ROWS_PER_EXPERT = [[0, 5, 128, 131, 300, 0], [0, 5, 33, 64, 1, 17], [40, 64, 0, 70, 3, 50], [2, 1, 150, 0, 3, 4]]
+# an average of 38 rows (64-row tiles for both bit widths); many rows
+ROWS_PER_EXPERT = [[0, 5, 128, 131, 300, 0], [0, 5, 33, 64, 1, 17], [40, 64, 0, 70, 3, 50], [2, 1, 150, 0, 3, 4],
+                   [600, 256, 0, 1000, 700, 520]]  # 512 and more on average: 256-row tiles for int8
 
 
 @pytest.mark.parametrize("dt", [H.F16, H.BF16])
 @pytest.mark.parametrize("bits", [8, 4])
-@pytest.mark.parametrize("per,inter", [(p, 512) for p in ROWS_PER_EXPERT] + [(p, 4096) for p in ROWS_PER_EXPERT[1:]])
+@pytest.mark.parametrize("per,inter", [(p, 512) for p in ROWS_PER_EXPERT] + [(p, 4096) for p in ROWS_PER_EXPERT[1:4]])
 def test_moe_ffn_against_oracle(device, oracle, dt, bits, per, inter):
     # inter = 4096 with few rows per expert: the second GEMM (K = 2048) runs with
     # its K cut into runs across workgroups and the kernel that adds them
