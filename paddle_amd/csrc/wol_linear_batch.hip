@@ -1,5 +1,5 @@
-// weight_only_linear for a small batch of rows (2 <= M <= 16): the decode
-// kernel for batched serving.
+// weight_only_linear for a small batch of rows (2 <= M <= 16, up to 32 in the
+// K-split form): the decode kernel for batched serving.
 //
 // What limits the one-row kernel's launch shape (a workgroup per 16-column
 // strip) at several rows is the activations: every workgroup needs all of x,
@@ -39,6 +39,14 @@
 // The per-channel scales and the bias of a run are parked in LDS at its start;
 // group-wise scales travel with their weight tiles, one 2-byte load per lane
 // and group.
+//
+// A second form of the kernel (SPLIT) cuts K into runs across workgroups as
+// well: workgroup b works on run b % runs of strip set b / runs, a run being
+// 16 wavefronts x 128 or 256 k, and the runs' fp32 sums meet in a scratch
+// buffer that reduce_partials_kernel (wol_linear_gemm.hip) adds up.  That
+// serves any K of whole weight tiles, keeps the activations a workgroup fetches
+// down to K / runs when the strips are few, and -- with two 16-row operands
+// per wavefront (MT = 2) -- takes up to 32 rows.
 #include <atomic>
 
 #include "wol_common.h"
