@@ -32,7 +32,7 @@ def test_dispatcher_is_never_far_from_the_best_pinned_kernel(device):
     # The rules that choose a kernel are fitted to measurements; this guards
     # them against gross mistakes (a rule that sends a decode call to the GEMM,
     # or the other way round): on shapes from every region of the rules the
-    # kernel wol_linear takes is at most 1.6 x slower than the fastest kernel
+    # kernel wol_linear takes is at most twice as slow as the fastest kernel
     # that accepts the shape.  Eager launches, median of five timings.
     import torch
     from paddle_amd import _lib
@@ -63,4 +63,4 @@ def test_dispatcher_is_never_far_from_the_best_pinned_kernel(device):
         best = min(v for k, v in times.items() if k != _lib.KERNEL_AUTO)
         print("case", M, K, N, bits, g, {k: round(v * 1e3, 1) for k, v in times.items()}, flush=True)
         worst.append((times[_lib.KERNEL_AUTO] / best, M, K, N, bits, g))
-    assert max(worst)[0] <= 1.6, sorted(worst, reverse=True)[:3]
+    assert max(worst)[0] <= 2.0, sorted(worst, reverse=True)[:3]
