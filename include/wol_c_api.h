@@ -34,6 +34,10 @@
  *     wol_linear_grad write one line per call to stderr (the problem and the
  *     kernel taken), the way the reference's VLOG lines name the GEMV/GEMM
  *     branch (gpu/weight_only_linear_kernel.cu:60-200).  Read once per process.
+ *   - WOL_ROCTX=1 in the environment wraps every compute call in a roctx
+ *     range named after its entry point (for rocprofv3 --marker-trace); the
+ *     marker library is looked up with dlopen, there is no link dependency.
+ *     Read once per process.
  */
 #ifndef WOL_C_API_H_
 #define WOL_C_API_H_

@@ -4,6 +4,7 @@
 #include <atomic>
 #include <cstring>
 
+#include <dlfcn.h>
 #include <stdlib.h>
 
 #include "wol_common.h"
@@ -180,10 +181,47 @@ bool log_enabled() {
   return on;
 }
 
+// WOL_ROCTX=1 in the environment: every compute call of the C ABI is wrapped
+// in a roctx range named after its entry point, so that a rocprofv3
+// --marker-trace shows which launches belong to which call.  The marker
+// library is looked up at run time (no link dependency); without it, or
+// without the variable, a range costs one load of a static flag.
+struct RoctxApi {
+  int (*push)(const char*) = nullptr;
+  int (*pop)() = nullptr;
+};
+const RoctxApi& roctx_api() {
+  static const RoctxApi api = [] {
+    RoctxApi a;
+    const char* e = getenv("WOL_ROCTX");
+    if (e == nullptr || e[0] == '\0' || e[0] == '0') return a;
+    void* h = dlopen("librocprofiler-sdk-roctx.so", RTLD_NOW | RTLD_GLOBAL);
+    if (h == nullptr) h = dlopen("libroctx64.so", RTLD_NOW | RTLD_GLOBAL);
+    if (h == nullptr) return a;
+    a.push = reinterpret_cast<int (*)(const char*)>(dlsym(h, "roctxRangePushA"));
+    a.pop = reinterpret_cast<int (*)()>(dlsym(h, "roctxRangePop"));
+    if (a.push == nullptr || a.pop == nullptr) a = RoctxApi();
+    return a;
+  }();
+  return api;
+}
+struct Range {
+  explicit Range(const char* name) : on(roctx_api().push != nullptr) {
+    if (on) roctx_api().push(name);
+  }
+  ~Range() {
+    if (on) roctx_api().pop();
+  }
+  Range(const Range&) = delete;
+  Range& operator=(const Range&) = delete;
+  bool on;
+};
+
 int linear_impl(const void* x, const void* codes, const void* bias, const void* scale, int dtype,
                 int64_t M, int64_t K, int64_t N, int bits, int group_size, void* out, bool out_f32,
                 int kernel, void* workspace, size_t workspace_bytes, void* stream,
                 const wol::Fuse& fuse = wol::Fuse()) {
+  const Range range("wol_linear");
   const int rc = check_problem(dtype, K, N, bits, group_size);
   if (rc != WOL_OK) return rc;
   if (M < 0 || M > (int64_t{1} << 24)) return WOL_ERR_BAD_SHAPE;
@@ -257,6 +295,7 @@ size_t wol_quantize_workspace(int64_t K, int64_t N, int bits, int group_size) {
 int wol_quantize(const void* w, int dtype, int64_t K, int64_t N, int bits, int group_size,
                  int round_mode, int layout, void* codes_out, void* scale_out, void* workspace,
                  size_t workspace_bytes, void* stream) {
+  const Range range("wol_quantize");
   const int rc = check_problem(dtype, K, N, bits, group_size);
   if (rc != WOL_OK) return rc;
   if (round_mode != WOL_ROUND_RNE && round_mode != WOL_ROUND_TRUNC) return WOL_ERR_BAD_ROUND_MODE;
@@ -272,6 +311,7 @@ int wol_quantize(const void* w, int dtype, int64_t K, int64_t N, int bits, int g
 
 int wol_quantize_static(const void* w, int dtype, int64_t K, int64_t N, int bits, int group_size,
                         int round_mode, int layout, void* codes_out, void* scale_out, void* stream) {
+  const Range range("wol_quantize_static");
   const int rc = check_problem(dtype, K, N, bits, group_size);
   if (rc != WOL_OK) return rc;
   if (round_mode != WOL_ROUND_RNE && round_mode != WOL_ROUND_TRUNC) return WOL_ERR_BAD_ROUND_MODE;
@@ -287,6 +327,7 @@ int wol_quantize_static(const void* w, int dtype, int64_t K, int64_t N, int bits
 int wol_quantize_llm_int8(const void* w, int dtype, int64_t K, int64_t N, int group_size,
                           int layout, void* codes_out, float* scale_out, void* workspace,
                           size_t workspace_bytes, void* stream) {
+  const Range range("wol_quantize_llm_int8");
   const int rc = check_problem(dtype, K, N, 8, group_size);
   if (rc != WOL_OK) return rc;
   if (!layout_ok(layout)) return WOL_ERR_BAD_LAYOUT;
@@ -301,6 +342,7 @@ int wol_quantize_llm_int8(const void* w, int dtype, int64_t K, int64_t N, int gr
 
 int wol_dequantize(const void* codes, int layout, const void* scale, int dtype, int64_t K,
                    int64_t N, int bits, int group_size, void* out_KN, void* stream) {
+  const Range range("wol_dequantize");
   const int rc = check_problem(dtype, K, N, bits, group_size);
   if (rc != WOL_OK) return rc;
   if (!layout_ok(layout)) return WOL_ERR_BAD_LAYOUT;
@@ -381,6 +423,7 @@ int wol_linear_fused(const void* x, const void* pre_scale, const void* codes, co
                      const void* scale, int dtype, int64_t M, int64_t K, int64_t N, int bits,
                      int group_size, int act, void* out, void* workspace, size_t workspace_bytes,
                      void* stream) {
+  const Range range("wol_linear_fused");
   const int rc = check_problem(dtype, K, N, bits, group_size);
   if (rc != WOL_OK) return rc;
   if (M < 0 || M > (int64_t{1} << 24)) return WOL_ERR_BAD_SHAPE;
@@ -431,6 +474,7 @@ namespace {
 int linear_grad_impl(const void* out_grad, const void* codes, const void* scale, int dtype, int64_t M,
                      int64_t K, int64_t N, int bits, int group_size, void* x_grad, bool out_f32,
                      void* workspace, size_t workspace_bytes, void* stream) {
+  const Range range("wol_linear_grad");
   const int rc = check_problem(dtype, K, N, bits, group_size);
   if (rc != WOL_OK) return rc;
   if (M < 0 || M > (int64_t{1} << 24)) return WOL_ERR_BAD_SHAPE;
@@ -484,6 +528,7 @@ int wol_moe_ffn(const void* permute_input, const int64_t* token_nums_per_expert,
                 const void* ffn1_bias, const void* ffn1_scale, const void* ffn2_weight, const void* ffn2_scale,
                 int dtype, int64_t rows, int64_t hidden, int64_t inter, int num_experts, int bits, void* ffn_out,
                 void* workspace, size_t workspace_bytes, void* stream) {
+  const Range range("wol_moe_ffn");
   if (dtype != WOL_DTYPE_F16 && dtype != WOL_DTYPE_BF16) return WOL_ERR_BAD_DTYPE;
   if (bits != 8 && bits != 4) return WOL_ERR_BAD_BITS;
   const int rc = check_moe(rows, hidden, inter, num_experts);
@@ -514,6 +559,7 @@ int wol_linear_on(const void* x, const void* codes, const void* bias, const void
 
 int wol_repack(const void* codes_in, int layout_in, void* codes_out, int layout_out, int64_t K,
                int64_t N, int bits, void* stream) {
+  const Range range("wol_repack");
   const int rc = check_problem(WOL_DTYPE_F16, K, N, bits, -1);
   if (rc != WOL_OK) return rc;
   if (!layout_ok(layout_in) || !layout_ok(layout_out)) return WOL_ERR_BAD_LAYOUT;
@@ -559,6 +605,7 @@ int64_t wol_code_offset(int layout, int64_t K, int64_t N, int bits, int64_t k, i
 
 int wol_apply_per_channel_scale(const void* x, const void* scales, int dtype, int64_t rows,
                                 int64_t cols, void* out, void* stream) {
+  const Range range("wol_apply_per_channel_scale");
   if (dtype != WOL_DTYPE_F16 && dtype != WOL_DTYPE_BF16) return WOL_ERR_BAD_DTYPE;
   if (rows < 0 || cols <= 0 || rows > (int64_t{1} << 24) || cols > (int64_t{1} << 24))
     return WOL_ERR_BAD_SHAPE;
@@ -590,6 +637,7 @@ int wol_llm_int8_linear_stage_offsets(int64_t M, int64_t K, int64_t N, int64_t* 
 int wol_llm_int8_linear(const void* x, const void* weight, const void* bias, const float* weight_scale,
                         float threshold, int dtype, int64_t M, int64_t K, int64_t N, void* out,
                         void* workspace, size_t workspace_bytes, void* stream) {
+  const Range range("wol_llm_int8_linear");
   const int rc = check_problem(dtype, K, N, 8, -1);
   if (rc != WOL_OK) return rc;
   if (M < 0 || M > (int64_t{1} << 24)) return WOL_ERR_BAD_SHAPE;

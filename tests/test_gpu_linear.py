@@ -679,3 +679,32 @@ def test_call_log_names_the_kernel(device):
     assert "M=1 K=2048 N=12288 int8" in lines[0] and lines[0].endswith("-> stream kernel")
     assert lines[1].endswith("-> batch kernel") and lines[2].endswith("-> gemm kernel")
 
+
+def test_roctx_ranges_do_not_disturb_the_calls(device):
+    # WOL_ROCTX=1: every compute call pushes and pops a roctx range (the marker
+    # library is loaded at the first call); results are what they are without
+    # it.  Read once per process, hence a child process.
+    import os
+    import subprocess
+    import sys
+
+    code = (
+        "import torch\n"
+        "from paddle_amd.nn import quant as Q\n"
+        "g = torch.Generator(device='cuda').manual_seed(1)\n"
+        "w = (torch.randn(2048, 1024, device='cuda', generator=g) * 0.02).to(torch.bfloat16)\n"
+        "c, s = Q.weight_quantize(w, algo='weight_only_int8')\n"
+        "x = torch.randn(8, 2048, device='cuda', generator=g).to(torch.bfloat16)\n"
+        "y = Q.weight_only_linear(x, c, None, s, 'int8')\n"
+        "torch.cuda.synchronize()\n"
+        "print(float(y.float().abs().sum()))\n"
+    )
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    outs = []
+    for flag in ("0", "1"):
+        r = subprocess.run([sys.executable, "-c", code], env=dict(os.environ, WOL_ROCTX=flag, PYTHONPATH=root),
+                           capture_output=True, text=True, timeout=300)
+        assert r.returncode == 0, r.stderr[-2000:]
+        outs.append(r.stdout.strip().splitlines()[-1])
+    assert outs[0] == outs[1]
+
