@@ -135,6 +135,31 @@ def test_fused_pre_scale_equals_the_two_ops(device, oracle, dt):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("act,use_pre", [(1, False), (2, True)])
+def test_fused_on_the_batched_kernel_with_k_runs(device, oracle, act, use_pre):
+    # 24 rows on a 25 MB int8 weight: wol_linear takes the batched kernel with K
+    # runs, so gelu and bias are applied by the kernel that adds the runs, swiglu
+    # by its pass over the fp32 sums, the pre-scale by a pass in front
+    from paddle_amd import _lib
+    import ctypes
+
+    dt, bits, g, M, K, N = H.BF16, 8, 64, 24, 2048, 12288
+    buf = ctypes.create_string_buffer(512)
+    assert _lib.lib.wol_linear_plan(M, K, N, bits, g, 1 << 30, buf, 512) == 0 and b"K runs" in buf.value
+    rng = np.random.default_rng(13)
+    wb = H.make_weight(K, N, dt, seed=3)
+    xb = H.make_act(M, K, dt, seed=4)
+    bb = H.make_bias(N, dt, seed=5)
+    pre = H.f32_to_bits((0.5 + rng.random(K, dtype=np.float32)).astype(np.float32), dt) if use_pre else None
+    oc, osc = oracle.weight_quantize(wb, dt, bits, g)
+    packed = H.gfx950_from_q(H.q_from_canonical(oc, bits), bits)
+    _, wantT = oracle.linear_fused(xb, pre, oc, osc, bb, dt, bits, g, act)
+    got = _fused(xb, pre, packed, bb, osc, dt, N, bits, g, act)
+    err = H.rel_l2(H.bits_to_f32(got, dt), H.bits_to_f32(wantT, dt))
+    assert err <= TOL, (err, act, use_pre)
+
+
+@pytest.mark.gpu
 def test_fused_python_wrapper_and_errors(device):
     import torch
     from paddle_amd.nn import quant as Q
