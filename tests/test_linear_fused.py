@@ -94,11 +94,16 @@ def test_fused_against_oracle(device, oracle, dt, bits, g):
         pre = H.f32_to_bits((0.5 + rng.random(K, dtype=np.float32)).astype(np.float32), dt)
         oc, osc = oracle.weight_quantize(wb, dt, bits, g)
         packed = H.gfx950_from_q(H.q_from_canonical(oc, bits), bits)
+        big = K * N > 1e7  # the large shapes take a subset that still has every activation, pre-scale and bias
         for act in (0, 1, 2):
             for use_pre in (False, True):
                 for bias in (None, bb):
                     if act == 0 and not use_pre:
                         continue  # plain wol_linear, covered elsewhere
+                    if big and (act, use_pre, bias is not None) not in ((0, True, True), (1, True, False),
+                                                                        (1, False, True), (2, True, False),
+                                                                        (2, False, True)):
+                        continue
                     print("case", dt, bits, g, M, K, N, act, use_pre, bias is not None, flush=True)
                     _, wantT = oracle.linear_fused(xb, pre if use_pre else None, oc, osc, bias, dt, bits, g, act)
                     got = _fused(xb, pre if use_pre else None, packed, bias, osc, dt, N, bits, g, act)
