@@ -396,12 +396,18 @@ def cpu_decode_baseline(np, torch, H, w_bits, x_bits, cfg, budget_s=10.0):
         "unit": "GB/s",
         "cores": int(cores),
         "kind": "port",
-        "sample": "first %d of %d output columns of the decode weight (K=%d, int%d, group %d), M=1; "
-                  "per call: dequantize %.2f ms (1 thread) + fp32 matmul %.2f ms (%d threads); %d repetitions"
-                  % (n_s, N, K, bits, g, t_dq * 1e3, t_mm * 1e3, cores, reps),
-        "quantize": {"ms": round(t_q * 1e3, 2), "cores": 1, "GB/s": round(K * n_s * 2 / t_q / 1e9, 4),
-                     "what": "oracle weight_quantize of the same %d x %d sample, GB/s on the bf16 weight read"
-                             % (K, n_s)},
+        "sample": "first %d of %d columns of the decode weight, M=1, %d repetitions" % (n_s, N, reps),
+        "sample_columns": n_s,
+        "repetitions": reps,
+        "dequantize_ms": round(t_dq * 1e3, 3),
+        "dequantize_cores": 1,
+        "matmul_ms": round(t_mm * 1e3, 3),
+        "matmul_cores": int(cores),
+        "quantize_ms": round(t_q * 1e3, 2),
+        "quantize_cores": 1,
+        "quantize_gbs": round(K * n_s * 2 / t_q / 1e9, 4),
+        "stages": "per call: oracle dequantize (1 thread) + fp32 matmul (torch CPU BLAS, all threads); quantize_ms is the "
+                  "one-time oracle weight_quantize of the same sample (1 thread), quantize_gbs on its bf16 weight read",
     }, (codes, scale, n_s)
 
 
@@ -423,10 +429,9 @@ def cpu_prefill_baseline(np, torch, H, pw_bits, px_bits, cfg, n_s=1024):
         ts.append(time.perf_counter() - t0)
     t = statistics.median(ts)
     return {"value": round(2.0 * M * K * n_s / t / 1e12, 4), "unit": "TFLOP/s", "cores": int(torch.get_num_threads()),
-            "kind": "port",
-            "sample": "first %d of %d output columns, M=%d K=%d int8 per-channel: dequantize (1 thread) + fp32 matmul "
-                      "(all threads) %.1f ms per call; one-time quantize %.1f ms (1 thread)"
-                      % (n_s, cfg["N"], M, K, t * 1e3, t_q * 1e3)}, (codes, scale, y.numpy())
+            "kind": "port", "ms": round(t * 1e3, 2), "quantize_ms": round(t_q * 1e3, 2), "sample_columns": n_s,
+            "sample": "first %d of %d columns, M=%d: dequantize (1 thread) + fp32 matmul (all threads)"
+                      % (n_s, cfg["N"], M)}, (codes, scale, y.numpy())
 
 
 def main():
@@ -618,6 +623,10 @@ def main():
     if not args.no_cpu_baseline:
         pcpu, _ = cpu_prefill_baseline(np, torch, H, pw_bits, px_bits, p)
         cpu["prefill"] = pcpu
+        cpu["prefill_tflops"] = pcpu["value"]
+        cpu["prefill_ms"] = pcpu["ms"]
+        cpu["prefill_quantize_ms"] = pcpu["quantize_ms"]
+        cpu["prefill_sample_columns"] = pcpu["sample_columns"]
 
     # llm_int8_linear: all rows (the outlier columns depend on every row), the first columns
     if ly is not None:
@@ -664,6 +673,14 @@ def main():
             "kernel": _plan(_lib, c["M"], c["K"], c["N"], c["bits"], c["group_size"]) or "wol::stream_kernel",
             "algorithmic_bytes_per_launch": wbytes,
             "total_bytes_per_launch": total_bytes,
+            # the M=2048 half of the metric and the two in-run bounds, as plain numbers
+            "prefill_tflops": round(pre_tf, 2),
+            "prefill_frac": round(pre_tf / MFMA_BF16_PEAK_TF, 4),
+            "prefill_ms_per_step": round(pre_s * 1e3, 4),
+            "prefill_peak_tflops": MFMA_BF16_PEAK_TF,
+            "mfma_ceiling_tflops": round(ceil_tf, 1),
+            "read_floor_gbs": round(wbytes / floor_s / 1e9, 1),
+            "read_floor_ms_per_step": round(floor_s * 1e3, 6),
             "read_floor": {
                 "what": "wol_read_floor: the same weight copies read by a kernel of the same launch shape "
                         "that computes nothing (no scales, activations, MFMAs or output)",
@@ -703,6 +720,22 @@ def main():
         "cpu_baseline": cpu,
         "parity": parity,
     }
+    # every per-configuration fraction of its roofline once more as plain numbers of `roofline`
+    flat = out["roofline"]
+    for e in configs or []:
+        tag = "north_star" if e["config"].startswith("north") else e["config"]
+        flat["%s_K%d_N%d_M%d_frac" % (tag, e["K"], e["N"], e["M"])] = e["frac"]
+    if stack:
+        flat["c5_decode_M8_frac"] = stack["decode_M8"]["frac"]
+        flat["c5_prefill_M1024_frac"] = stack["prefill_M1024"]["frac"]
+    if grad:
+        for r in grad["rows"]:
+            flat["linear_grad_M%d_vs_composition" % r["M"]] = r["speed_vs_composition"]
+    if moe:
+        for r in moe["rows"]:
+            flat["moe_ffn_rows%d_frac" % r["rows"]] = r["frac"]
+    if llm:
+        flat["llm_int8_frac"] = llm["roofline"]["frac"]
     print(json.dumps(out))
     if failures:
         print("bench.py: PARITY FAILURE: " + "; ".join(failures), file=sys.stderr)
