@@ -161,7 +161,9 @@ int wol_dequantize(const void* codes, int layout, const void* scale, int dtype,
 /* Bytes of device scratch wol_linear can use for this problem (may be 0).  The
  * scratch is optional: without it (NULL or fewer bytes) the result is the
  * same to fp32 summation order and only the speed of small-M problems drops,
- * because K can no longer be split across workgroups.  Must be 16-byte aligned. */
+ * because K can no longer be split across workgroups.  Must be 16-byte aligned.
+ * wol_linear takes the same kernel with exactly this many bytes as with any
+ * larger buffer. */
 size_t wol_linear_workspace(int64_t M, int64_t K, int64_t N, int bits,
                             int group_size);
 
@@ -178,7 +180,9 @@ size_t wol_linear_workspace(int64_t M, int64_t K, int64_t N, int bits,
  * allows and it is measured faster (10 to 32 rows on some shapes), the
  * batched kernel with K cut into runs across workgroups runs instead.  The
  * reference's split is M <= 3 (gpu/weight_only_linear_kernel.cu:60-61).
- * x, codes and scale must be 16-byte aligned.
+ * x, codes, scale, out and (when given) bias must be 16-byte aligned: the
+ * kernels read and write 16 bytes at a time, the output rows included
+ * (WOL_ERR_ALIGNMENT otherwise).
  */
 int wol_linear(const void* x, const void* codes, const void* bias,
                const void* scale, int dtype, int64_t M, int64_t K, int64_t N,

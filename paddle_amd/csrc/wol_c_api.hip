@@ -78,7 +78,7 @@ bool gemm_fast_path(int64_t K, int bits) {
   return K % tk == 0 && K / tk >= 2;
 }
 
-// have_ws: the caller's scratch buffer holds at least two K runs of partial sums
+// have_ws: the caller's scratch buffer holds what the GEMM asks for on this problem
 bool use_stream(int64_t M, int64_t K, int64_t N, int bits, bool have_ws) {
   if (M > kStreamMaxM) return false;
   if (M <= kStreamAlwaysM || !gemm_fast_path(K, bits)) return true;
@@ -158,8 +158,13 @@ int resolve_kernel(int kernel, int64_t M, int64_t K, int64_t N, int bits, int gr
   if (kernel != WOL_KERNEL_AUTO) return kernel;
   if (use_batch_split(M, K, N, bits, group_size, ws_bytes)) return WOL_KERNEL_BATCH_SPLIT;
   if (use_batch(M, K, N, bits, group_size)) return WOL_KERNEL_BATCH;
-  const bool have_ws = ws_bytes / sizeof(float) / 2 >= static_cast<size_t>(M) * static_cast<size_t>(N);
-  return use_stream(M, K, N, bits, have_ws) ? WOL_KERNEL_STREAM : WOL_KERNEL_GEMM;
+  // With ample scratch first: if the streaming kernel wins there it is taken
+  // whatever the caller brought (wol_linear_workspace then reports 0 bytes, and
+  // a caller who passes exactly that gets the same kernel).  Only a GEMM that
+  // cannot have its K runs is compared again, as the unsplit GEMM it becomes.
+  if (use_stream(M, K, N, bits, true)) return WOL_KERNEL_STREAM;
+  if (ws_bytes >= wol::linear_gemm_workspace(M, K, N, bits, group_size)) return WOL_KERNEL_GEMM;
+  return use_stream(M, K, N, bits, false) ? WOL_KERNEL_STREAM : WOL_KERNEL_GEMM;
 }
 
 const char* kernel_name(int which) {
@@ -236,7 +241,9 @@ int linear_impl(const void* x, const void* codes, const void* bias, const void* 
   if (M == 0) return WOL_OK;  // empty batch: nothing to write
   if (x == nullptr || codes == nullptr || scale == nullptr || out == nullptr)
     return WOL_ERR_NULL_POINTER;
-  if (!aligned16(x) || !aligned16(codes) || !aligned16(scale)) return WOL_ERR_ALIGNMENT;
+  // the kernels read and write 16 bytes at a time (the output rows included)
+  if (!aligned16(x) || !aligned16(codes) || !aligned16(scale) || !aligned16(out) || !aligned16(bias))
+    return WOL_ERR_ALIGNMENT;
   if (const int dv = require_gfx950(); dv != WOL_OK) return dv;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (workspace == nullptr || !aligned16(workspace)) workspace_bytes = 0;  // optional: only speeds up
@@ -431,7 +438,8 @@ int wol_linear_fused(const void* x, const void* pre_scale, const void* codes, co
   if (act == WOL_ACT_SWIGLU && N % 32 != 0) return WOL_ERR_BAD_SHAPE;
   if (M == 0) return WOL_OK;
   if (x == nullptr || codes == nullptr || scale == nullptr || out == nullptr) return WOL_ERR_NULL_POINTER;
-  if (!aligned16(x) || !aligned16(codes) || !aligned16(scale)) return WOL_ERR_ALIGNMENT;
+  if (!aligned16(x) || !aligned16(codes) || !aligned16(scale) || !aligned16(out) || !aligned16(bias))
+    return WOL_ERR_ALIGNMENT;
   if (pre_scale != nullptr && !aligned16(pre_scale)) return WOL_ERR_ALIGNMENT;
   const FusedPlan f = plan_fused(M, K, N, bits, group_size, pre_scale != nullptr, act);
   if (f.prepass || f.swiglu_pass) {

@@ -1156,28 +1156,35 @@ void launch_fast(const Args& a) {
 // rows cum[e-1] .. cum[e]-1 and ceil(rows / bm) tiles.  One workgroup; the
 // table has max_tiles entries, unused ones marked -1.
 __global__ __launch_bounds__(256) void moe_plan_kernel(const int64_t* __restrict__ cum, int num_experts, int bm,
-                                                       int max_tiles, MoeTile* __restrict__ table) {
+                                                       int max_tiles, int64_t rows, MoeTile* __restrict__ table) {
   __shared__ int first_tile[1025];  // exclusive running total of tiles, by expert
+  __shared__ int row_end[1025];     // end of expert e's rows is row_end[e + 1]; row_end[0] = 0
   for (int i = threadIdx.x; i < max_tiles; i += 256) table[i] = MoeTile{-1, 0, 0, 0};
   if (threadIdx.x == 0) {
+    // The running totals come from the device and are not trusted: each is
+    // clamped to [previous total, rows], so an expert's count is never negative
+    // and no tile reaches past the last row of the input.
     int acc = 0;
     int64_t prev = 0;
+    row_end[0] = 0;
     for (int e = 0; e < num_experts; ++e) {
       first_tile[e] = acc;
-      const int64_t rows = cum[e] - prev;
-      prev = cum[e];
-      acc += static_cast<int>((rows + bm - 1) / bm);
+      int64_t end = cum[e];
+      end = end < prev ? prev : (end > rows ? rows : end);
+      acc += static_cast<int>((end - prev + bm - 1) / bm);
+      prev = end;
+      row_end[e + 1] = static_cast<int>(end);
     }
     first_tile[num_experts] = acc;
   }
   __syncthreads();
   for (int e = threadIdx.x; e < num_experts; e += 256) {
-    const int64_t r0 = e > 0 ? cum[e - 1] : 0, r1 = cum[e];
+    const int r0 = row_end[e], r1 = row_end[e + 1];
     const int t0 = first_tile[e], nt = first_tile[e + 1] - t0;
     for (int t = 0; t < nt && t0 + t < max_tiles; ++t) {
-      const int64_t row = r0 + static_cast<int64_t>(t) * bm;
-      const int64_t left = r1 - row;
-      table[t0 + t] = MoeTile{e, static_cast<int>(row), static_cast<int>(left < bm ? left : bm), 0};
+      const int row = r0 + t * bm;
+      const int left = r1 - row;
+      table[t0 + t] = MoeTile{e, row, left < bm ? left : bm, 0};
     }
   }
 }
@@ -1418,7 +1425,7 @@ int launch_moe_ffn(const void* x, const int64_t* rows_before_expert, const void*
   const MoeLaunch l1{reinterpret_cast<const int*>(table), max_tiles, bm, 1, rows, nullptr, nullptr};
   const MoeLaunch l2{reinterpret_cast<const int*>(table), max_tiles, bm, moe_runs(inter / 2, hidden, bits, bm, max_tiles),
                      rows, bm < 128 ? partial : nullptr, rows_before_expert + (num_experts - 1)};
-  moe_plan_kernel<<<dim3(1), dim3(256), 0, stream>>>(rows_before_expert, num_experts, bm, max_tiles, table);
+  moe_plan_kernel<<<dim3(1), dim3(256), 0, stream>>>(rows_before_expert, num_experts, bm, max_tiles, rows, table);
 #define WOL_MOE(DT, B)                                                                                        \
   do {                                                                                                        \
     launch_moe_gemm<DT, B>(x, l1, ffn1_codes, ffn1_bias, ffn1_scale, hidden, inter, fc1, stream);  \

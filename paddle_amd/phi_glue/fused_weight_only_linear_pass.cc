@@ -28,33 +28,17 @@
 #include "paddle/fluid/pir/utils/general_functions.h"
 #include "paddle/pir/include/pass/pass.h"
 #include "paddle/pir/include/pass/pass_registry.h"
-#if defined(PADDLE_WITH_CUDA)
-#include "paddle/phi/core/platform/device/gpu/gpu_info.h"
-#endif
 
 namespace {
 
-// Value of the ops' `arch` attribute.  -1 means "no kernel for this build".
-int ArchTag() {
-#if defined(PADDLE_WITH_HIP)
-  return 80;  // not read by the gfx950 kernels; 80 keeps every arch check above them quiet
-#elif defined(PADDLE_WITH_CUDA) && defined(PADDLE_WITH_CUTLASS)
-  return paddle::platform::GetGPUComputeCapability(paddle::platform::GetCurrentDeviceId());
-#else
-  return -1;
-#endif
-}
+// This file replaces the reference's pass in a ROCm build that links the
+// gfx950 kernels; it is not meant for any other build.
 
-bool ArchSupported(int arch) {
-#if defined(PADDLE_WITH_HIP)
-  return arch > 0;
-#else
-  switch (arch) {
-    case 70: case 75: case 80: case 86: case 89: case 90: return true;
-    default: return false;
-  }
-#endif
-}
+// Value of the ops' `arch` attribute.  The gfx950 kernels do not read it; 80
+// keeps every arch check above them (Python wrapper, InferMeta) quiet.
+int ArchTag() { return 80; }
+
+bool ArchSupported(int arch) { return arch > 0; }
 
 enum class BiasSide { kNone, kAfterMatmul, kBeforeMatmul };  // add(matmul, b) or add(b, matmul)
 

@@ -99,12 +99,19 @@ def test_argument_errors_return_before_device_work(lib):
     assert q(w=None) == 1
     assert q(w=ctypes.c_void_p(0x1008)) == 9
     assert q(g=-1) == 8  # per-channel needs the abs-max workspace
-    lin = lambda **kw: L.wol_linear(kw.get("x", p), p, None, p, kw.get("dt", 1), kw.get("M", 1), kw.get("K", 64),
-                                    kw.get("N", 16), kw.get("bits", 4), kw.get("g", -1), p, None, 0, None)
+    lin = lambda **kw: L.wol_linear(kw.get("x", p), p, kw.get("bias", None), p, kw.get("dt", 1), kw.get("M", 1),
+                                    kw.get("K", 64), kw.get("N", 16), kw.get("bits", 4), kw.get("g", -1),
+                                    kw.get("out", p), None, 0, None)
     assert lin(dt=5) == 2 and lin(bits=2) == 3 and lin(g=100) == 4 and lin(K=100) == 5 and lin(M=-1) == 5
     assert lin(K=(1 << 24) + 64) == 5 and lin(N=(1 << 24) + 16) == 5 and lin(M=(1 << 24) + 1) == 5
     assert lin(x=None) == 1
     assert lin(x=ctypes.c_void_p(0x1004)) == 9
+    # the output rows and the bias are accessed 16 bytes at a time as well
+    assert lin(out=ctypes.c_void_p(0x1008)) == 9 and lin(bias=ctypes.c_void_p(0x1002)) == 9
+    assert lin(out=None) == 1
+    fused = lambda **kw: L.wol_linear_fused(p, None, p, kw.get("bias", None), p, 1, 1, 64, 32, 4, -1, 0,
+                                            kw.get("out", p), None, 0, None)
+    assert fused(out=ctypes.c_void_p(0x1008)) == 9 and fused(bias=ctypes.c_void_p(0x1004)) == 9
     assert lin(M=0) == 0  # empty batch is a no-op
     on = lambda **kw: L.wol_linear_on(p, p, None, kw.get("scale", p), 1, kw.get("M", 1), 64, 16, 4, -1, p, 0,
                                       kw.get("kernel", 0), None, 0, None)
@@ -250,6 +257,31 @@ def test_linear_plan_names_the_kernel_per_shape(lib):
     assert "gemm_dma_kernel" in plan(2048, 4096, 12288, 8, -1)
     assert "256x256" in plan(2048, 4096, 12288, 8, -1)
     assert lib.lib.wol_linear_plan(4, 4096, 100, 8, -1, 0, ctypes.create_string_buffer(8), 8) == 5
+
+
+def test_linear_plan_is_the_same_with_the_advised_scratch_as_with_any_larger(lib):
+    # wol_linear_workspace() bytes are enough for the kernel wol_linear would
+    # take with unlimited scratch -- also where that is 0 bytes (a GEMM that
+    # needs no K runs, a decode kernel): the choice must not flip between the
+    # two.  Sweep of the region between the decode kernels and the prefill GEMM.
+    size_max = ctypes.c_size_t(-1).value
+
+    def plan(M, K, N, bits, g, ws):
+        buf = ctypes.create_string_buffer(256)
+        assert lib.lib.wol_linear_plan(M, K, N, bits, g, ws, buf, 256) == 0
+        return buf.value.decode()
+
+    flips = []
+    for bits in (4, 8):
+        for g in (-1, 128):
+            for K in (1024, 2048, 4096, 8192, 11008):
+                for N in (2048, 4096, 11008, 12288, 14336, 28672):
+                    for M in (1, 2, 8, 12, 16, 17, 20, 24, 27, 32, 40, 49, 56, 57, 64, 65, 128):
+                        need = lib.lib.wol_linear_workspace(M, K, N, bits, g)
+                        a, b = plan(M, K, N, bits, g, need), plan(M, K, N, bits, g, size_max)
+                        if a != b:
+                            flips.append((M, K, N, bits, g, a, b))
+    assert not flips, flips[:5]
 
 
 @pytest.mark.parametrize("bits", [8, 4])

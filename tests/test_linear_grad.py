@@ -105,13 +105,15 @@ def test_linear_grad_against_oracle(device, oracle, dt, bits, g):
         print("case", dt, bits, g, M, K, N, flush=True)
         err32, errT = _case(oracle, dt, bits, g, M, K, N)
         # The fp32 sums carry the one rounding of code * scale to 11 bits
-        # (about 1.5e-4).  The T outputs of kernel and oracle are casts of sums
-        # that differ by that much, so now and then they land on neighbouring T
-        # values: with bfloat16's coarse grid (spacing 2^-8 .. 2^-7 of the
-        # value) that alone is about 8e-4 in rel-L2 on average and more on a
-        # small output, hence the allowance below 4096 elements.
+        # (about 1.5e-4) and are held to 3e-4; _case has already checked that
+        # the T output is exactly their round-to-nearest-even cast.  Together
+        # that is the whole statement about the T output.  Comparing it with
+        # the oracle's T output on top is only meaningful where the output is
+        # large enough for the rel-L2 of two bfloat16 roundings of nearby sums
+        # (neighbouring values now and then, 2^-8 apart) to average out.
         assert err32 <= 3e-4, (err32, dt, bits, g, M, K, N)
-        assert errT <= (TOL if dt == H.F16 or M * K >= 4096 else 2e-3), (errT, dt, bits, g, M, K, N)
+        if dt == H.F16 or M * K >= 4096:
+            assert errT <= TOL, (errT, dt, bits, g, M, K, N)
 
 
 @pytest.mark.gpu

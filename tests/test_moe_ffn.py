@@ -75,6 +75,30 @@ def test_moe_ffn_against_oracle(device, oracle, dt, bits, per, inter):
             prev = int(end)
 
 
+def test_moe_ffn_clamps_running_totals_it_cannot_trust(device):
+    # token_nums_per_expert comes from the device and is read there only.  Totals
+    # that run backwards or past the input's rows are clamped by the table
+    # builder to [previous total, rows]: the call computes what it would with
+    # the clamped totals and touches no row outside the input.
+    import torch
+    from paddle_amd.nn import quant as Q
+
+    hidden, inter, E = 256, 512, 5
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    w1 = (torch.randn(E, hidden, inter, device="cuda", generator=gen) * 0.02).to(torch.bfloat16)
+    w2 = (torch.randn(E, inter // 2, hidden, device="cuda", generator=gen) * 0.02).to(torch.bfloat16)
+    q1, s1 = Q.moe_quantize_experts(w1)
+    q2, s2 = Q.moe_quantize_experts(w2)
+    rows = 200
+    x = torch.randn(rows, hidden, device="cuda", generator=gen).to(torch.bfloat16)
+    bad = torch.tensor([70, 30, 150, 10 ** 9, -5], dtype=torch.int64, device="cuda")   # backwards, huge, negative
+    good = torch.tensor([70, 70, 150, 200, 200], dtype=torch.int64, device="cuda")     # what the clamp makes of it
+    want = Q.moe_ffn(x, good, q1, q2, None, s1, s2, "weight_only_int8")
+    got = Q.moe_ffn(x, bad, q1, q2, None, s1, s2, "weight_only_int8")
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+
+
 def test_moe_ffn_equals_per_expert_calls(device):
     # the grouped launches against a loop of ordinary calls on each expert's rows
     import torch
