@@ -533,22 +533,40 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   const int sfold = sval / BN;
   int scol = strip_blk * kStripCols + sval % BN;
   scol = scol < n_hi ? scol : n_hi - 2;  // past the last column: valid data, never used
-  auto issue = [&](int it) {
+  // Loads lo .. hi-1 of tile `it` into its stage; a stage's loads are numbered
+  // [scales,] A loads, B loads.
+  auto issue_range = [&](int it, int lo, int hi) {
     const int t = tile_index(it);  // past the end: reload the last tile into a spare stage
     unsigned char* stage = smem + (it % kStages) * kStage;
-    if (G != 0) {
+    constexpr int kS = G == 0 ? 0 : 1;
+    if (G != 0 && lo == 0 && hi > 0) {
       const int64_t row = (static_cast<int64_t>(t0 + t) * TK + sfold * kFoldK) >> kGShift;
       __builtin_amdgcn_global_load_lds(scale + row * N + scol,
                                        (lds_ptr_t)(stage + kABytes + kBBytes + wave * 256), 4, 0, 0);
     }
 #pragma unroll
     for (int c = 0; c < kALoads; ++c)
-      __builtin_amdgcn_global_load_lds(asrc[c] + t * TK, (lds_ptr_t)(stage + (c * NW + wave) * 1024), 16, 0, 0);
+      if (kS + c >= lo && kS + c < hi)
+        __builtin_amdgcn_global_load_lds(asrc[c] + t * TK, (lds_ptr_t)(stage + (c * NW + wave) * 1024), 16, 0, 0);
 #pragma unroll
     for (int c = 0; c < kBLoads; ++c)
-      __builtin_amdgcn_global_load_lds(bsrc[c] + t * 1024,
-                                       (lds_ptr_t)(stage + kABytes + (c * NW + wave) * 1024), 16, 0, 0);
+      if (kS + kALoads + c >= lo && kS + kALoads + c < hi)
+        __builtin_amdgcn_global_load_lds(bsrc[c] + t * 1024,
+                                         (lds_ptr_t)(stage + kABytes + (c * NW + wave) * 1024), 16, 0, 0);
   };
+  auto issue = [&](int it) { issue_range(it, 0, kPerStage); };
+  // With three stages the loads of tile it+3 may be issued anywhere between the
+  // barrier of tile `it` (which frees their stage) and the barrier of tile it+1,
+  // and still have a whole tile period to land.  They are spread over that
+  // period, a few per slice: issued in one burst right behind the barrier, the
+  // loads of all wavefronts meet in the one load path of the CU at the same
+  // moment, and a wavefront that waits there issues no MFMA.  Segment 0 is the
+  // half slice behind the barrier, segment 1 the last slice of the tile,
+  // segments 2 .. Q-1 the slices 0 .. Q-3 of the next tile.  Two stages leave
+  // no such freedom: everything goes out behind the barrier.
+  constexpr bool kSpread = kStages == 3;
+  auto seg_lo = [](int s) { return kSpread ? (s * kPerStage + Q - 1) / Q : (s > 0 ? kPerStage : 0); };
+  auto seg_n = [&](int s) { return seg_lo(s + 1) - seg_lo(s); };
 
   // columns of this lane's accumulators: block c of the wavefront, column r32
   const int col0 = (strip_blk + wn * TN * 2) * 16;
@@ -666,8 +684,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
 
   issue(0);
   issue(1);
-  if (kStages == 3) issue(2);
-  wait_vmcnt<(kStages - 1) * kPerStage>();  // tile 0 has landed
+  if (kStages == 3) issue_range(2, 0, seg_lo(2));  // the rest of tile 2 goes out during tile 0
+  wait_vmcnt<(kStages - 2) * kPerStage + (kStages == 3 ? (2 * kPerStage + Q - 1) / Q : kPerStage)>();  // tile 0 has landed
   __builtin_amdgcn_s_barrier();
   read_b(smem, braw[0]);
   read_a(smem, af[0], 0);
@@ -687,6 +705,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
     for (int q = 0; q < Q; ++q) {
       if (q != Q - 2) {
         const bool last = q == Q - 1;
+        // this slice's share of the tile loads (segment 1 of tile it+3, or segment q+2 of tile it+2)
+        const int seg = last ? 1 : q + 2;
+        if (kSpread) issue_range(last ? it + kStages : it + kStages - 1, seg_lo(seg), seg_lo(seg + 1));
         read_a(last ? next : stage, af[(q + 1) & 1], last ? 0 : q + 1);
         dequant(bf[(q + 1) & 1], last ? raw_next : raw, last ? 0 : q + 1);
         mfmas(af[q & 1], bf[q & 1], q, 0, TM * TN);
@@ -694,6 +715,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
         for (int i = 0; i < TM * TN; ++i) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                   // one MFMA
           if (i < TM) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);       // one LDS read
+          if (kSpread && i % 2 == 1 && i / 2 < seg_n(seg)) {
+            __builtin_amdgcn_sched_group_barrier(0x004, 2, 0);                 // its LDS address into m0
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                 // one tile load
+          }
           __builtin_amdgcn_sched_group_barrier(0x002, kValuPerMfma, 0);        // VALU
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -713,7 +738,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
         __builtin_amdgcn_s_waitcnt(0x0070 | (0xF << 0) | (3 << 14));  // lgkmcnt(0)
         wait_vmcnt<(kStages - 2) * kPerStage>();
         __builtin_amdgcn_s_barrier();
-        issue(it + kStages);
+        issue_range(it + kStages, 0, seg_lo(1));
         read_b(next, raw_next);
         dequant(bf[(q + 1) & 1], raw, q + 1);
         mfmas(af[q & 1], bf[q & 1], q, kHalf, TM * TN);
@@ -721,6 +746,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
         for (int i = 0; i < TM * TN - kHalf + 1; ++i) {
           if (i < TM * TN - kHalf) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
           if (i < 2 * TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          if (kSpread && i < seg_n(0)) {
+            __builtin_amdgcn_sched_group_barrier(0x004, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+          }
           __builtin_amdgcn_sched_group_barrier(0x002, 2 * kValuPerMfma, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
