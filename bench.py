@@ -64,23 +64,29 @@ def _quantize(Q, w, bits, group_size):
 EAGER = False  # --eager: every leg launches eagerly (for counter collection, which needs plain dispatches)
 
 
-def time_graph(torch, fn, launches, warm_launches=400, warm_ms=50.0, replays=REPLAYS, eager=False):
+def time_graph(torch, fn, launches, warm_launches=400, warm_ms=50.0, replays=REPLAYS, eager=False, whole=None):
     """fn(i) enqueues launch i on the current stream.  Captures `launches`
     calls into one HIP graph, replays it untimed until both warm-up thresholds
     are met, then times `replays` replays one by one (events on the current
-    stream).  Returns (median, minimum) seconds per replay."""
+    stream).  Returns (median, minimum) seconds per replay.  whole: a callable
+    that enqueues all `launches` launches itself (it may fork onto other
+    streams and must join back into the current one)."""
+    def all_launches():
+        if whole is not None:
+            whole()
+        else:
+            for i in range(launches):
+                fn(i)
+
     for i in range(3):
         fn(i)
     torch.cuda.synchronize()
     if eager or EAGER:
-        def run():
-            for i in range(launches):
-                fn(i)
+        run = all_launches
     else:
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
-            for i in range(launches):
-                fn(i)
+            all_launches()
         run = g.replay
     torch.cuda.synchronize()
     done, batch = 0, 1
@@ -518,6 +524,39 @@ def main():
     floor_med, _ = time_graph(torch, floor_step, args.steps, warm_launches=max(400, args.warmup), eager=args.eager)
     floor_s = floor_med / args.steps
 
+    # Independent decode GEMVs with no edge between them: --steps calls dealt
+    # round-robin to four streams that fork from and join the launching stream
+    # inside the same graph, so up to four launches are in flight at a time
+    # (independent projections of one input: q/k/v or gate/up kept as separate
+    # weights, the experts of a mixture).  Every call still reads its own
+    # weight copy from HBM once; what overlaps is one call's launch and drain
+    # with another's stream.
+    n_par = 4
+    par_streams = [torch.cuda.Stream(device=dev) for _ in range(n_par - 1)]
+    par_x = [x.clone() for _ in range(n_par)]
+
+    def par_call(i, s):
+        j = i % ncopies
+        with torch.cuda.stream(s):
+            return Q.weight_only_linear(par_x[i % n_par], copies[j], None, scales[j], wd, None, c["group_size"])
+
+    def par_whole():
+        cur = torch.cuda.current_stream()
+        fork = torch.cuda.Event()
+        fork.record(cur)
+        for s in par_streams:
+            s.wait_event(fork)
+        for i in range(args.steps):
+            par_call(i, cur if i % n_par == 0 else par_streams[i % n_par - 1])
+        for s in par_streams:
+            e = torch.cuda.Event()
+            e.record(s)
+            cur.wait_event(e)
+
+    par_med, par_min = time_graph(torch, decode_step, args.steps, warm_launches=max(400, args.warmup),
+                                  eager=args.eager, whole=par_whole)
+    par_s = par_med / args.steps
+
     # ---------------- prefill ----------------
     p = PREFILL
     pw_bits = H.make_weight(p["K"], p["N"], dt, seed=1236)
@@ -681,6 +720,10 @@ def main():
             "mfma_ceiling_tflops": round(ceil_tf, 1),
             "read_floor_gbs": round(wbytes / floor_s / 1e9, 1),
             "read_floor_ms_per_step": round(floor_s * 1e3, 6),
+            # the same decode call, four independent calls in flight (no edge between them in the graph)
+            "decode_4_in_flight_gbs": round(wbytes / par_s / 1e9, 1),
+            "decode_4_in_flight_frac": round(wbytes / par_s / 1e9 / HBM_PEAK_GBS, 4),
+            "decode_4_in_flight_ms_per_step": round(par_s * 1e3, 6),
             "read_floor": {
                 "what": "wol_read_floor: the same weight copies read by a kernel of the same launch shape "
                         "that computes nothing (no scales, activations, MFMAs or output)",

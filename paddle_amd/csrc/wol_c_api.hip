@@ -250,6 +250,7 @@ int linear_impl(const void* x, const void* codes, const void* bias, const void* 
   int which = resolve_kernel(kernel, M, K, N, bits, group_size, workspace_bytes);
   if (which == WOL_KERNEL_BATCH_SPLIT && kernel == WOL_KERNEL_AUTO && fuse.pre_scale != nullptr)
     which = resolve_kernel(kernel, M, K, N, bits, group_size, 0);  // that kernel applies no pre-scale
+  if (fuse.act == WOL_ACT_SWIGLU && which != WOL_KERNEL_GEMM) return WOL_ERR_BAD_SHAPE;  // only the GEMM's epilogue forms it
   if (log_enabled())
     fprintf(stderr, "[wol] linear M=%lld K=%lld N=%lld int%d group=%d %s%s%s act=%d -> %s kernel\n",
             static_cast<long long>(M), static_cast<long long>(K), static_cast<long long>(N), bits, group_size,
@@ -407,7 +408,9 @@ FusedPlan plan_fused(int64_t M, int64_t K, int64_t N, int bits, int group_size, 
   const bool fused_pre = (which == WOL_KERNEL_BATCH && wol::linear_batch_fuses_pre_scale(K, bits, group_size)) ||
                          (which == WOL_KERNEL_STREAM && M == 1);
   f.prepass = has_pre && !fused_pre;
-  f.swiglu_pass = act == WOL_ACT_SWIGLU;
+  // the GEMM's large tiles form the swiglu in their epilogue; elsewhere it is a pass over fp32 sums
+  f.swiglu_pass = act == WOL_ACT_SWIGLU &&
+                  !(which == WOL_KERNEL_GEMM && wol::linear_gemm_fuses_swiglu(M, K, N, bits, group_size));
   auto up = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
   f.linear_ws = lws;
   f.x_off = up(lws);
@@ -450,7 +453,7 @@ int wol_linear_fused(const void* x, const void* pre_scale, const void* codes, co
   hipStream_t s = static_cast<hipStream_t>(stream);
   unsigned char* ws = static_cast<unsigned char*>(workspace);
   wol::Fuse fuse;
-  fuse.act = act == WOL_ACT_GELU ? WOL_ACT_GELU : WOL_ACT_NONE;
+  fuse.act = act == WOL_ACT_GELU || (act == WOL_ACT_SWIGLU && !f.swiglu_pass) ? act : WOL_ACT_NONE;
   const void* xin = x;
   if (f.prepass) {
     const int prc = wol::launch_prescale(x, pre_scale, dtype, M, K, ws + f.x_off, s);

@@ -330,6 +330,7 @@ size_t llm_int8_workspace(int64_t M, int64_t K, int64_t N);
 void llm_int8_workspace_offsets(int64_t M, int64_t K, int64_t N, int64_t* offsets);
 // Scratch bytes with which launch_linear_gemm splits K across workgroups (0: none needed).
 size_t linear_gemm_workspace(int64_t M, int64_t K, int64_t N, int bits, int group_size);
+bool linear_gemm_fuses_swiglu(int64_t M, int64_t K, int64_t N, int bits, int group_size);
 
 inline int check_launch() {
   return hipGetLastError() == hipSuccess ? WOL_OK : WOL_ERR_HIP;

@@ -432,7 +432,15 @@ struct MoeTile {
 // With nsplit > 1 a workgroup covers only a run of k tiles and leaves its
 // fp32 sums (scaled, without bias) in a partial buffer; reduce_partials_kernel
 // adds the runs.  That is what fills the CUs when M is small.
-template <int DT, int BITS, int G, bool OFFS, int WM, int WN, int TM, int TN, int STAGES>
+//
+// SWI != 0: swiglu in the epilogue (TN = 2, per-channel scales).  The weight is
+// a gate | up projection, [K, N] with the gate in columns 0 .. N/2-1; block 0
+// of every wavefront then takes 32 gate columns and block 1 the 32 up columns
+// N/2 further on, so that silu(gate) * up is formed lane by lane from the two
+// accumulators and only [M, N/2] leaves the kernel.  SWI = 1 applies it to the
+// fp32 sums (wol_linear_fused); SWI = 2 first rounds both sums to T, as a
+// separate fc1 output would have been (the mixture-of-experts FFN).
+template <int DT, int BITS, int G, bool OFFS, int WM, int WN, int TM, int TN, int STAGES, int SWI = 0>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   constexpr int NW = WM * WN;
@@ -463,6 +471,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   constexpr int kPerStage = kALoads + kBLoads + (G == 0 ? 0 : 1);
   static_assert(Q >= 2 && (Q - 2) % kFold != 0 && (Q - 2) % kFold != kFold - 1,
                 "the slice that holds the barrier neither starts nor ends a group");
+  static_assert(SWI == 0 || (TN == 2 && G == 0), "the swiglu epilogue pairs the two blocks of a wavefront");
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
   const uint16_t* __restrict__ x = p.x;
@@ -488,16 +497,18 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
     if (t.expert < 0) return;
     x += static_cast<int64_t>(t.row0) * K;
     if (p.nsplit > 1) outp = static_cast<float*>(outp) + static_cast<int64_t>(t.row0) * N;  // partial sums
-    else outp = static_cast<uint16_t*>(outp) + static_cast<int64_t>(t.row0) * N;
+    else outp = static_cast<uint16_t*>(outp) + static_cast<int64_t>(t.row0) * (SWI ? N / 2 : N);
     codes += static_cast<int64_t>(t.expert) * p.moe_codes_stride;
     scale += static_cast<int64_t>(t.expert) * N;
     if (bias != nullptr) bias += static_cast<int64_t>(t.expert) * N;
     M = t.rows;
     m0 = 0;
   }
-  const int strip_blk = p.strip_lo + bx * (BN / 16);
+  // SWI: a workgroup takes BN / 2 gate columns and the BN / 2 up columns that go with them
+  const int strip_blk = p.strip_lo + bx * (SWI ? BN / 32 : BN / 16);
   const int nstrips = p.strip_hi;
   const int n_hi = p.strip_hi * kStripCols;
+  const int up_strips = N / 2 / kStripCols;  // SWI: strips between a gate column and its up column
   // this workgroup's run of k tiles
   const int t0 = split * p.tiles_per_split;
   const int niter = (K / TK - t0) < p.tiles_per_split ? (K / TK - t0) : p.tiles_per_split;
@@ -521,7 +532,13 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
 #pragma unroll
   for (int c = 0; c < kBLoads; ++c) {
     int st = strip_blk + c * NW + wave;
+    if (SWI) {
+      // LDS slot L of the B tile serves wavefront column L / 4, block (L / 2) % 2, half L % 2
+      const int L = c * NW + wave;
+      st = strip_blk + (L / 4) * 2 + L % 2;
+    }
     st = st < nstrips ? st : nstrips - 1;  // past the last column: valid data, never stored
+    if (SWI && ((c * NW + wave) / 2) % 2 == 1) st += up_strips;  // block 1: the up columns
     bsrc[c] = codes + static_cast<int64_t>(st) * strip_bytes(K, BITS) +
               static_cast<int64_t>(t0) * 1024 + lane * 16;
   }
@@ -569,12 +586,13 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   auto seg_n = [&](int s) { return seg_lo(s + 1) - seg_lo(s); };
 
   // columns of this lane's accumulators: block c of the wavefront, column r32
-  const int col0 = (strip_blk + wn * TN * 2) * 16;
+  const int col0 = (strip_blk + wn * (SWI ? 1 : TN) * 2) * 16;
   int ncol[TN];
 #pragma unroll
   for (int c = 0; c < TN; ++c) {
     const int n = col0 + c * 32 + r32;
     ncol[c] = n < n_hi ? n : n_hi - 1;
+    if (SWI && c == 1) ncol[c] = ncol[0] + N / 2;
   }
   // this lane's scales of the tile in `stage`, out of LDS
   auto read_scales = [&](const unsigned char* stage, uint16_t (&dst)[kGT > 0 ? kGT : 1][TN]) {
@@ -803,26 +821,40 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
     return;
   }
   uint16_t* out = static_cast<uint16_t*>(outp);
-  constexpr int kSlabRow = TN * 32 + 8;  // padded, in elements
+  constexpr int kOutBlocks = SWI ? 1 : TN;        // 32-column blocks a wavefront writes
+  constexpr int kSlabRow = kOutBlocks * 32 + 8;   // padded, in elements
   static_assert(NW * 32 * kSlabRow * 2 <= kStages * kStage, "slabs must fit in the stage buffers");
   uint16_t* slab = reinterpret_cast<uint16_t*>(smem) + wave * 32 * kSlabRow;
-  constexpr int kPieces = 32 * (TN * 32 / 8);
+  constexpr int kPieces = 32 * (kOutBlocks * 32 / 8);
+  const int ld_out = SWI ? N / 2 : N;             // row length of the output
 #pragma unroll
   for (int a = 0; a < TM; ++a) {
+    if (SWI) {
 #pragma unroll
-    for (int c = 0; c < TN; ++c)
+      for (int r = 0; r < 16; ++r) {
+        float g = tot[a][0][r] * sc[0] + bv[0], u = tot[a][1][r] * sc[1] + bv[1];
+        if (SWI == 2) {  // as if fc1 had been written out in T and read back
+          g = to_f32<DT>(cast_out<DT>(g));
+          u = to_f32<DT>(cast_out<DT>(u));
+        }
+        slab[(8 * (r / 4) + 4 * b + r % 4) * kSlabRow + r32] = cast_out<DT>(act_swiglu(g, u));
+      }
+    } else {
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        slab[(8 * (r / 4) + 4 * b + r % 4) * kSlabRow + c * 32 + r32] =
-            cast_out<DT>(act_apply(tot[a][c][r] * sc[c] + bv[c], p.act));
+      for (int c = 0; c < TN; ++c)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          slab[(8 * (r / 4) + 4 * b + r % 4) * kSlabRow + c * 32 + r32] =
+              cast_out<DT>(act_apply(tot[a][c][r] * sc[c] + bv[c], p.act));
+    }
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int q = lane; q < kPieces; q += 64) {
-      const int r = q / (TN * 4), cc = q % (TN * 4);
+      const int r = q / (kOutBlocks * 4), cc = q % (kOutBlocks * 4);
       const int m = m0 + (wm * TM + a) * 32 + r;
       const int n = col0 + cc * 8;
       const u32x4 v = *reinterpret_cast<const u32x4*>(&slab[r * kSlabRow + cc * 8]);
-      if (m < M && n < n_hi) *reinterpret_cast<u32x4*>(out + static_cast<int64_t>(m) * N + n) = v;
+      if (m < M && n < n_hi) *reinterpret_cast<u32x4*>(out + static_cast<int64_t>(m) * ld_out + n) = v;
     }
     __builtin_amdgcn_wave_barrier();
   }
@@ -948,12 +980,14 @@ constexpr size_t dma_lds_bytes() {
 
 // Launches the fast kernel on the columns of strips [strip_lo, strip_hi), K
 // cut into nsplit runs (nsplit > 1 needs a.ws: nsplit x M x columns floats).
-template <int DT, int BITS, int G, bool OFFS, int WM, int WN, int TM, int TN, int STAGES = 3>
+// SWI != 0 (swiglu epilogue): the strips are those of the gate half, [0, N / 32), a.out is [M, N / 2].
+template <int DT, int BITS, int G, bool OFFS, int WM, int WN, int TM, int TN, int STAGES = 3, int SWI = 0>
 void launch_dma(const Args& a, int strip_lo, int strip_hi, int nsplit) {
-  constexpr int BM = WM * TM * 32, BN = WN * TN * 32, TK = BITS == 8 ? 64 : 128;
+  constexpr int BM = WM * TM * 32, BN = (SWI ? 1 : TN) * WN * 32, TK = BITS == 8 ? 64 : 128;
   if (strip_hi <= strip_lo) return;
+  if (SWI) nsplit = 1;
   constexpr size_t lds = dma_lds_bytes<BITS, G, WM, WN, TM, TN, STAGES>();
-  auto kern = gemm_dma_kernel<DT, BITS, G, OFFS, WM, WN, TM, TN, STAGES>;
+  auto kern = gemm_dma_kernel<DT, BITS, G, OFFS, WM, WN, TM, TN, STAGES, SWI>;
   static std::atomic<uint32_t> configured{0};  // per instantiation
   allow_lds(reinterpret_cast<const void*>(kern), lds, configured);
   const int ncols = (strip_hi - strip_lo) * kStripCols;
@@ -974,7 +1008,7 @@ void launch_dma(const Args& a, int strip_lo, int strip_hi, int nsplit) {
   const int tiles = a.K / TK;
   p.tiles_per_split = (tiles + nsplit - 1) / nsplit;
   p.nsplit = (tiles + p.tiles_per_split - 1) / p.tiles_per_split;
-  p.xcd_rows = plan_xcd_rows(p.nbx, p.nby, BM * 2, BN * BITS / 8);
+  p.xcd_rows = plan_xcd_rows(p.nbx, p.nby, BM * 2, WN * TN * 32 * BITS / 8);
   p.act = a.act;
   p.moe_table = nullptr;
   p.moe_codes_stride = 0;
@@ -1249,14 +1283,16 @@ struct MoeLaunch {
 
 // One grouped GEMM: every expert's rows against that expert's weights, tiles
 // of WM * TM * 32 rows x 256 columns, per-channel scales, out [rows, N] T.
-template <int DT, int BITS, bool OFFS, int WM, int WN, int TM, int TN, int STAGES>
+// SWI = 2: the swiglu of the fc1 output is formed in the epilogue and out is
+// [rows, N / 2] (the configurations with two blocks per wavefront).
+template <int DT, int BITS, bool OFFS, int WM, int WN, int TM, int TN, int STAGES, int SWI = 0>
 void launch_moe_gemm_cfg(const void* x, const MoeLaunch& ml, const void* codes, const void* bias,
                          const void* scale, int64_t K, int64_t N, void* out, hipStream_t stream) {
   const int* table = ml.table;
   const int max_tiles = ml.max_tiles;
-  constexpr int BN = WN * TN * 32;
+  constexpr int BN = (SWI ? 1 : TN) * WN * 32;  // output columns of a tile
   constexpr size_t lds = dma_lds_bytes<BITS, 0, WM, WN, TM, TN, STAGES>();
-  auto kern = gemm_dma_kernel<DT, BITS, 0, OFFS, WM, WN, TM, TN, STAGES>;
+  auto kern = gemm_dma_kernel<DT, BITS, 0, OFFS, WM, WN, TM, TN, STAGES, SWI>;
   static std::atomic<uint32_t> configured{0};
   allow_lds(reinterpret_cast<const void*>(kern), lds, configured);
   DmaParams p;
@@ -1265,11 +1301,12 @@ void launch_moe_gemm_cfg(const void* x, const MoeLaunch& ml, const void* codes, 
   p.bias = static_cast<const uint16_t*>(bias);
   p.scale = static_cast<const uint16_t*>(scale);
   const int tiles = static_cast<int>(K / (BITS == 8 ? 64 : 128));
-  const int ns = bias == nullptr && ml.partial != nullptr ? ml.ns : 1;
+  const int ns = !SWI && bias == nullptr && ml.partial != nullptr ? ml.ns : 1;
   p.M = WM * TM * 32; p.K = static_cast<int>(K); p.N = static_cast<int>(N);
   p.out_f32 = 0;
-  p.strip_lo = 0; p.strip_hi = static_cast<int>(N / kStripCols);
-  p.nbx = static_cast<int>((N + BN - 1) / BN);
+  const int64_t out_cols = SWI ? N / 2 : N;
+  p.strip_lo = 0; p.strip_hi = static_cast<int>(out_cols / kStripCols);
+  p.nbx = static_cast<int>((out_cols + BN - 1) / BN);
   p.nby = max_tiles;
   p.tiles_per_split = (tiles + ns - 1) / ns;
   p.nsplit = (tiles + p.tiles_per_split - 1) / p.tiles_per_split;
@@ -1288,11 +1325,25 @@ void launch_moe_gemm_cfg(const void* x, const MoeLaunch& ml, const void* codes, 
   }
 }
 
-// ml.bm: the tile rows the table was built for (moe_tile_rows)
+// Whether the grouped GEMM with tiles of bm rows forms the swiglu of its output itself.
+inline bool moe_fuses_swiglu(int bm) { return bm >= 128; }
+
+// ml.bm: the tile rows the table was built for (moe_tile_rows).  swiglu: out is
+// [rows, N / 2], the swiglu of the product (only where moe_fuses_swiglu(ml.bm)).
 template <int DT, int BITS>
 void launch_moe_gemm(const void* x, const MoeLaunch& ml, const void* codes, const void* bias,
-                     const void* scale, int64_t K, int64_t N, void* out, hipStream_t stream) {
+                     const void* scale, int64_t K, int64_t N, void* out, hipStream_t stream, bool swiglu = false) {
   constexpr bool kOffs = BITS == 4 && DT == WOL_DTYPE_BF16;  // as the ungrouped launch chooses
+  if (swiglu) {
+    if constexpr (BITS == 8) {
+      if (ml.bm == 256) {
+        launch_moe_gemm_cfg<DT, 8, false, 2, 4, 4, 2, 3, 2>(x, ml, codes, bias, scale, K, N, out, stream);
+        return;
+      }
+    }
+    launch_moe_gemm_cfg<DT, BITS, kOffs, 2, 4, 2, 2, 3, 2>(x, ml, codes, bias, scale, K, N, out, stream);
+    return;
+  }
   if constexpr (BITS == 4) {
     if (ml.bm == 32) {
       launch_moe_gemm_cfg<DT, 4, true, 1, 8, 1, 1, 2>(x, ml, codes, bias, scale, K, N, out, stream);
@@ -1405,6 +1456,28 @@ void describe_linear_gemm(int64_t M, int64_t K, int64_t N, int bits, int group_s
                     t.ns > 1 ? " with K in runs + reduce_partials_kernel" : "");
 }
 
+// swiglu of a gate | up projection inside the GEMM's epilogue: the tiles with two
+// blocks per wavefront, per-channel scales, above the small-M configurations.
+bool linear_gemm_fuses_swiglu(int64_t M, int64_t K, int64_t N, int bits, int group_size) {
+  const int tk = bits == 8 ? 64 : 128;
+  return M > kSkinnyMaxM && group_size == -1 && K % tk == 0 && K / tk >= 2 && N % 32 == 0;
+}
+
+namespace {
+// out [M, N / 2] = T(swiglu(x . W + bias)) in one launch
+template <int DT, int BITS>
+void launch_swiglu_gemm(const Args& a) {
+  const int gate_strips = a.N / 2 / kStripCols;
+  if constexpr (BITS == 8) {
+    if (a.M >= 192) launch_dma<DT, 8, 0, false, 2, 4, 4, 2, 3, 1>(a, 0, gate_strips, 1);
+    else launch_dma<DT, 8, 0, false, 2, 4, 2, 2, 3, 1>(a, 0, gate_strips, 1);
+  } else {
+    launch_dma<DT, 4, 0, DT == WOL_DTYPE_BF16, 2, 4, 2, 2, 3, 1>(a, 0, gate_strips, 1);
+  }
+}
+}  // namespace
+
+// f.act == WOL_ACT_SWIGLU (only where linear_gemm_fuses_swiglu): out is [M, N / 2] T.
 int launch_linear_gemm(const void* x, const void* codes, const void* bias, const void* scale,
                        int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
                        void* out, bool out_f32, void* workspace, size_t workspace_bytes,
@@ -1412,6 +1485,15 @@ int launch_linear_gemm(const void* x, const void* codes, const void* bias, const
   const int gshift = group_size == 64 ? 6 : (group_size == 128 ? 7 : -1);
   const Args a{x, codes, bias, scale, out, static_cast<int>(M), static_cast<int>(K),
                static_cast<int>(N), gshift, out_f32 ? 1 : 0, workspace, workspace_bytes, stream, f.act};
+  if (f.act == WOL_ACT_SWIGLU) {
+    if (out_f32 || !linear_gemm_fuses_swiglu(M, K, N, bits, group_size)) return WOL_ERR_BAD_SHAPE;
+    if (dtype == WOL_DTYPE_BF16) {
+      if (bits == 8) launch_swiglu_gemm<WOL_DTYPE_BF16, 8>(a); else launch_swiglu_gemm<WOL_DTYPE_BF16, 4>(a);
+    } else {
+      if (bits == 8) launch_swiglu_gemm<WOL_DTYPE_F16, 8>(a); else launch_swiglu_gemm<WOL_DTYPE_F16, 4>(a);
+    }
+    return check_launch();
+  }
   if (dtype == WOL_DTYPE_BF16) {
     if (bits == 8) launch_cfg<WOL_DTYPE_BF16, 8>(a); else launch_cfg<WOL_DTYPE_BF16, 4>(a);
   } else {
@@ -1457,9 +1539,13 @@ int launch_moe_ffn(const void* x, const int64_t* rows_before_expert, const void*
   moe_plan_kernel<<<dim3(1), dim3(256), 0, stream>>>(rows_before_expert, num_experts, bm, max_tiles, rows, table);
 #define WOL_MOE(DT, B)                                                                                        \
   do {                                                                                                        \
-    launch_moe_gemm<DT, B>(x, l1, ffn1_codes, ffn1_bias, ffn1_scale, hidden, inter, fc1, stream);  \
-    const int rc = launch_swiglu_t(fc1, dtype, rows, inter, act, stream);                                     \
-    if (rc != WOL_OK) return rc;                                                                              \
+    if (moe_fuses_swiglu(bm)) {                                                                               \
+      launch_moe_gemm<DT, B>(x, l1, ffn1_codes, ffn1_bias, ffn1_scale, hidden, inter, act, stream, true);     \
+    } else {                                                                                                  \
+      launch_moe_gemm<DT, B>(x, l1, ffn1_codes, ffn1_bias, ffn1_scale, hidden, inter, fc1, stream);           \
+      const int rc = launch_swiglu_t(fc1, dtype, rows, inter, act, stream);                                   \
+      if (rc != WOL_OK) return rc;                                                                            \
+    }                                                                                                         \
     launch_moe_gemm<DT, B>(act, l2, ffn2_codes, nullptr, ffn2_scale, inter / 2, hidden, out, stream); \
   } while (0)
   if (dtype == WOL_DTYPE_BF16) {

@@ -113,6 +113,32 @@ def test_fused_against_oracle(device, oracle, dt, bits, g):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dt", [H.F16, H.BF16])
+@pytest.mark.parametrize("bits", [8, 4])
+def test_swiglu_in_the_gemm_epilogue(device, oracle, dt, bits):
+    # above 64 rows with per-channel scales the GEMM pairs gate and up columns in
+    # one wavefront and writes [M, N/2] itself: no fp32 sums, no extra pass.
+    # 128-row and 256-row tiles, rows off the tile height, a gate half that ends
+    # inside a column tile (N/2 = 1168), with and without bias
+    from paddle_amd import _lib
+
+    for M, K, N in ((100, 512, 1024), (200, 512, 512), (300, 1024, 2336), (513, 256, 768)):
+        assert _lib.lib.wol_linear_fused_workspace(M, K, N, bits, -1, 0, 2) == _lib.lib.wol_linear_workspace(M, K, N, bits, -1)
+        assert _lib.lib.wol_linear_fused_workspace(M, K, N, bits, 128, 0, 2) >= M * N * 4  # group-wise: the pass
+        wb = H.make_weight(K, N, dt, seed=K + N + M)
+        xb = H.make_act(M, K, dt, seed=M)
+        bb = H.make_bias(N, dt, seed=6)
+        oc, osc = oracle.weight_quantize(wb, dt, bits, -1)
+        packed = H.gfx950_from_q(H.q_from_canonical(oc, bits), bits)
+        for bias in (None, bb):
+            _, wantT = oracle.linear_fused(xb, None, oc, osc, bias, dt, bits, -1, 2)
+            got = _fused(xb, None, packed, bias, osc, dt, N, bits, -1, 2)
+            assert got.shape == (M, N // 2)
+            err = H.rel_l2(H.bits_to_f32(got, dt), H.bits_to_f32(wantT, dt))
+            assert err <= TOL, (err, dt, bits, M, K, N, bias is not None)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
 def test_fused_pre_scale_equals_the_two_ops(device, oracle, dt):
     # folding apply_per_channel_scale into the linear must not change a bit:
     # the same products, rounded the same way, enter the same kernel
