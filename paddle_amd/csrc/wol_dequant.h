@@ -29,6 +29,7 @@ __device__ inline uint32_t and_or(uint32_t v, uint32_t mask, uint32_t magic) {
 template <>
 struct Dequant<WOL_DTYPE_BF16, 4> {
   static constexpr uint32_t kCancel = 0xC308C308u;  // -136, -136
+  static constexpr float kOffset = 136.0f;
   static constexpr uint32_t kMagic = 0x43004300u;
   __device__ static inline u32x4 run(const uint32_t* w, uint32_t magic) {
     const uint32_t v = w[0];
@@ -44,6 +45,7 @@ struct Dequant<WOL_DTYPE_BF16, 4> {
 template <>
 struct Dequant<WOL_DTYPE_F16, 4> {
   static constexpr uint32_t kCancel = 0xD480D480u;  // -72, -72
+  static constexpr float kOffset = 72.0f;
   static constexpr uint32_t kMagic = 0x54005400u;
   __device__ static inline u32x4 run(const uint32_t* w, uint32_t magic) {
     const uint32_t v = w[0];
@@ -59,6 +61,7 @@ struct Dequant<WOL_DTYPE_F16, 4> {
 template <>
 struct Dequant<WOL_DTYPE_BF16, 8> {
   static constexpr uint32_t kCancel = 0xC300C300u;  // -128, -128
+  static constexpr float kOffset = 128.0f;
   static constexpr uint32_t kMagic = 0u;
   __device__ static inline uint32_t pair(uint32_t lo_byte_val, uint32_t hi_byte_val) {
     // high halves of two fp32 values side by side (both are exact in bf16)
@@ -78,6 +81,7 @@ struct Dequant<WOL_DTYPE_BF16, 8> {
 template <>
 struct Dequant<WOL_DTYPE_F16, 8> {
   static constexpr uint32_t kCancel = 0xE480E480u;  // -1152, -1152
+  static constexpr float kOffset = 1152.0f;
   static constexpr uint32_t kMagic = 0x64646464u;
   __device__ static inline u32x4 run(const uint32_t* w, uint32_t magic) {
     u32x4 o;

@@ -370,6 +370,23 @@ __device__ inline f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
                                                 __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
 }
 
+// acc + the sum of the eight T values of an operand fragment, in fp32 (four
+// packed dot products against (1, 1)).
+template <int DT>
+__device__ inline float sum8(u32x4 v, float acc) {
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  typedef _Float16 h16x2 __attribute__((ext_vector_type(2)));
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if (DT == WOL_DTYPE_BF16)
+      acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, w[i]), __builtin_bit_cast(bf16x2, 0x3F803F80u), acc, false);
+    else
+      acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h16x2, w[i]), __builtin_bit_cast(h16x2, 0x3C003C00u), acc, false);
+  }
+  return acc;
+}
+
 // What one launch of the fast kernel works on.
 struct DmaParams {
   const uint16_t* x;
@@ -423,11 +440,16 @@ struct MoeTile {
 // folded into the running sum with the group's scale (an fp32 FMA per
 // accumulator element), so code * scale is never rounded to T.
 //
-// OFFS selects the offset dequantiser: a fraction of the VALU work, paid for
-// with one more MFMA per A fragment and slice (into `canc`, which holds
-// -offset * sum of the activations and is added when the scale is applied).
-// It is the right trade when M is small: the matrix pipe idles, the VALU does
-// not.
+// OFFS selects the offset dequantiser: a fraction of the VALU work, and the
+// constant offset of every code is taken out again as -offset * (sum of the
+// row's activations).  OFFS = 1 forms that sum with one more MFMA per A
+// fragment and slice against a constant B operand (into `canc`, added when
+// the scale is applied) -- the right trade when M is small: the matrix pipe
+// idles, the VALU does not.  OFFS = 2 forms it with four packed dot products
+// per A fragment (a lane adds up the eight activations of its fragment; the
+// two lanes that share a row meet in the epilogue), which costs no MFMA and
+// no accumulators and is what lets int4 weights under bf16 activations take
+// the largest tile; per-channel scales only.
 //
 // With nsplit > 1 a workgroup covers only a run of k tiles and leaves its
 // fp32 sums (scaled, without bias) in a partial buffer; reduce_partials_kernel
@@ -440,7 +462,7 @@ struct MoeTile {
 // accumulators and only [M, N/2] leaves the kernel.  SWI = 1 applies it to the
 // fp32 sums (wol_linear_fused); SWI = 2 first rounds both sums to T, as a
 // separate fc1 output would have been (the mixture-of-experts FFN).
-template <int DT, int BITS, int G, bool OFFS, int WM, int WN, int TM, int TN, int STAGES, int SWI = 0>
+template <int DT, int BITS, int G, int OFFS, int WM, int WN, int TM, int TN, int STAGES, int SWI = 0>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   constexpr int NW = WM * WN;
@@ -472,6 +494,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   static_assert(Q >= 2 && (Q - 2) % kFold != 0 && (Q - 2) % kFold != kFold - 1,
                 "the slice that holds the barrier neither starts nor ends a group");
   static_assert(SWI == 0 || (TN == 2 && G == 0), "the swiglu epilogue pairs the two blocks of a wavefront");
+  static_assert(OFFS != 2 || G == 0, "row sums by dot products are taken out once, in the epilogue");
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
   const uint16_t* __restrict__ x = p.x;
@@ -608,17 +631,19 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
 
   f32x16 tot[TM][TN];
   f32x16 part[G != 0 ? TM : 1][G != 0 ? TN : 1];
-  f32x16 canc[OFFS ? TM : 1];
+  f32x16 canc[OFFS == 1 ? TM : 1];
+  float rsum[OFFS == 2 ? TM : 1];  // this lane's share of the sum of the activations of row r32 of block a
 #pragma unroll
   for (int a = 0; a < TM; ++a) {
 #pragma unroll
     for (int c = 0; c < TN; ++c)
 #pragma unroll
       for (int r = 0; r < 16; ++r) tot[a][c][r] = 0.0f;
-    if (OFFS) {
+    if (OFFS == 1) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) canc[a][r] = 0.0f;
     }
+    if (OFFS == 2) rsum[a] = 0.0f;
   }
   uint32_t magic = Dequant<DT, BITS>::kMagic;
   asm volatile("" : "+v"(magic));  // keep the constant in a VGPR
@@ -626,7 +651,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   // byte offsets inside a stage that do not change from tile to tile
   const int a_row_off = (wm * TM * 32 + r32) * (TK * 2);
   const int b_off = kABytes + (wn * TN * 2 + sp) * 1024 + (j + 16 * b) * 16;
-  constexpr int kValuPerMfma = ((BITS == 8 ? 16 : 12) * TN + TM * TN - 1) / (TM * TN) + 2;
+  constexpr int kValuPerMfma = ((OFFS == 2 ? 4 * TN + 4 * TM : (BITS == 8 ? 16 : 12) * TN) + TM * TN - 1) / (TM * TN) + 2;
   constexpr int kHalf = (TM * TN + 1) / 2;  // MFMAs of a slice issued before the barrier
 
   // The wavefront's pipeline registers: raw codes of the current and the next
@@ -671,7 +696,13 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
 #pragma unroll
       for (int c = 0; c < TN; ++c)
         if (a * TN + c >= lo && a * TN + c < hi) {
-          if (OFFS && c == 0) {
+          if (OFFS == 2 && c == 0) {
+            rsum[a] = sum8<DT>(a4[a], rsum[a]);
+            // pinned to this slice: left alone the compiler sinks the sums of a
+            // whole tile behind the loop's branch and keeps every fragment alive for them
+            asm volatile("" : "+v"(rsum[a]));
+          }
+          if (OFFS == 1 && c == 0) {
             const u32x4 cb = {Dequant<DT, BITS>::kCancel, Dequant<DT, BITS>::kCancel,
                               Dequant<DT, BITS>::kCancel, Dequant<DT, BITS>::kCancel};
             canc[a] = mfma32<DT>(a4[a], cb, (G != 0 && first) ? zero : canc[a]);
@@ -695,7 +726,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
         for (int a = 0; a < TM; ++a)
 #pragma unroll
           for (int r = 0; r < 16; ++r)
-            tot[a][c][r] = fmaf(OFFS ? part[a][c][r] + canc[a][r] : part[a][c][r], sc, tot[a][c][r]);
+            tot[a][c][r] = fmaf(OFFS == 1 ? part[a][c][r] + canc[a][r] : part[a][c][r], sc, tot[a][c][r]);
       }
     }
   };
@@ -789,13 +820,38 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
     sc[c] = G == 0 ? to_f32<DT>(scale[ncol[c]]) : 1.0f;
     bv[c] = (bias != nullptr && p.nsplit == 1) ? to_f32<DT>(bias[ncol[c]]) : 0.0f;
   }
-  if (OFFS && G == 0) {
+  if (OFFS == 1 && G == 0) {
 #pragma unroll
     for (int a = 0; a < TM; ++a)
 #pragma unroll
       for (int c = 0; c < TN; ++c)
 #pragma unroll
         for (int r = 0; r < 16; ++r) tot[a][c][r] += canc[a][r];
+  }
+  if (OFFS == 2) {
+    // Row sums: lanes l and l + 32 hold the two halves of row r32's sum.  They
+    // are added and parked in LDS (the stages are free now), from where a lane
+    // takes the sums of the sixteen rows its accumulators belong to.
+    constexpr int kRsOff = kStages * kStage - NW * TM * 32 * 4;  // the end of the stages; the slabs use their start
+    static_assert(kRsOff >= NW * 32 * ((SWI ? 1 : TN) * 32 + 8) * 2, "row sums and slabs must not overlap");
+    float* rsl = reinterpret_cast<float*>(smem + kRsOff) + wave * TM * 32;
+#pragma unroll
+    for (int a = 0; a < TM; ++a) {
+      const float other = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(((lane ^ 32) << 2), __builtin_bit_cast(int, rsum[a])));
+      if (b == 0) rsl[a * 32 + r32] = rsum[a] + other;
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const f32x4 rv = *reinterpret_cast<const f32x4*>(&rsl[a * 32 + 8 * q4 + 4 * b]);
+#pragma unroll
+        for (int c = 0; c < TN; ++c)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) tot[a][c][4 * q4 + e] = fmaf(-Dequant<DT, BITS>::kOffset, rv[e], tot[a][c][4 * q4 + e]);
+      }
+    __builtin_amdgcn_wave_barrier();
   }
   if (p.out_f32 || p.nsplit > 1) {
     // fp32 results (verification mode) or partial sums of this run of k tiles: plain stores
@@ -981,7 +1037,7 @@ constexpr size_t dma_lds_bytes() {
 // Launches the fast kernel on the columns of strips [strip_lo, strip_hi), K
 // cut into nsplit runs (nsplit > 1 needs a.ws: nsplit x M x columns floats).
 // SWI != 0 (swiglu epilogue): the strips are those of the gate half, [0, N / 32), a.out is [M, N / 2].
-template <int DT, int BITS, int G, bool OFFS, int WM, int WN, int TM, int TN, int STAGES = 3, int SWI = 0>
+template <int DT, int BITS, int G, int OFFS, int WM, int WN, int TM, int TN, int STAGES = 3, int SWI = 0>
 void launch_dma(const Args& a, int strip_lo, int strip_hi, int nsplit) {
   constexpr int BM = WM * TM * 32, BN = (SWI ? 1 : TN) * WN * 32, TK = BITS == 8 ? 64 : 128;
   if (strip_hi <= strip_lo) return;
@@ -1035,11 +1091,11 @@ inline bool tall_half_tile(int M) {
 // columns run with 128-row tiles.  Cost model: a workgroup owns its CU, so a
 // launch takes ceil(tiles / CUs) tile times; a half-size tile costs kSmall of a
 // full one (a little more than half).
-inline int plan_big_columns(int M, int N) {
+inline int plan_big_columns(int M, int N, bool tall_ok = true) {
   const int cus = num_cus();
   constexpr double kSmall = 0.55;
   const int nbx = (N + 255) / 256, nby_big = (M + 255) / 256, nby_small = (M + 127) / 128;
-  const bool tall = tall_half_tile(M);  // half tiles of 256 x 128 instead of 128 x 256
+  const bool tall = tall_ok && tall_half_tile(M);  // half tiles of 256 x 128 instead of 128 x 256
   int best = nbx;
   double best_t = 1e30;
   for (int c = nbx; c >= 0; --c) {
@@ -1114,8 +1170,8 @@ inline SkinnyPlan plan_skinny(int M, int K, int N, int bits, int group, size_t w
 // 256 x 256 tiles (above 64 rows), and the first strip of those columns.
 inline void half_tile_config(int M, int N, int bits, int group, int* bm, int* bn, int* strip_lo) {
   *strip_lo = 0;
-  if (bits == 8 && group == 0) {
-    const int c = plan_big_columns(M, N) * 16, nstrips = N / kStripCols;
+  if (group == 0) {  // per-channel scales: 256 x 256 tiles on whole rounds of the CUs
+    const int c = plan_big_columns(M, N, bits == 8) * 16, nstrips = N / kStripCols;
     *strip_lo = c < nstrips ? c : nstrips;
   }
   if (bits == 8) {
@@ -1204,8 +1260,14 @@ void launch_fast(const Args& a) {
     WOL_HALF(false, 2, 4, 2, 1);
   } else if constexpr (G == 0 && DT == WOL_DTYPE_BF16) {
     // the exact int4 -> bf16 dequantiser costs 32 VALU instructions per 8
-    // codes; the offset form plus one cancelling MFMA per A block is faster
+    // codes; the offset form is faster: with row sums by dot products on the
+    // 256 x 256 tile (two stages of 64 + 16 KiB fill the LDS), with one
+    // cancelling MFMA per A block on the 128 x 256 tiles of the remainder
+    launch_dma<DT, BITS, G, 2, 2, 4, 4, 2, 2>(a, 0, lo, 1);
     WOL_HALF(true, 2, 4, 2, 2);
+  } else if constexpr (G == 0) {
+    launch_dma<DT, BITS, G, 0, 2, 4, 4, 2, 2>(a, 0, lo, 1);
+    WOL_HALF(false, 2, 4, 2, 2);
   } else {
     WOL_HALF(false, 2, 4, 2, 2);
   }
@@ -1258,14 +1320,14 @@ __global__ __launch_bounds__(256) void moe_plan_kernel(const int64_t* __restrict
 // when the experts have few rows each -- a decode step of a mixture of
 // experts -- where the large tile would do up to eight times the MFMA work
 // and hold one workgroup per CU where three fit.
-// From 512 rows per expert on, int8 takes the 256 x 256 tile of the ungrouped
-// prefill launch (more MFMAs per dequantised fragment; a partial last tile per
-// expert then weighs little).
+// From 512 rows per expert on, the 256 x 256 tile of the ungrouped prefill
+// launch (more MFMAs per dequantised fragment; a partial last tile per expert
+// then weighs little).
 inline int moe_tile_rows(int64_t rows, int num_experts, int bits) {
   const int64_t avg = rows / (num_experts > 0 ? num_experts : 1);
   if (avg <= 32 && bits == 4) return 32;
   if (avg <= 64) return 64;
-  if (avg >= 512 && bits == 8) return 256;
+  if (avg >= 512) return 256;
   return 128;
 }
 
@@ -1285,7 +1347,7 @@ struct MoeLaunch {
 // of WM * TM * 32 rows x 256 columns, per-channel scales, out [rows, N] T.
 // SWI = 2: the swiglu of the fc1 output is formed in the epilogue and out is
 // [rows, N / 2] (the configurations with two blocks per wavefront).
-template <int DT, int BITS, bool OFFS, int WM, int WN, int TM, int TN, int STAGES, int SWI = 0>
+template <int DT, int BITS, int OFFS, int WM, int WN, int TM, int TN, int STAGES, int SWI = 0>
 void launch_moe_gemm_cfg(const void* x, const MoeLaunch& ml, const void* codes, const void* bias,
                          const void* scale, int64_t K, int64_t N, void* out, hipStream_t stream) {
   const int* table = ml.table;
@@ -1334,14 +1396,13 @@ template <int DT, int BITS>
 void launch_moe_gemm(const void* x, const MoeLaunch& ml, const void* codes, const void* bias,
                      const void* scale, int64_t K, int64_t N, void* out, hipStream_t stream, bool swiglu = false) {
   constexpr bool kOffs = BITS == 4 && DT == WOL_DTYPE_BF16;  // as the ungrouped launch chooses
+  constexpr int kBigOffs = kOffs ? 2 : 0;           // the 256-row tile: row sums by dot products
+  constexpr int kBigStages = BITS == 8 ? 3 : 2;     // 128-deep int4 tiles: two stages fill the LDS
   if (swiglu) {
-    if constexpr (BITS == 8) {
-      if (ml.bm == 256) {
-        launch_moe_gemm_cfg<DT, 8, false, 2, 4, 4, 2, 3, 2>(x, ml, codes, bias, scale, K, N, out, stream);
-        return;
-      }
-    }
-    launch_moe_gemm_cfg<DT, BITS, kOffs, 2, 4, 2, 2, 3, 2>(x, ml, codes, bias, scale, K, N, out, stream);
+    if (ml.bm == 256)
+      launch_moe_gemm_cfg<DT, BITS, kBigOffs, 2, 4, 4, 2, kBigStages, 2>(x, ml, codes, bias, scale, K, N, out, stream);
+    else
+      launch_moe_gemm_cfg<DT, BITS, kOffs, 2, 4, 2, 2, 3, 2>(x, ml, codes, bias, scale, K, N, out, stream);
     return;
   }
   if constexpr (BITS == 4) {
@@ -1350,11 +1411,9 @@ void launch_moe_gemm(const void* x, const MoeLaunch& ml, const void* codes, cons
       return;
     }
   }
-  if constexpr (BITS == 8) {
-    if (ml.bm == 256) {
-      launch_moe_gemm_cfg<DT, 8, false, 2, 4, 4, 2, 3>(x, ml, codes, bias, scale, K, N, out, stream);
-      return;
-    }
+  if (ml.bm == 256) {
+    launch_moe_gemm_cfg<DT, BITS, kBigOffs, 2, 4, 4, 2, kBigStages>(x, ml, codes, bias, scale, K, N, out, stream);
+    return;
   }
   if (ml.bm == 64)
     launch_moe_gemm_cfg<DT, BITS, false, 1, 8, 2, 1, 2>(x, ml, codes, bias, scale, K, N, out, stream);
@@ -1472,7 +1531,8 @@ void launch_swiglu_gemm(const Args& a) {
     if (a.M >= 192) launch_dma<DT, 8, 0, false, 2, 4, 4, 2, 3, 1>(a, 0, gate_strips, 1);
     else launch_dma<DT, 8, 0, false, 2, 4, 2, 2, 3, 1>(a, 0, gate_strips, 1);
   } else {
-    launch_dma<DT, 4, 0, DT == WOL_DTYPE_BF16, 2, 4, 2, 2, 3, 1>(a, 0, gate_strips, 1);
+    if (a.M >= 192) launch_dma<DT, 4, 0, DT == WOL_DTYPE_BF16 ? 2 : 0, 2, 4, 4, 2, 2, 1>(a, 0, gate_strips, 1);
+    else launch_dma<DT, 4, 0, DT == WOL_DTYPE_BF16 ? 1 : 0, 2, 4, 2, 2, 3, 1>(a, 0, gate_strips, 1);
   }
 }
 }  // namespace

@@ -590,6 +590,19 @@ def test_config_4_full_size_properties(device, M):
     _full_size_properties(H.BF16, 8, -1, M, 4096, 12288)
 
 
+@pytest.mark.parametrize("dt", [H.BF16, H.F16])
+def test_int4_prefill_full_size_properties(device, dt):
+    # int4 per-channel at prefill size: 256 x 256 tiles on the columns of whole
+    # rounds (bf16: offset dequantiser with row sums by dot products; fp16: the
+    # exact dequantiser), 128 x 256 tiles on the rest
+    from paddle_amd import _lib
+    import ctypes
+
+    buf = ctypes.create_string_buffer(256)
+    assert _lib.lib.wol_linear_plan(2048, 4096, 12288, 4, -1, 0, buf, 256) == 0 and b"256x256" in buf.value
+    _full_size_properties(dt, 4, -1, 2048, 4096, 12288)
+
+
 @pytest.mark.parametrize("shape", [(8, 4096, 22016), (1024, 4096, 22016), (1024, 11008, 4096), (1024, 4096, 12288)])
 def test_config_5_full_size_properties(device, shape):
     _full_size_properties(H.BF16, 8, 64, *shape)
