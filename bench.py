@@ -449,6 +449,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU timing (parity still runs)")
     ap.add_argument("--no-llm-int8", action="store_true", help="skip the llm_int8_linear timing")
     ap.add_argument("--no-configs", action="store_true", help="skip the per-configuration table")
+    ap.add_argument("--no-ladder", action="store_true", help="skip the wol_mfma_probe ladder")
     ap.add_argument("--quick", action="store_true", help="shorter per-configuration runs, 8 decoder layers")
     ap.add_argument("--eager", action="store_true", help="time eager launches instead of a graph")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -586,6 +587,25 @@ def main():
 
     ceil_med, _ = time_graph(torch, ceil_step, 4, warm_launches=8, warm_ms=30.0, replays=5, eager=args.eager)
     ceil_tf = ceil_wgs * 8.0 * ceil_iters * 8 * 2 * 32 * 32 * 16 / (ceil_med / 4) / 1e12
+
+    # the prefill tile's inner loop with its ingredients switched on one at a time (wol_mfma_probe)
+    ladder = None
+    if not args.no_ladder:
+        probe_ops = torch.randn(12 * 1024 * 1024 + 65536, device=dev).to(torch.bfloat16)  # > WOL_MFMA_PROBE_OPERAND_BYTES
+        names = ["mfma_only", "plus_dequant", "plus_a_reads", "plus_dequant_and_a_reads", "plus_barrier",
+                 "plus_barrier_and_tile_loads", "mfma_barrier_and_tile_loads", "mfma16x16x32_only",
+                 "mfma16x16x32_dequant_a_reads_barrier"]
+        p_wgs, p_iters = 1024, 400
+        p_out = torch.empty(p_wgs * 512, dtype=torch.float32, device=dev)
+        ladder = {}
+        for v, nm in enumerate(names):
+            def probe_step(_i, v=v):
+                _lib.check(_lib.lib.wol_mfma_probe(v, probe_ops.data_ptr(), probe_ops.numel() * 2, p_wgs, p_iters,
+                                                   p_out.data_ptr(), stream()))
+
+            med, _ = time_graph(torch, probe_step, 4, warm_launches=8, warm_ms=20.0, replays=5, eager=args.eager)
+            ladder[nm] = round(p_wgs * 8.0 * p_iters * 1048576 / (med / 4) / 1e12, 1)
+        del probe_ops
 
     # ---------------- llm_int8_linear on the prefill shape ----------------
     # the sibling op on the same weight (algo="llm.int8"): activations N(0,1)
@@ -753,6 +773,7 @@ def main():
                     "frac_of_peak": round(ceil_tf / MFMA_BF16_PEAK_TF, 4),
                     "prefill_over_ceiling": round(pre_tf / ceil_tf, 4),
                 },
+                "inner_loop_ladder_tflops": ladder,
             },
         },
         "configs": configs,
@@ -779,6 +800,8 @@ def main():
             flat["moe_ffn_rows%d_frac" % r["rows"]] = r["frac"]
     if llm:
         flat["llm_int8_frac"] = llm["roofline"]["frac"]
+    for nm, tf in (ladder or {}).items():
+        flat["ladder_%s_tflops" % nm] = tf
     print(json.dumps(out))
     if failures:
         print("bench.py: PARITY FAILURE: " + "; ".join(failures), file=sys.stderr)

@@ -129,6 +129,9 @@ int wol_quantize(const void* w, int dtype, int64_t K, int64_t N, int bits,
  * has no extra limit.  The call allocates and frees nothing.  All calls on one
  * GPU share that GPU's array: per-channel calls that overlap on one GPU (two
  * streams, two threads) race and must be serialised by the caller.
+ * The first call on a device looks up that device's properties and the
+ * address of its copy of the array; make one call outside of any stream
+ * capture (any size) before capturing calls on that device.
  */
 int wol_quantize_static(const void* w, int dtype, int64_t K, int64_t N, int bits,
                         int group_size, int round_mode, int layout,

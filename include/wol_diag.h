@@ -46,6 +46,32 @@ int wol_mfma_ceiling(const void* operands, int workgroups, int iters, float* out
                      void* stream);
 
 /*
+ * The inner loop of the prefill GEMM's 256 x 256 tile with its ingredients
+ * switched on one at a time, for a bottom-up account of where the matrix
+ * pipes' time goes: same register tile (4 x 2 blocks of 32 x 32 per
+ * wavefront, 8 wavefronts per workgroup, one workgroup per CU), same
+ * instruction mix per k tile, no global traffic unless the variant says so.
+ *   0  MFMAs only (what wol_mfma_ceiling measures)
+ *   1  + the int8 -> bf16 dequantisation of two B fragments per slice
+ *   2  + four A fragments read from LDS per slice
+ *   3  + both
+ *   4  + both and one workgroup barrier per k tile
+ *   5  + both, the barrier and six direct-to-LDS loads (1 KiB each) per
+ *        wavefront and k tile
+ *   6  MFMAs, the barrier and the loads only
+ *   7  v_mfma_f32_16x16x32 on 8 x 4 blocks, MFMAs only
+ *   8  the same with dequantisation, A reads and barrier
+ * operands: random bf16 data, at least WOL_MFMA_PROBE_OPERAND_BYTES of it
+ * (operand_bytes says how much).  A launch performs
+ *     workgroups * 8 * iters * 1048576 floating-point operations.
+ * out receives one float per thread (workgroups * 512).
+ */
+#define WOL_MFMA_PROBE_VARIANTS 9
+#define WOL_MFMA_PROBE_OPERAND_BYTES (64 * 8 * 49152 + 65536)
+int wol_mfma_probe(int variant, const void* operands, size_t operand_bytes,
+                   int workgroups, int iters, float* out, void* stream);
+
+/*
  * Writes into buf (NUL-terminated, at most buf_bytes) one line naming the
  * kernel and launch shape wol_linear takes for a problem when it is handed
  * workspace_bytes of scratch.  No device work.  For benchmarks and dispatch

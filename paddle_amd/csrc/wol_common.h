@@ -308,6 +308,7 @@ int launch_linear_grad(const void* out_grad, const void* codes, const void* scal
                        void* workspace, hipStream_t stream);
 int launch_read_floor(const void* codes, int64_t K, int64_t N, int bits, void* out,
                       hipStream_t stream);
+int launch_mfma_probe(int variant, const void* ops, int workgroups, int iters, float* out, hipStream_t stream);
 int launch_mfma_ceiling(const void* operands, int workgroups, int iters, float* out,
                         hipStream_t stream);
 int launch_prescale(const void* x, const void* scales, int dtype, int64_t rows, int64_t cols,

@@ -113,4 +113,14 @@ int wol_mfma_ceiling(const void* operands, int workgroups, int iters, float* out
   return wol::launch_mfma_ceiling(operands, workgroups, iters, out, static_cast<hipStream_t>(stream));
 }
 
+int wol_mfma_probe(int variant, const void* operands, size_t operand_bytes, int workgroups, int iters, float* out,
+                   void* stream) {
+  if (variant < 0 || variant >= WOL_MFMA_PROBE_VARIANTS) return WOL_ERR_BAD_SHAPE;
+  if (workgroups <= 0 || workgroups > 65536 || iters <= 0 || iters > (1 << 24)) return WOL_ERR_BAD_SHAPE;
+  if (operands == nullptr || out == nullptr) return WOL_ERR_NULL_POINTER;
+  if ((reinterpret_cast<uintptr_t>(operands) & 15u) != 0) return WOL_ERR_ALIGNMENT;
+  if (operand_bytes < WOL_MFMA_PROBE_OPERAND_BYTES) return WOL_ERR_WORKSPACE;  // the variants with loads read this much
+  return wol::launch_mfma_probe(variant, operands, workgroups, iters, out, static_cast<hipStream_t>(stream));
+}
+
 }  // extern "C"

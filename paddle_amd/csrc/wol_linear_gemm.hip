@@ -1617,4 +1617,187 @@ int launch_moe_ffn(const void* x, const int64_t* rows_before_expert, const void*
   return check_launch();
 }
 
+// ---- the prefill kernel's inner loop, one ingredient at a time (wol_mfma_probe) ----
+namespace {
+
+// The register tile and instruction mix of gemm_dma_kernel's 256 x 256
+// configuration (4 x 2 blocks of v_mfma_f32_32x32x16 per wavefront, k tiles of
+// four slices) with its ingredients switched on one by one, and no global
+// memory traffic other than what LOADS adds:
+//   DQ     B fragments dequantised per slice (int8 -> bf16, exact) out of raw
+//          codes read from LDS once per tile (0 or 2)
+//   NA     A fragments read from LDS per slice (0 or 4)
+//   BAR    one workgroup barrier per tile
+//   LOADS  six direct-to-LDS loads (1 KiB each) per wavefront and tile out of
+//          a 25 MB region of `ops`, two stages, waited for before the barrier
+//   M16    v_mfma_f32_16x16x32 on 8 x 4 blocks instead (the same flops)
+template <bool M16, int DQ, int NA, bool BAR, bool LOADS>
+__global__ __launch_bounds__(512) void mfma_probe_kernel(const u32x4* __restrict__ ops, int iters,
+                                                         float* __restrict__ out) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  for (int i = tid; i < 6144; i += 512) reinterpret_cast<u32x4*>(smem)[i] = ops[i & 511];  // 96 KiB of operand pattern
+  __syncthreads();
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const unsigned char* base = smem + (wave & 3) * 4096 + lane * 16;
+  float total = 0.0f;
+  if constexpr (!M16) {
+    f32x16 acc[4][2];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[a][c][r] = 0.0f;
+    u32x4 af[2][4], bf[2][2], raw[2][2];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) af[0][a] = af[1][a] = *reinterpret_cast<const u32x4*>(base + a * 1024);
+#pragma unroll
+    for (int c = 0; c < 2; ++c) bf[0][c] = bf[1][c] = *reinterpret_cast<const u32x4*>(base + 16384 + c * 1024);
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) raw[c][h] = *reinterpret_cast<const u32x4*>(base + 32768 + (c * 2 + h) * 1024);
+    for (int it = 0; it < iters; ++it) {
+      const unsigned char* tb = base + ((it & 3) << 14);
+      if (DQ > 0) {
+#pragma unroll
+        for (int c = 0; c < 2; ++c)
+#pragma unroll
+          for (int h = 0; h < 2; ++h) raw[c][h] = *reinterpret_cast<const u32x4*>(tb + (c * 2 + h) * 1024 + 8192);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        if (NA > 0) {
+#pragma unroll
+          for (int a = 0; a < NA; ++a)
+            af[(q + 1) & 1][a] = *reinterpret_cast<const u32x4*>(tb + ((q * 4 + a) & 7) * 1024);
+        }
+        if (DQ > 0) {
+          const int step = ((q + 1) & 3) / 2, h = (q + 1) % 2;
+#pragma unroll
+          for (int c = 0; c < DQ; ++c) {
+            const uint32_t w4[4] = {raw[c][h].x, raw[c][h].y, raw[c][h].z, raw[c][h].w};
+            bf[(q + 1) & 1][c] = DequantExact<WOL_DTYPE_BF16, 8>::run(&w4[step * 2]);
+          }
+        }
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+          for (int c = 0; c < 2; ++c) acc[a][c] = mfma32<WOL_DTYPE_BF16>(af[q & 1][a], bf[q & 1][c], acc[a][c]);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (i < NA) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          if (DQ > 0) __builtin_amdgcn_sched_group_barrier(0x002, (14 * DQ + 7) / 8 + 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (LOADS) {
+        wait_vmcnt<6>();
+        __builtin_amdgcn_s_barrier();
+        unsigned char* stage = smem + 65536 + (it & 1) * 49152;
+        const unsigned char* g = reinterpret_cast<const unsigned char*>(ops) +
+                                 ((static_cast<int>(blockIdx.x) & 63) * 8 + (it & 7)) * 49152;
+#pragma unroll
+        for (int c = 0; c < 6; ++c)
+          __builtin_amdgcn_global_load_lds(g + (c * 8 + wave) * 1024 + lane * 16,
+                                           (lds_ptr_t)(stage + (c * 8 + wave) * 1024), 16, 0, 0);
+      } else if (BAR) {
+        __builtin_amdgcn_s_barrier();
+      }
+    }
+    if (LOADS) wait_vmcnt<0>();
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) total += acc[a][c][r];
+  } else {
+    f32x4 acc[8][4];
+#pragma unroll
+    for (int a = 0; a < 8; ++a)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) acc[a][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+    u32x4 af[2][8], bf[2][4], raw[4];
+#pragma unroll
+    for (int a = 0; a < 8; ++a) af[0][a] = af[1][a] = *reinterpret_cast<const u32x4*>(base + a * 1024);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) bf[0][c] = bf[1][c] = *reinterpret_cast<const u32x4*>(base + 16384 + c * 1024);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) raw[c] = *reinterpret_cast<const u32x4*>(base + 32768 + c * 1024);
+    for (int it = 0; it < iters; ++it) {
+      const unsigned char* tb = base + ((it & 3) << 14);
+      if (DQ > 0) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) raw[c] = *reinterpret_cast<const u32x4*>(tb + c * 1024 + 8192);
+      }
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        if (NA > 0) {
+#pragma unroll
+          for (int a = 0; a < 2 * NA; ++a)
+            af[(st + 1) & 1][a] = *reinterpret_cast<const u32x4*>(tb + ((st * 8 + a) & 7) * 1024);
+        }
+        if (DQ > 0) {
+#pragma unroll
+          for (int c = 0; c < 2 * DQ; ++c) {
+            const uint32_t w4[4] = {raw[c].x, raw[c].y, raw[c].z, raw[c].w};
+            bf[(st + 1) & 1][c] = DequantExact<WOL_DTYPE_BF16, 8>::run(&w4[((st + 1) & 1) * 2]);
+          }
+        }
+#pragma unroll
+        for (int a = 0; a < 8; ++a)
+#pragma unroll
+          for (int c = 0; c < 4; ++c) acc[a][c] = mfma16<WOL_DTYPE_BF16>(af[st & 1][a], bf[st & 1][c], acc[a][c]);
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (i < 2 * NA) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          if (DQ > 0) __builtin_amdgcn_sched_group_barrier(0x002, (14 * 2 * DQ + 31) / 32 + 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (BAR) __builtin_amdgcn_s_barrier();
+    }
+#pragma unroll
+    for (int a = 0; a < 8; ++a)
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) total += acc[a][c][r];
+  }
+  out[static_cast<int64_t>(blockIdx.x) * 512 + tid] = total;
+#endif
+}
+
+template <bool M16, int DQ, int NA, bool BAR, bool LOADS>
+void launch_probe(const void* ops, int wgs, int iters, float* out, hipStream_t s) {
+  auto kern = mfma_probe_kernel<M16, DQ, NA, BAR, LOADS>;
+  static std::atomic<uint32_t> configured{0};
+  const size_t lds = LOADS ? 160 * 1024 : 96 * 1024;  // one workgroup per CU either way
+  allow_lds(reinterpret_cast<const void*>(kern), lds, configured);
+  kern<<<dim3(static_cast<unsigned>(wgs)), dim3(512), lds, s>>>(static_cast<const u32x4*>(ops), iters, out);
+}
+
+}  // namespace
+
+int launch_mfma_probe(int variant, const void* ops, int workgroups, int iters, float* out, hipStream_t stream) {
+  switch (variant) {
+    case 0: launch_probe<false, 0, 0, false, false>(ops, workgroups, iters, out, stream); break;
+    case 1: launch_probe<false, 2, 0, false, false>(ops, workgroups, iters, out, stream); break;
+    case 2: launch_probe<false, 0, 4, false, false>(ops, workgroups, iters, out, stream); break;
+    case 3: launch_probe<false, 2, 4, false, false>(ops, workgroups, iters, out, stream); break;
+    case 4: launch_probe<false, 2, 4, true, false>(ops, workgroups, iters, out, stream); break;
+    case 5: launch_probe<false, 2, 4, true, true>(ops, workgroups, iters, out, stream); break;
+    case 6: launch_probe<false, 0, 0, true, true>(ops, workgroups, iters, out, stream); break;
+    case 7: launch_probe<true, 0, 0, false, false>(ops, workgroups, iters, out, stream); break;
+    case 8: launch_probe<true, 2, 4, true, false>(ops, workgroups, iters, out, stream); break;
+    default: return WOL_ERR_BAD_SHAPE;
+  }
+  return check_launch();
+}
+
 }  // namespace wol

@@ -62,10 +62,16 @@ def linear(x_bits, codes_u8, bias_bits, scale_bits, dt, N, bits, g, f32=False, n
     runs 4) through wol_linear_on;
     ws_bytes overrides the size of the scratch buffer handed in."""
     x = H.bits_to_torch(x_bits, dt, DEV)
-    M, K = x.shape
     c = torch.from_numpy(np.ascontiguousarray(codes_u8)).to(DEV)
     s = H.bits_to_torch(scale_bits, dt, DEV)
     b = None if bias_bits is None else H.bits_to_torch(bias_bits, dt, DEV)
+    out = linear_dev(x, c, b, s, dt, N, bits, g, f32=f32, no_workspace=no_workspace, kernel=kernel, ws_bytes=ws_bytes)
+    return out.cpu().numpy() if f32 else H.torch_to_bits(out)
+
+
+def linear_dev(x, c, b, s, dt, N, bits, g, f32=False, no_workspace=False, kernel=None, ws_bytes=None):
+    """The same on tensors that already live on the device; returns the output tensor."""
+    M, K = x.shape
     out = torch.full((M, N), float("nan"), dtype=torch.float32 if f32 else x.dtype, device=DEV)
     if kernel is None:
         wsb = _lib.lib.wol_linear_workspace(M, K, N, bits, g)
@@ -85,7 +91,7 @@ def linear(x_bits, codes_u8, bias_bits, scale_bits, dt, N, bits, g, f32=False, n
     else:
         _lib.check(_lib.lib.wol_linear_on(*args, 1 if f32 else 0, kernel, *tail))
     torch.cuda.synchronize()
-    return out.cpu().numpy() if f32 else H.torch_to_bits(out)
+    return out
 
 
 def linear_plan(M, K, N, bits, g, ws_bytes):

@@ -234,6 +234,17 @@ def test_read_floor_argument_errors(lib):
     assert f(None, 64, 16, 4, None, None) == 5  # a strip smaller than one piece per wavefront
 
 
+def test_mfma_probe_argument_errors(lib):
+    L = lib.lib
+    p = ctypes.c_void_p(0x1000)
+    need = 64 * 8 * 49152 + 65536
+    assert L.wol_mfma_probe(9, p, need, 1, 1, p, None) == 5 and L.wol_mfma_probe(-1, p, need, 1, 1, p, None) == 5
+    assert L.wol_mfma_probe(0, p, need, 0, 1, p, None) == 5 and L.wol_mfma_probe(0, p, need, 1, 0, p, None) == 5
+    assert L.wol_mfma_probe(0, None, need, 1, 1, p, None) == 1
+    assert L.wol_mfma_probe(0, ctypes.c_void_p(0x1008), need, 1, 1, p, None) == 9
+    assert L.wol_mfma_probe(5, p, need - 1, 1, 1, p, None) == 8  # too few operand bytes for the variants that load
+
+
 def test_linear_plan_names_the_kernel_per_shape(lib):
     # wol_linear's choice between its three kernels, as the library reports it
     # (no device work): one row streams a workgroup per strip; 2 and 5..16 rows

@@ -52,17 +52,13 @@ def test_oracle_swiglu_against_numpy_float64(oracle):
 
 
 # ---- the fused entry point ----------------------------------------------------
-def _fused(x_bits, pre_bits, packed, bias_bits, scale_bits, dt, N, bits, g, act):
+def _fused_dev(x, ps, c, b, s, dt, N, bits, g, act):
+    """wol_linear_fused on device tensors; returns the output tensor."""
     import torch
     from paddle_amd import _lib
 
     dev = "cuda:0"
-    x = H.bits_to_torch(x_bits, dt, dev)
     M, K = x.shape
-    c = torch.from_numpy(np.ascontiguousarray(packed)).to(dev)
-    s = H.bits_to_torch(scale_bits, dt, dev)
-    b = None if bias_bits is None else H.bits_to_torch(bias_bits, dt, dev)
-    ps = None if pre_bits is None else H.bits_to_torch(pre_bits, dt, dev)
     No = N // 2 if act == 2 else N
     out = torch.full((M, No), float("nan"), dtype=x.dtype, device=dev)
     wsb = _lib.lib.wol_linear_fused_workspace(M, K, N, bits, g, 0 if ps is None else 1, act)
@@ -71,7 +67,19 @@ def _fused(x_bits, pre_bits, packed, bias_bits, scale_bits, dt, N, bits, g, act)
                                          None if b is None else b.data_ptr(), s.data_ptr(), dt, M, K, N, bits, g, act,
                                          out.data_ptr(), ws.data_ptr() if wsb else None, wsb, None))
     torch.cuda.synchronize()
-    return H.torch_to_bits(out)
+    return out
+
+
+def _fused(x_bits, pre_bits, packed, bias_bits, scale_bits, dt, N, bits, g, act):
+    import torch
+
+    dev = "cuda:0"
+    x = H.bits_to_torch(x_bits, dt, dev)
+    c = torch.from_numpy(np.ascontiguousarray(packed)).to(dev)
+    s = H.bits_to_torch(scale_bits, dt, dev)
+    b = None if bias_bits is None else H.bits_to_torch(bias_bits, dt, dev)
+    ps = None if pre_bits is None else H.bits_to_torch(pre_bits, dt, dev)
+    return H.torch_to_bits(_fused_dev(x, ps, c, b, s, dt, N, bits, g, act))
 
 
 # rows x (K, N): one row (streaming kernel), a small batch on a K and N the
@@ -86,15 +94,34 @@ SHAPES = [(1, 512, 256), (1, 4096, 1024), (8, 2048, 12288), (5, 4096, 10272), (3
 @pytest.mark.parametrize("bits", [8, 4])
 @pytest.mark.parametrize("g", [-1, 64, 128])
 def test_fused_against_oracle(device, oracle, dt, bits, g):
+    import torch
+    from paddle_amd.nn import quant as Q
+
     rng = np.random.default_rng(11)
     for M, K, N in SHAPES:
-        wb = H.make_weight(K, N, dt, seed=K + N)
         xb = H.make_act(M, K, dt, seed=M)
         bb = H.make_bias(N, dt, seed=5)
         pre = H.f32_to_bits((0.5 + rng.random(K, dtype=np.float32)).astype(np.float32), dt)
-        oc, osc = oracle.weight_quantize(wb, dt, bits, g)
-        packed = H.gfx950_from_q(H.q_from_canonical(oc, bits), bits)
         big = K * N > 1e7  # the large shapes take a subset that still has every activation, pre-scale and bias
+        if big:
+            # weight made and quantised on the device (its quantiser has its own
+            # bit-exact tests); the oracle quantises and multiplies column slices
+            gen = torch.Generator(device="cuda").manual_seed(K + N)
+            w = (torch.randn(K, N, device="cuda", generator=gen) * 0.02).to(H.torch_dtype(dt))
+            codes, scale = Q.weight_quantize(w, algo="weight_only_int8" if bits == 8 else "weight_only_int4",
+                                             group_size=g)
+            x_d, b_d, p_d = (H.bits_to_torch(v, dt, "cuda:0") for v in (xb, bb, pre))
+            slices = {}
+            for c0 in (0, (N // 4) // 32 * 32, N // 2 - 32):
+                for pair in (False, True):  # swiglu needs a gate slice and the up slice that goes with it
+                    cols = np.r_[c0:c0 + 32, N // 2 + c0:N // 2 + c0 + 32] if pair else np.r_[c0:c0 + 64]
+                    oc, osc = oracle.weight_quantize(H.torch_to_bits(w[:, cols].contiguous()), dt, bits, g)
+                    assert np.array_equal(osc, H.torch_to_bits(scale[..., cols].contiguous()))
+                    slices[(c0, pair)] = (cols, oc, osc)
+        else:
+            wb = H.make_weight(K, N, dt, seed=K + N)
+            oc, osc = oracle.weight_quantize(wb, dt, bits, g)
+            packed = H.gfx950_from_q(H.q_from_canonical(oc, bits), bits)
         for act in (0, 1, 2):
             for use_pre in (False, True):
                 for bias in (None, bb):
@@ -105,10 +132,23 @@ def test_fused_against_oracle(device, oracle, dt, bits, g):
                                                                         (2, False, True)):
                         continue
                     print("case", dt, bits, g, M, K, N, act, use_pre, bias is not None, flush=True)
-                    _, wantT = oracle.linear_fused(xb, pre if use_pre else None, oc, osc, bias, dt, bits, g, act)
-                    got = _fused(xb, pre if use_pre else None, packed, bias, osc, dt, N, bits, g, act)
-                    err = H.rel_l2(H.bits_to_f32(got, dt), H.bits_to_f32(wantT, dt))
-                    assert err <= TOL, (err, dt, bits, g, M, K, N, act, use_pre)
+                    if not big:
+                        _, wantT = oracle.linear_fused(xb, pre if use_pre else None, oc, osc, bias, dt, bits, g, act)
+                        got = _fused(xb, pre if use_pre else None, packed, bias, osc, dt, N, bits, g, act)
+                        err = H.rel_l2(H.bits_to_f32(got, dt), H.bits_to_f32(wantT, dt))
+                        assert err <= TOL, (err, dt, bits, g, M, K, N, act, use_pre)
+                        continue
+                    got = _fused_dev(x_d, p_d if use_pre else None, codes, None if bias is None else b_d, scale, dt, N,
+                                     bits, g, act)
+                    assert bool(torch.isfinite(got.float()).all())
+                    for (c0, pair), (cols, soc, sosc) in slices.items():
+                        if pair != (act == 2):
+                            continue
+                        _, wantT = oracle.linear_fused(xb, pre if use_pre else None, soc, sosc,
+                                                       None if bias is None else bias[cols], dt, bits, g, act)
+                        part = got[:, c0:c0 + (32 if act == 2 else 64)].contiguous()
+                        err = H.rel_l2(H.bits_to_f32(H.torch_to_bits(part), dt), H.bits_to_f32(wantT, dt))
+                        assert err <= TOL, (err, dt, bits, g, M, K, N, act, use_pre, c0)
 
 
 @pytest.mark.gpu
