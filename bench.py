@@ -533,6 +533,7 @@ def main():
     # weight copy from HBM once; what overlaps is one call's launch and drain
     # with another's stream.
     n_par = 4
+    par_steps = max(args.steps, 400)  # the fork and join of a replay cost as much as several calls: many calls per replay
     par_streams = [torch.cuda.Stream(device=dev) for _ in range(n_par - 1)]
     par_x = [x.clone() for _ in range(n_par)]
 
@@ -547,16 +548,16 @@ def main():
         fork.record(cur)
         for s in par_streams:
             s.wait_event(fork)
-        for i in range(args.steps):
+        for i in range(par_steps):
             par_call(i, cur if i % n_par == 0 else par_streams[i % n_par - 1])
         for s in par_streams:
             e = torch.cuda.Event()
             e.record(s)
             cur.wait_event(e)
 
-    par_med, par_min = time_graph(torch, decode_step, args.steps, warm_launches=max(400, args.warmup),
+    par_med, par_min = time_graph(torch, decode_step, par_steps, warm_launches=max(400, args.warmup),
                                   eager=args.eager, whole=par_whole)
-    par_s = par_med / args.steps
+    par_s = par_med / par_steps
 
     # ---------------- prefill ----------------
     p = PREFILL
@@ -744,6 +745,7 @@ def main():
             "decode_4_in_flight_gbs": round(wbytes / par_s / 1e9, 1),
             "decode_4_in_flight_frac": round(wbytes / par_s / 1e9 / HBM_PEAK_GBS, 4),
             "decode_4_in_flight_ms_per_step": round(par_s * 1e3, 6),
+            "decode_4_in_flight_steps_per_replay": par_steps,
             "read_floor": {
                 "what": "wol_read_floor: the same weight copies read by a kernel of the same launch shape "
                         "that computes nothing (no scales, activations, MFMAs or output)",

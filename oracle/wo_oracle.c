@@ -488,6 +488,40 @@ void wo_linear_grad(const uint16_t* out_grad, const int8_t* codes,
   free(g); free(wdq);
 }
 
+/* The reference's own composition of the same gradient
+ * (paddle/phi/kernels/gpu/weight_only_linear_grad_kernel.cu:52-69): the
+ * dequantised weight is written out in T (weight_dequantize, :52-60), i.e.
+ * every code * scale is rounded to T, and that tensor goes through a library
+ * GEMM with fp32 accumulation.  Same arguments as wo_linear_grad; the only
+ * difference is the rounding of the weight.  It is what the kernel's distance
+ * to the reference is measured against (tests/test_linear_grad.py). */
+void wo_linear_grad_rounded_weight(const uint16_t* out_grad, const int8_t* codes,
+                                   const uint16_t* scale, int64_t M, int64_t K, int64_t N,
+                                   int dtype, int bits, int64_t group_size, int nibble_bias,
+                                   int acc64, float* out32, uint16_t* outT) {
+  uint16_t* wT = (uint16_t*)malloc((size_t)K * (size_t)N * sizeof(uint16_t));
+  wo_dequantize(codes, scale, K, N, dtype, bits, group_size, nibble_bias,
+                WO_CAST_RNE, NULL, wT);
+  float* g = (float*)malloc((size_t)N * sizeof(float));
+  for (int64_t m = 0; m < M; ++m) {
+    for (int64_t n = 0; n < N; ++n) g[n] = wo_to_f32(out_grad[m * N + n], dtype);
+    for (int64_t k = 0; k < K; ++k) {
+      const uint16_t* wr = wT + k * N;
+      double a = 0.0;
+      float af = 0.0f;
+      for (int64_t n = 0; n < N; ++n) {
+        const float w = wo_to_f32(wr[n], dtype);
+        if (acc64) a += (double)g[n] * (double)w;
+        else af += g[n] * w;
+      }
+      const float v = acc64 ? (float)a : af;
+      out32[m * K + k] = v;
+      if (outT) outT[m * K + k] = wo_from_f32(v, dtype, WO_CAST_RNE);
+    }
+  }
+  free(g); free(wT);
+}
+
 /* ---- pre-quant activation smoothing ------------------------------------ */
 
 /* out[r,c] = T(x[r,c] * scales[c]): ApplyPerChannelScaleKernel

@@ -72,6 +72,9 @@ def lib():
         L.wo_linear_grad.argtypes = [_u16p, _i8p, _u16p, _i64, _i64, _i64, _int, _int, _i64, _int, _int, _f32p,
                                      ctypes.c_void_p]
         L.wo_linear_grad.restype = None
+        L.wo_linear_grad_rounded_weight.argtypes = [_u16p, _i8p, _u16p, _i64, _i64, _i64, _int, _int, _i64, _int, _int, _f32p,
+                                     ctypes.c_void_p]
+        L.wo_linear_grad_rounded_weight.restype = None
         _lib = L
     return _lib
 
@@ -235,6 +238,22 @@ def linear_grad(out_grad_bits, codes, scale, dtype, bits, group_size=-1, acc64=F
     outT = np.empty((M, K), np.uint16)
     lib().wo_linear_grad(g, codes, scale, M, K, N, dtype, bits, group_size, 0, 1 if acc64 else 0, out32,
                          outT.ctypes.data)
+    return out32, outT
+
+
+def linear_grad_rounded_weight(out_grad_bits, codes, scale, dtype, bits, group_size=-1, acc64=False):
+    """The reference's composition of the same gradient: the dequantised weight
+    rounded to T (weight_dequantize), then the product with fp32 sums.  Returns
+    (fp32, T-bits)."""
+    g = np.ascontiguousarray(out_grad_bits, dtype=np.uint16)
+    codes = np.ascontiguousarray(codes, dtype=np.int8)
+    scale = np.ascontiguousarray(scale, dtype=np.uint16)
+    M, N = g.shape
+    K = codes.shape[0]
+    out32 = np.empty((M, K), np.float32)
+    outT = np.empty((M, K), np.uint16)
+    lib().wo_linear_grad_rounded_weight(g, codes, scale, M, K, N, dtype, bits, group_size, 0, 1 if acc64 else 0,
+                                        out32, outT.ctypes.data)
     return out32, outT
 
 

@@ -31,6 +31,25 @@ def test_oracle_linear_grad_against_float64_matmul(oracle, dt, bits, g):
     assert np.array_equal(oT, H.f32_to_bits(o32, dt))
 
 
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+def test_oracle_reference_composition_of_the_gradient(oracle, dt):
+    # the reference dequantises to T and multiplies that tensor: pinned against
+    # numpy in float64 on the oracle's T-rounded dequantised weight (itself
+    # bit-exact against the reference's formula elsewhere)
+    M, K, N, bits, g = 4, 192, 80, 8, 64
+    wb = H.make_weight(K, N, dt, seed=5)
+    oc, osc = oracle.weight_quantize(wb, dt, bits, g)
+    _, wT = oracle.dequantize(oc, osc, dt, bits, g)
+    gb = H.make_act(M, N, dt, seed=6)
+    want = H.bits_to_f32(gb, dt).astype(np.float64) @ H.bits_to_f32(wT, dt).astype(np.float64).T
+    o64, _ = oracle.linear_grad_rounded_weight(gb, oc, osc, dt, bits, g, acc64=True)
+    assert np.array_equal(o64, want.astype(np.float32))
+    # it differs from the fp32-weight contract by one rounding of every weight to T
+    exact, _ = oracle.linear_grad(gb, oc, osc, dt, bits, g, acc64=True)
+    d = H.rel_l2(o64, exact)
+    assert (5e-4 < d < 4e-3) if dt == H.BF16 else (5e-5 < d < 5e-4), d
+
+
 def test_oracle_linear_grad_is_the_adjoint_of_linear(oracle):
     # <linear(x), g> == <x, linear_grad(g)> for any x and g: fixes the pairing of
     # the two functions' index conventions independently of the dequantiser
@@ -114,6 +133,33 @@ def test_linear_grad_against_oracle(device, oracle, dt, bits, g):
         assert err32 <= 3e-4, (err32, dt, bits, g, M, K, N)
         if dt == H.F16 or M * K >= 4096:
             assert errT <= TOL, (errT, dt, bits, g, M, K, N)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+@pytest.mark.parametrize("bits", [8, 4])
+def test_linear_grad_distance_to_the_reference_composition(device, oracle, dt, bits):
+    # The reference rounds code * scale to T before its GEMM; this kernel rounds
+    # it to 11 bits (fp16 operands for both dtypes).  Its fp32 sums are therefore
+    # not the reference's bits: recorded here is how far they are from the
+    # reference's composition (one T rounding of the weights: about 2e-3 for
+    # bfloat16, 2e-4 for float16) and that they are nearer to the exact product
+    # than that composition is for bfloat16.
+    M, K, N, g = 96, 512, 384, -1
+    wb = H.make_weight(K, N, dt, seed=21)
+    oc, osc = oracle.weight_quantize(wb, dt, bits, g)
+    packed = H.gfx950_from_q(H.q_from_canonical(oc, bits), bits)
+    gb = H.make_act(M, N, dt, seed=22)
+    exact, _ = oracle.linear_grad(gb, oc, osc, dt, bits, g)
+    ref, _ = oracle.linear_grad_rounded_weight(gb, oc, osc, dt, bits, g)
+    got32 = _grad(gb, packed, osc, dt, K, bits, g, f32=True)
+    to_ref, to_exact, ref_to_exact = H.rel_l2(got32, ref), H.rel_l2(got32, exact), H.rel_l2(ref, exact)
+    print("distance to the reference composition %.2e, to the exact product %.2e (the composition's own %.2e)"
+          % (to_ref, to_exact, ref_to_exact))
+    assert to_ref <= (4e-3 if dt == H.BF16 else 6e-4), to_ref
+    assert to_exact <= 3e-4
+    if dt == H.BF16:
+        assert to_exact < ref_to_exact
 
 
 @pytest.mark.gpu
