@@ -220,10 +220,12 @@ int wol_linear_f32(const void* x, const void* codes, const void* bias,
  *   v  = x' . dequant(W) + bias      fp32 accumulation, as wol_linear
  *   out = T(act(v))                  act applied to the fp32 sum, one rounding
  * pre_scale: [K] T.  out: [M, N] T, or [M, N/2] T for WOL_ACT_SWIGLU.
- * The decode kernels apply pre_scale while they load the activations and the
- * activation in their epilogues; the MFMA GEMM applies gelu in its epilogue
- * and takes pre-scaled activations and swiglu through the workspace (one
- * element-wise pass each, inside this call).  The workspace is therefore
+ * The decode kernels (up to 16 rows) apply pre_scale while they load the
+ * activations and gelu or swiglu in their epilogues (with K cut into runs: in
+ * the kernel that adds the runs); the MFMA GEMM applies gelu in its epilogue,
+ * swiglu too with per-channel scales above 64 rows, and takes pre-scaled
+ * activations -- and the swiglu of its other forms -- through the workspace
+ * (one element-wise pass each, inside this call).  The workspace is therefore
  * required whenever wol_linear_fused_workspace() is non-zero.
  */
 size_t wol_linear_fused_workspace(int64_t M, int64_t K, int64_t N, int bits,

@@ -222,6 +222,15 @@ struct Range {
   bool on;
 };
 
+// Whether kernel `which` forms the swiglu of a gate|up projection in its own epilogue.
+bool kernel_fuses_swiglu(int which, int64_t M, int64_t K, int64_t N, int bits, int group_size) {
+  if (which == WOL_KERNEL_GEMM) return wol::linear_gemm_fuses_swiglu(M, K, N, bits, group_size);
+  if (which == WOL_KERNEL_STREAM) return wol::linear_stream_fuses_swiglu(M, N);
+  if (which == WOL_KERNEL_BATCH) return wol::linear_batch_fuses_swiglu(K, N, bits);
+  if (which == WOL_KERNEL_BATCH_SPLIT) return N % 32 == 0;  // in the kernel that adds the runs
+  return false;
+}
+
 int linear_impl(const void* x, const void* codes, const void* bias, const void* scale, int dtype,
                 int64_t M, int64_t K, int64_t N, int bits, int group_size, void* out, bool out_f32,
                 int kernel, void* workspace, size_t workspace_bytes, void* stream,
@@ -250,7 +259,7 @@ int linear_impl(const void* x, const void* codes, const void* bias, const void* 
   int which = resolve_kernel(kernel, M, K, N, bits, group_size, workspace_bytes);
   if (which == WOL_KERNEL_BATCH_SPLIT && kernel == WOL_KERNEL_AUTO && fuse.pre_scale != nullptr)
     which = resolve_kernel(kernel, M, K, N, bits, group_size, 0);  // that kernel applies no pre-scale
-  if (fuse.act == WOL_ACT_SWIGLU && which != WOL_KERNEL_GEMM) return WOL_ERR_BAD_SHAPE;  // only the GEMM's epilogue forms it
+  if (fuse.act == WOL_ACT_SWIGLU && !kernel_fuses_swiglu(which, M, K, N, bits, group_size)) return WOL_ERR_BAD_SHAPE;
   if (log_enabled())
     fprintf(stderr, "[wol] linear M=%lld K=%lld N=%lld int%d group=%d %s%s%s act=%d -> %s kernel\n",
             static_cast<long long>(M), static_cast<long long>(K), static_cast<long long>(N), bits, group_size,
@@ -408,9 +417,10 @@ FusedPlan plan_fused(int64_t M, int64_t K, int64_t N, int bits, int group_size, 
   const bool fused_pre = (which == WOL_KERNEL_BATCH && wol::linear_batch_fuses_pre_scale(K, bits, group_size)) ||
                          (which == WOL_KERNEL_STREAM && M == 1);
   f.prepass = has_pre && !fused_pre;
-  // the GEMM's large tiles form the swiglu in their epilogue; elsewhere it is a pass over fp32 sums
-  f.swiglu_pass = act == WOL_ACT_SWIGLU &&
-                  !(which == WOL_KERNEL_GEMM && wol::linear_gemm_fuses_swiglu(M, K, N, bits, group_size));
+  // the decode kernels and the GEMM's large tiles form the swiglu in their epilogue; elsewhere it is a pass over fp32 sums
+  // (the batched kernel applies activation scales or forms the swiglu, not both)
+  f.swiglu_pass = act == WOL_ACT_SWIGLU && !(kernel_fuses_swiglu(which, M, K, N, bits, group_size) &&
+                                             !(which == WOL_KERNEL_BATCH && has_pre && fused_pre));
   auto up = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
   f.linear_ws = lws;
   f.x_off = up(lws);
@@ -445,7 +455,8 @@ int wol_linear_fused(const void* x, const void* pre_scale, const void* codes, co
     return WOL_ERR_ALIGNMENT;
   if (pre_scale != nullptr && !aligned16(pre_scale)) return WOL_ERR_ALIGNMENT;
   const FusedPlan f = plan_fused(M, K, N, bits, group_size, pre_scale != nullptr, act);
-  if (f.prepass || f.swiglu_pass) {
+  // (a swiglu formed inside the kernel: the kernel must be the one the plan was made for, scratch included)
+  if (f.prepass || f.swiglu_pass || (act == WOL_ACT_SWIGLU && f.total > 0)) {
     if (workspace == nullptr || workspace_bytes < f.total) return WOL_ERR_WORKSPACE;
     if (!aligned16(workspace)) return WOL_ERR_ALIGNMENT;
   }

@@ -273,7 +273,8 @@ int launch_linear_stream(const void* x, const void* codes, const void* bias, con
 bool linear_batch_supports(int64_t M, int64_t K, int bits, int group_size);
 bool linear_batch_fuses_pre_scale(int64_t K, int bits, int group_size);
 int linear_batch_cus();  // CUs of the current device (256 when it cannot be asked)
-void plan_linear_batch(int64_t K, int64_t N, int bits, int* grid, int* tpw);
+void plan_linear_batch(int64_t K, int64_t N, int bits, int* grid, int* tpw, bool swi = false);
+bool linear_batch_fuses_swiglu(int64_t K, int64_t N, int bits);
 int launch_linear_batch(const void* x, const void* codes, const void* bias, const void* scale,
                         int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
                         void* out, bool out_f32, hipStream_t stream, const Fuse& f = Fuse());
@@ -289,7 +290,9 @@ int launch_linear_batch_split(const void* x, const void* codes, const void* bias
                               const Fuse& f = Fuse());
 void describe_linear_batch_split(int64_t M, int64_t K, int64_t N, int bits, int group_size, char* buf, size_t n);
 // out[m, n] = T(act(sum over the runs of part[run][m][n] + bias[n])): the second
-// kernel of every K-split launch (wol_linear_gemm.hip).  N % 4 == 0.
+// kernel of every K-split launch (wol_linear_gemm.hip).  N % 4 == 0.  act may also be
+// WOL_ACT_SWIGLU (N % 8 == 0): out is then [M, N/2], silu of the first half of a row's sums
+// times the second half.
 int launch_reduce_partials(const float* part, int nsplit, const void* bias, int dtype, void* out,
                            bool out_f32, int64_t M, int64_t N, int act, hipStream_t stream);
 // One-line descriptions of what the launchers would run for a problem.
@@ -332,6 +335,7 @@ void llm_int8_workspace_offsets(int64_t M, int64_t K, int64_t N, int64_t* offset
 // Scratch bytes with which launch_linear_gemm splits K across workgroups (0: none needed).
 size_t linear_gemm_workspace(int64_t M, int64_t K, int64_t N, int bits, int group_size);
 bool linear_gemm_fuses_swiglu(int64_t M, int64_t K, int64_t N, int bits, int group_size);
+bool linear_stream_fuses_swiglu(int64_t M, int64_t N);
 
 inline int check_launch() {
   return hipGetLastError() == hipSuccess ? WOL_OK : WOL_ERR_HIP;

@@ -80,7 +80,7 @@ struct BatchParams {
   int M, K, N;
   int gshift;   // log2(group size), -1 per-channel
   int out_f32;
-  int strips_q, strips_r;  // strips per workgroup: N / 16 = grid * strips_q + strips_r
+  int strips_q, strips_r;  // strips (SWI: pairs of strips) per workgroup: N / 16 = grid * strips_q + strips_r
   const uint16_t* pre;     // [K] per-channel scales of the activations, or null
   int act;                 // WOL_ACT_NONE or WOL_ACT_GELU
   // K cut into runs across workgroups (SPLIT): workgroup b takes run b % nseg
@@ -107,7 +107,12 @@ struct BatchParams {
 // kernel adds the runs (bias and activation function there).  This is what
 // serves any K made of whole tiles, and what keeps x down to K / nseg per CU
 // when the strips are few.
-template <int DT, int BITS, int G, int TPW, int IT, int D, bool PRE, int MT, bool SPLIT>
+// SWI: the weight is a gate|up projection and the kernel writes
+// silu(gate) * up, [M, N/2].  The unit of work is then a pair of strips, gate
+// strip u and up strip u + N/32: a workgroup owns a contiguous range of pairs,
+// a run holds up to three of them with the strips in the order gate, up, gate,
+// up ..., and the end of a run combines the two sums of every output element.
+template <int DT, int BITS, int G, int TPW, int IT, int D, bool PRE, int MT, bool SPLIT, bool SWI>
 __global__ __launch_bounds__(kBatchWaves * 64) void batch_kernel(const BatchParams p) {
   constexpr int WK = kBatchWaves;
   constexpr int TK = BITS == 8 ? 64 : 128;   // k per 1 KiB weight tile
@@ -122,6 +127,8 @@ __global__ __launch_bounds__(kBatchWaves * 64) void batch_kernel(const BatchPara
   constexpr bool kKeepCancel = MT * TPW * SPT <= 8 && MT * TPW * CPT <= 4;  // cancelling terms computed once and kept
                                                                          // where 32 registers of A leave 16 for them
   static_assert(!(PRE && (SPLIT || MT > 1)), "the fused activation scales exist for the one-run, 16-row form");
+  static_assert(!(SWI && (SPLIT || MT > 1 || PRE)), "the gate|up form exists for the one-run, 16-row form without activation scales");
+  constexpr int SPU = SWI ? 2 : 1;  // strips per unit of the workgroup's range
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
   const int lane = threadIdx.x & 63;
@@ -208,31 +215,45 @@ __global__ __launch_bounds__(kBatchWaves * 64) void batch_kernel(const BatchPara
   const __amdgpu_buffer_rsrc_t bias_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<uint16_t*>(p.bias != nullptr ? p.bias : p.scale), 0, N * 2, 0x00020000);
 
-  constexpr int kRun = kBatchRun / MT;  // strips whose partial sums share the LDS
+  constexpr int kRun = kBatchRun / MT / SPU;  // units (strips, or pairs of them) whose partial sums share the LDS
+  const int up0 = N / kStripCols / 2;         // SWI: the first up strip
   for (int sr = s0; sr < s1; sr += kRun) {
-    const int cnt = s1 - sr < kRun ? s1 - sr : kRun;  // strips of this run
-    const int nitems = cnt * P;  // item it: strip sr + it / P, part it % P
+    const int cnt = s1 - sr < kRun ? s1 - sr : kRun;  // units of this run
+    const int nstr = cnt * SPU;                       // strips of this run
+    const int nitems = nstr * P;  // item it: strip it / P of the run, part it % P
 
-    const int ncols = cnt * kStripCols;
-    float* red = reinterpret_cast<float*>(smem);                               // [cnt][WK][MT * 4][64]
-    uint16_t* lsc = reinterpret_cast<uint16_t*>(smem + cnt * WK * MT * 1024);  // [ncols] per-channel scales
+    const int ncols = nstr * kStripCols;
+    float* red = reinterpret_cast<float*>(smem);                                // [nstr][WK][MT * 4][64]
+    uint16_t* lsc = reinterpret_cast<uint16_t*>(smem + nstr * WK * MT * 1024);  // [ncols] per-channel scales
     uint16_t* lbi = lsc + ncols;                                          // [ncols] bias
+    // strip sl of the run is strip run_strip(sl) of the weight
+    auto run_strip = [&](int sl) { return SWI ? sr + (sl >> 1) + (sl & 1) * up0 : sr + sl; };
 
     // What the end of the run needs -- per-channel scales and bias of its
     // columns -- is requested first (one load each by the first threads; the
     // others read past the end of the descriptor: nothing) and parked in LDS
     // once the weight ring has been requested as well.
-    const int boff = static_cast<int>(threadIdx.x) < ncols ? (sr * kStripCols + static_cast<int>(threadIdx.x)) * 2 : 0x7FFFFFF0;
+    int boff = static_cast<int>(threadIdx.x) < ncols ? (sr * kStripCols + static_cast<int>(threadIdx.x)) * 2 : 0x7FFFFFF0;
+    if constexpr (SWI) {
+      if (static_cast<int>(threadIdx.x) < ncols)
+        boff = (run_strip(static_cast<int>(threadIdx.x) / kStripCols) * kStripCols +
+                static_cast<int>(threadIdx.x) % kStripCols) * 2;
+    }
     const uint16_t sstage = __builtin_amdgcn_raw_buffer_load_b16(scale_rsrc, boff, 0, 0);
     const uint16_t bstage = __builtin_amdgcn_raw_buffer_load_b16(bias_rsrc, boff, 0, 0);
 
     // fill the ring; slots past the last item load nothing
+    // (SWI: from the run's first gate strip to its last up strip, half the
+    // weight further on: the host keeps that below 2 GiB)
     const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint8_t*>(p.codes + sr * sbytes), 0, cnt * static_cast<int>(sbytes), 0x00020000);
+        const_cast<uint8_t*>(p.codes + sr * sbytes), 0, ((SWI ? up0 : 0) + cnt) * static_cast<int>(sbytes), 0x00020000);
 #pragma unroll
     for (int d = 0; d < D; ++d) {
-      const int sl = d / P < cnt ? d / P : cnt - 1;
-      load_item(wrsrc, sr + sl, d / P, d % P, d < nitems, W[d], S[d]);
+      const int sl = d / P < nstr ? d / P : nstr - 1;
+      if constexpr (SWI)
+        load_item(wrsrc, run_strip(sl), (sl >> 1) + (sl & 1) * up0, d % P, d < nitems, W[d], S[d]);
+      else
+        load_item(wrsrc, sr + sl, d / P, d % P, d < nitems, W[d], S[d]);
     }
 
     // the staged values have arrived before the ring (they were requested first)
@@ -322,15 +343,53 @@ __global__ __launch_bounds__(kBatchWaves * 64) void batch_kernel(const BatchPara
           }
         }
         // the slot is free: refill it with the item D places further on (if there is one)
-        const int nsl = (it + D) / P < cnt ? (it + D) / P : cnt - 1;
-        load_item(wrsrc, sr + nsl, (it + D) / P, part, it + D < nitems, W[d], S[d]);
+        const int nsl = (it + D) / P < nstr ? (it + D) / P : nstr - 1;
+        if constexpr (SWI)
+          load_item(wrsrc, run_strip(nsl), (nsl >> 1) + (nsl & 1) * up0, part, it + D < nitems, W[d], S[d]);
+        else
+          load_item(wrsrc, sr + nsl, (it + D) / P, part, it + D < nitems, W[d], S[d]);
       }
     }
 
     // ---- the run is done: partial sums of the 16 wavefronts meet in LDS ----
     __syncthreads();
+    if constexpr (SWI) {
+      // (the ring's registers are named before the sums here, see the end of the run: they are free for the epilogue)
 #pragma unroll
-    for (int q = 0; q < 2; ++q) {
+      for (int d = 0; d < D; ++d) {
+#pragma unroll
+        for (int i = 0; i < IT; ++i) asm volatile("" ::"v"(W[d][i]));
+#pragma unroll
+        for (int q = 0; q < NS; ++q) asm volatile("" ::"v"(S[d][q]));
+      }
+      const int e = threadIdx.x;  // at most 3 pairs x 256 elements
+      if (e < cnt * 256) {
+        // e = (pair of the run * 4 + r) * 64 + lane of the MFMA result
+        const int u = e >> 8, rr = (e >> 6) & 3, l = e & 63;
+        const int m = 4 * (l >> 4) + rr;
+        if (m < M) {
+          float v[2];
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            float s = 0.0f;
+#pragma unroll
+            for (int w = 0; w < WK; ++w) s += red[(((2 * u + h) * WK + w) * 4 + rr) * 64 + l];
+            const int cl = (2 * u + h) * kStripCols + (l & 15);
+            const float ep_scale = G == 0 ? to_f32<DT>(lsc[cl]) : 1.0f;
+            const float ep_bias = p.bias != nullptr ? to_f32<DT>(lbi[cl]) : 0.0f;
+            v[h] = s * ep_scale + ep_bias;
+          }
+          const float s = act_swiglu(v[0], v[1]);
+          const int64_t o = static_cast<int64_t>(m) * (N / 2) + (sr + u) * kStripCols + (l & 15);
+          if (p.out_f32)
+            static_cast<float*>(p.out)[o] = s;
+          else
+            static_cast<uint16_t*>(p.out)[o] = cast_out<DT>(s);
+        }
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < (SWI ? 0 : 2); ++q) {
       const int e = threadIdx.x + q * WK * 64;
       if (e < cnt * MT * 256) {
         // e = ((strip of the run * MT + mt) * 4 + r) * 64 + lane of the MFMA result
@@ -360,12 +419,14 @@ __global__ __launch_bounds__(kBatchWaves * 64) void batch_kernel(const BatchPara
     // nothing) are then known to have completed here, and the next run starts
     // with a load queue whose content the compiler knows exactly -- otherwise
     // the first loads of a run would wait for older ones they do not depend on.
+    if constexpr (!SWI) {
 #pragma unroll
-    for (int d = 0; d < D; ++d) {
+      for (int d = 0; d < D; ++d) {
 #pragma unroll
-      for (int i = 0; i < IT; ++i) asm volatile("" ::"v"(W[d][i]));
+        for (int i = 0; i < IT; ++i) asm volatile("" ::"v"(W[d][i]));
 #pragma unroll
-      for (int q = 0; q < NS; ++q) asm volatile("" ::"v"(S[d][q]));
+        for (int q = 0; q < NS; ++q) asm volatile("" ::"v"(S[d][q]));
+      }
     }
     if (sr + kRun < s1) __syncthreads();  // the next run overwrites the partial sums
   }
@@ -376,6 +437,7 @@ struct Args {
   int M, K, N, gshift, out_f32; hipStream_t stream;
   const void* pre; int act;
   int nseg; float* ws;  // K runs across workgroups and where their sums go (nseg = 1: none)
+  bool swi = false;     // gate|up projection: write silu(gate) * up (the one-run form)
 };
 
 inline int num_cus() {
@@ -401,18 +463,21 @@ inline void allow_lds(const void* kern, size_t lds, std::atomic<uint32_t>& done)
 
 // LDS of a launch: partial sums, scales and bias of the longest run of strips.
 // sets: strip sets (workgroups, or workgroups / K runs); mt: 16-row operands.
-inline size_t batch_lds(int64_t N, int sets, int mt) {
-  const int64_t nstrips = N / kStripCols;
-  int64_t per_wg = (nstrips + sets - 1) / sets;
-  if (per_wg > kBatchRun / mt) per_wg = kBatchRun / mt;
+// swi: the sets are sets of strip pairs.
+inline size_t batch_lds(int64_t N, int sets, int mt, bool swi = false) {
+  const int spu = swi ? 2 : 1;
+  const int64_t units = N / kStripCols / spu;
+  int64_t per_wg = (units + sets - 1) / sets;
+  if (per_wg > kBatchRun / mt / spu) per_wg = kBatchRun / mt / spu;
+  per_wg *= spu;  // strips
   return static_cast<size_t>(per_wg * kBatchWaves * mt * 1024 + 2 * per_wg * kStripCols * 2);
 }
 
 // grid: strip sets; with SPLIT every set is worked on by a.nseg workgroups
-template <int DT, int BITS, int G, int TPW, int IT, int D, bool PRE, int MT = 1, bool SPLIT = false>
+template <int DT, int BITS, int G, int TPW, int IT, int D, bool PRE, int MT = 1, bool SPLIT = false, bool SWI = false>
 void launch_pre(const Args& a, int grid) {
-  const size_t lds = batch_lds(a.N, grid, MT);
-  auto kern = batch_kernel<DT, BITS, G, TPW, IT, D, PRE, MT, SPLIT>;
+  const size_t lds = batch_lds(a.N, grid, MT, SWI);
+  auto kern = batch_kernel<DT, BITS, G, TPW, IT, D, PRE, MT, SPLIT, SWI>;
   static std::atomic<uint32_t> configured{0};  // per instantiation
   allow_lds(reinterpret_cast<const void*>(kern), 160 * 1024, configured);
   BatchParams p;
@@ -424,8 +489,8 @@ void launch_pre(const Args& a, int grid) {
   p.M = a.M; p.K = a.K; p.N = a.N;
   p.gshift = a.gshift;
   p.out_f32 = a.out_f32;
-  p.strips_q = a.N / kStripCols / grid;
-  p.strips_r = a.N / kStripCols % grid;
+  p.strips_q = a.N / kStripCols / (SWI ? 2 : 1) / grid;
+  p.strips_r = a.N / kStripCols / (SWI ? 2 : 1) % grid;
   p.pre = PRE ? static_cast<const uint16_t*>(a.pre) : nullptr;
   p.act = a.act;
   p.nseg = SPLIT ? a.nseg : 1;
@@ -444,12 +509,13 @@ constexpr bool pre_fits(int bits, int group, int k_steps_per_wave) {
 template <int DT, int BITS, int G, int TPW, int IT, int D>
 void launch_one(const Args& a, int grid) {
   if constexpr (pre_fits(BITS, G, TPW * (BITS == 8 ? 2 : 4))) {
-    if (a.pre != nullptr) {
+    if (a.pre != nullptr) {  // (never together with the gate|up form: launch_linear_batch refuses)
       launch_pre<DT, BITS, G, TPW, IT, D, true>(a, grid);
       return;
     }
   }
-  launch_pre<DT, BITS, G, TPW, IT, D, false>(a, grid);
+  if (a.swi) launch_pre<DT, BITS, G, TPW, IT, D, false, 1, false, true>(a, grid);
+  else launch_pre<DT, BITS, G, TPW, IT, D, false>(a, grid);
 }
 
 // tpw = K / (16 * tile depth): 1, 2 or 4.  Items and ring depths by what the
@@ -519,6 +585,13 @@ bool linear_batch_supports(int64_t M, int64_t K, int bits, int group_size) {
 
 int linear_batch_cus() { return num_cus(); }
 
+// The one-run form writes silu(gate) * up of a gate|up projection itself when
+// the halves are whole strips and a run's gate and up strips lie within 2 GiB
+// of each other (no activation scales in the same call).
+bool linear_batch_fuses_swiglu(int64_t K, int64_t N, int bits) {
+  return N % (2 * kStripCols) == 0 && (N / kStripCols / 2 + kBatchRun) * strip_bytes(K, bits) < (int64_t{1} << 31);
+}
+
 // Whether launch_linear_batch applies a Fuse::pre_scale itself for this K.
 bool linear_batch_fuses_pre_scale(int64_t K, int bits, int group_size) {
   return pre_fits(bits, group_size > 0 ? group_size : 0, static_cast<int>(K / 32 / kBatchWaves));
@@ -526,8 +599,9 @@ bool linear_batch_fuses_pre_scale(int64_t K, int bits, int group_size) {
 
 // Grid (workgroups: one per CU, fewer when there are fewer strips) and the
 // weight tiles of a strip per wavefront.
-void plan_linear_batch(int64_t K, int64_t N, int bits, int* grid, int* tpw) {
-  const int64_t nstrips = N / kStripCols;
+// swi: the unit a workgroup owns is a pair of strips.
+void plan_linear_batch(int64_t K, int64_t N, int bits, int* grid, int* tpw, bool swi) {
+  const int64_t nstrips = N / kStripCols / (swi ? 2 : 1);
   const int cus = num_cus();
   *grid = static_cast<int>(nstrips < cus ? nstrips : cus);
   *tpw = static_cast<int>(K / (bits == 8 ? 64 : 128) / kBatchWaves);
@@ -538,10 +612,13 @@ int launch_linear_batch(const void* x, const void* codes, const void* bias, cons
                         void* out, bool out_f32, hipStream_t stream, const Fuse& f) {
   const int gshift = group_size == 64 ? 6 : (group_size == 128 ? 7 : -1);
   int grid = 1, tpw = 1;
-  plan_linear_batch(K, N, bits, &grid, &tpw);
+  const bool swi = f.act == WOL_ACT_SWIGLU;
+  if (swi && (!linear_batch_fuses_swiglu(K, N, bits) || f.pre_scale != nullptr)) return WOL_ERR_BAD_SHAPE;
+  plan_linear_batch(K, N, bits, &grid, &tpw, swi);
   const Args a{x, codes, bias, scale, out, static_cast<int>(M), static_cast<int>(K),
                static_cast<int>(N), gshift, out_f32 ? 1 : 0, stream,
-               linear_batch_fuses_pre_scale(K, bits, group_size) ? f.pre_scale : nullptr, f.act, 1, nullptr};
+               linear_batch_fuses_pre_scale(K, bits, group_size) ? f.pre_scale : nullptr,
+               swi ? WOL_ACT_NONE : f.act, 1, nullptr, swi};
   if (dtype == WOL_DTYPE_BF16) {
     if (bits == 8) launch_g<WOL_DTYPE_BF16, 8>(a, grid, tpw); else launch_g<WOL_DTYPE_BF16, 4>(a, grid, tpw);
   } else {

@@ -968,6 +968,56 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(
   }
 }
 
+// The same for a gate|up projection: out[m, c] = T(silu(g) * u) with g and u the sums (plus bias)
+// of columns c and N/2 + c; out is [M, N/2], four columns per thread, total = M * N / 2,
+// N % 8 == 0.  The runs are [run][M][N].
+template <int DT>
+__global__ __launch_bounds__(256) void reduce_partials_swiglu_kernel(
+    const float* __restrict__ part, int nsplit, const uint16_t* __restrict__ bias,
+    void* __restrict__ out, int out_f32, int64_t total, int N) {
+  const int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
+  if (i >= total) return;
+  const int half = N / 2;
+  const int64_t m = i / half;
+  const int c = static_cast<int>(i % half);
+  const int64_t run = total * 2;
+  f32x4 s[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+  for (int r0 = 0; r0 < nsplit; r0 += 4) {
+    f32x4 v[4][2];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int r = r0 + u < nsplit ? r0 + u : nsplit - 1;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) v[u][h] = *reinterpret_cast<const f32x4*>(part + r * run + m * N + h * half + c);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (r0 + u < nsplit) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) s[h][e] += v[u][h][e];
+      }
+  }
+  if (bias != nullptr) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s[h][e] += to_f32<DT>(bias[h * half + c + e]);
+  }
+  f32x4 o;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) o[e] = act_swiglu(s[0][e], s[1][e]);
+  if (out_f32) {
+    *reinterpret_cast<f32x4*>(static_cast<float*>(out) + i) = o;
+  } else {
+    u32x2 v;
+    v.x = cast_out<DT>(o[0]) | (static_cast<uint32_t>(cast_out<DT>(o[1])) << 16);
+    v.y = cast_out<DT>(o[2]) | (static_cast<uint32_t>(cast_out<DT>(o[3])) << 16);
+    *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(out) + i) = v;
+  }
+}
+
 struct Args {
   const void* x; const void* codes; const void* bias; const void* scale; void* out;
   int M, K, N, gshift, out_f32;
@@ -1454,6 +1504,18 @@ void launch_cfg(const Args& a) {
 
 int launch_reduce_partials(const float* part, int nsplit, const void* bias, int dtype, void* out,
                            bool out_f32, int64_t M, int64_t N, int act, hipStream_t stream) {
+  if (act == WOL_ACT_SWIGLU) {  // out is [M, N/2]
+    if (N % 8 != 0) return WOL_ERR_BAD_SHAPE;
+    const int64_t total = M * N / 2;
+    const dim3 grid(static_cast<unsigned>((total / 4 + 255) / 256)), block(256);
+    if (dtype == WOL_DTYPE_BF16)
+      reduce_partials_swiglu_kernel<WOL_DTYPE_BF16><<<grid, block, 0, stream>>>(
+          part, nsplit, static_cast<const uint16_t*>(bias), out, out_f32 ? 1 : 0, total, static_cast<int>(N));
+    else
+      reduce_partials_swiglu_kernel<WOL_DTYPE_F16><<<grid, block, 0, stream>>>(
+          part, nsplit, static_cast<const uint16_t*>(bias), out, out_f32 ? 1 : 0, total, static_cast<int>(N));
+    return check_launch();
+  }
   const int64_t total = M * N;
   const dim3 grid(static_cast<unsigned>((total / 4 + 255) / 256)), block(256);
   if (dtype == WOL_DTYPE_BF16)

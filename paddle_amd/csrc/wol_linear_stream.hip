@@ -72,9 +72,17 @@ __device__ inline float sum_lane_groups(float v, bool x16, bool x32) {
 // way into the A operand, each product rounded to T as
 // apply_per_channel_scale rounds it (built for one row only; other row counts
 // get the scaled activations from a pass of that kernel).
-template <int DT, int BITS, int MP, int MT, int WK, int NU, int TN, bool GROUPED, bool PRE>
+//
+// SWI: the weight is a gate|up projection and the kernel writes
+// silu(gate) * up, [M, N/2].  The first half of the workgroup's wavefronts
+// works on gate strip b, the second half on up strip b + N/32, each half
+// splitting K as a whole workgroup does otherwise; the two sums of an output
+// element meet in the epilogue, which is the only place that differs.
+template <int DT, int BITS, int MP, int MT, int WK, int NU, int TN, bool GROUPED, bool PRE, bool SWI>
 struct StreamKernel {
   static_assert(MT == 1 || MP == 16, "several M tiles only with full 16-row operands");
+  static_assert(!SWI || (TN == 1 && MT == 1 && WK >= 2), "the gate|up form pairs two single strips");
+  static constexpr int kWS = SWI ? WK / 2 : WK;       // wavefronts that share a strip
   static constexpr int kS = 16 / MP;                  // k steps sharing one A operand
   static constexpr int kSPT = BITS == 8 ? 2 : 4;      // k steps per 16-byte weight tile
   static constexpr int kDw = BITS == 8 ? 2 : 1;       // dwords per k step
@@ -295,7 +303,8 @@ struct StreamKernel {
   __device__ inline void run(const uint8_t* codes, const uint16_t* bias, void* out, int out_f32,
                              float* red) {
     lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wave_all = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wave = SWI ? wave_all % kWS : wave_all;  // its place among the wavefronts of its strip
     j = lane & 15;
     kb = lane >> 4;
     const int nstrips = N / kStripCols;
@@ -303,6 +312,7 @@ struct StreamKernel {
 #pragma unroll
     for (int t = 0; t < TN; ++t) {
       int tn = blockIdx.x * TN + t;
+      if (SWI) tn += (wave_all / kWS) * (nstrips / 2);  // the up strip of the same output columns
       tn = tn < nstrips ? tn : nstrips - 1;  // a strip past the end repeats the last one and is not stored
       n[t] = tn * kStripCols + j;
       strip[t] = codes + static_cast<int64_t>(tn) * strip_bytes(K, BITS);
@@ -322,14 +332,18 @@ struct StreamKernel {
     // what the epilogue needs from memory, requested before the long loads:
     // thread t always stores column t % 16 of the strip
     // (raw bits; they are converted where they are used, after the long loads)
-    uint16_t ep_sraw[TN], ep_braw[TN];
+    // (SWI: the gate column's and, in slot 1, the up column's)
+    constexpr int kEp = SWI ? 2 : TN;
+    uint16_t ep_sraw[kEp], ep_braw[kEp];
     const u32x4* tp[TN];
 #pragma unroll
-    for (int t = 0; t < TN; ++t) {
-      ep_sraw[t] = scale[n[t]];
-      ep_braw[t] = (bias != nullptr ? bias : scale)[n[t]];  // one unconditional load
-      tp[t] = reinterpret_cast<const u32x4*>(strip[t]) + lane;
+    for (int t = 0; t < kEp; ++t) {
+      const int col = SWI ? static_cast<int>(blockIdx.x) * kStripCols + j + t * (N / 2) : n[t];
+      ep_sraw[t] = scale[col];
+      ep_braw[t] = (bias != nullptr ? bias : scale)[col];  // one unconditional load
     }
+#pragma unroll
+    for (int t = 0; t < TN; ++t) tp[t] = reinterpret_cast<const u32x4*>(strip[t]) + lane;
     if (NU > 0) {
       Unit d[NU > 0 ? NU : 1];
 #pragma unroll
@@ -338,7 +352,7 @@ struct StreamKernel {
 #pragma unroll
       for (int i = 0; i < NU; ++i) compute_unit(d[i]);
     } else {
-      const int u0 = nunits * wave / WK, u1 = nunits * (wave + 1) / WK;
+      const int u0 = nunits * wave / kWS, u1 = nunits * (wave + 1) / kWS;
       // the partial unit that ends K goes to wavefront 0 (the floor split
       // gives it the fewest whole units), ahead of its walk
       const bool tail = kPartial && wave == 0 && nunits * kU < vsteps;
@@ -413,7 +427,7 @@ struct StreamKernel {
     // naming them here keeps the compiler from sinking those loads (and the
     // reads of the kernel arguments) into the tail of the kernel.
 #pragma unroll
-    for (int t = 0; t < TN; ++t) asm volatile("" ::"v"(ep_sraw[t]), "v"(ep_braw[t]));
+    for (int t = 0; t < kEp; ++t) asm volatile("" ::"v"(ep_sraw[t]), "v"(ep_braw[t]));
     asm volatile("" ::"s"(out), "s"(out_f32));
 
 #pragma unroll
@@ -449,10 +463,36 @@ struct StreamKernel {
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int r = 0; r < kLive; ++r)
-          red[(((t * WK + wave) * MT + mt) * 4 + r) * 64 + lane] = tot[mt][r];
+          red[(((t * WK + wave_all) * MT + mt) * 4 + r) * 64 + lane] = tot[mt][r];
     }
     __syncthreads();
     const int rows = M < 16 * MT ? M : 16 * MT;
+    if (SWI) {
+      float ep_scale[2], ep_bias[2];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        ep_scale[h] = GROUPED ? 1.0f : to_f32<DT>(ep_sraw[h]);
+        ep_bias[h] = bias != nullptr ? to_f32<DT>(ep_braw[h]) : 0.0f;
+      }
+      for (int idx = threadIdx.x; idx < rows * 16; idx += WK * 64) {
+        const int m = idx / 16, nl = idx % 16;  // nl == j
+        float v[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          float s = 0.0f;
+#pragma unroll
+          for (int w = 0; w < kWS; ++w) s += red[((h * kWS + w) * 4 + (m % 4)) * 64 + (m / 4) * 16 + nl];
+          v[h] = s * ep_scale[h] + ep_bias[h];
+        }
+        const float s = act_swiglu(v[0], v[1]);
+        const int64_t o = static_cast<int64_t>(m) * (N / 2) + static_cast<int>(blockIdx.x) * kStripCols + nl;
+        if (out_f32)
+          static_cast<float*>(out)[o] = s;
+        else
+          static_cast<uint16_t*>(out)[o] = cast_out<DT>(s);
+      }
+      return;
+    }
 #pragma unroll
     for (int t = 0; t < TN; ++t) {
       if (static_cast<int>(blockIdx.x) * TN + t >= nstrips) break;  // the repeated last strip
@@ -476,13 +516,13 @@ struct StreamKernel {
   }
 };
 
-template <int DT, int BITS, int MP, int MT, int WK, int NU, int TN, bool GROUPED, bool PRE>
+template <int DT, int BITS, int MP, int MT, int WK, int NU, int TN, bool GROUPED, bool PRE, bool SWI>
 __global__ __launch_bounds__(WK * 64) void stream_kernel(
     const uint16_t* __restrict__ x, const uint8_t* __restrict__ codes,
     const uint16_t* __restrict__ bias, const uint16_t* __restrict__ scale, void* __restrict__ out,
     int M, int K, int N, int gshift, int out_f32, const uint16_t* __restrict__ pre, int act) {
   extern __shared__ float red[];
-  StreamKernel<DT, BITS, MP, MT, WK, NU, TN, GROUPED, PRE> k;
+  StreamKernel<DT, BITS, MP, MT, WK, NU, TN, GROUPED, PRE, SWI> k;
   k.x = x;
   k.scale = scale;
   k.pre = pre;
@@ -497,13 +537,13 @@ __global__ __launch_bounds__(WK * 64) void stream_kernel(
 struct Args {
   const void* x; const void* codes; const void* bias; const void* scale; void* out;
   int M, K, N, gshift, out_f32, tn; hipStream_t stream;
-  const void* pre; int act;
+  const void* pre; int act;  // act: none or gelu; the gate|up form is a template argument
 };
 
-template <int DT, int BITS, int MP, int MT, int WK, int NU, int TN>
+template <int DT, int BITS, int MP, int MT, int WK, int NU, int TN, bool SWI = false>
 void launch_tn(const Args& a) {
   const size_t lds = static_cast<size_t>(TN) * WK * MT * 256 * sizeof(float);
-  const dim3 grid(static_cast<unsigned>((a.N / kStripCols + TN - 1) / TN)), block(WK * 64);
+  const dim3 grid(static_cast<unsigned>(SWI ? a.N / kStripCols / 2 : (a.N / kStripCols + TN - 1) / TN)), block(WK * 64);
   const uint16_t* x = static_cast<const uint16_t*>(a.x);
   const uint8_t* codes = static_cast<const uint8_t*>(a.codes);
   const uint16_t* bias = static_cast<const uint16_t*>(a.bias);
@@ -512,19 +552,19 @@ void launch_tn(const Args& a) {
   if constexpr (MP == 1) {  // the fused activation scales exist for one row
     if (pre != nullptr) {
       if (a.gshift >= 0)
-        stream_kernel<DT, BITS, MP, MT, WK, NU, TN, true, true><<<grid, block, lds, a.stream>>>(
+        stream_kernel<DT, BITS, MP, MT, WK, NU, TN, true, true, SWI><<<grid, block, lds, a.stream>>>(
             x, codes, bias, scale, a.out, a.M, a.K, a.N, a.gshift, a.out_f32, pre, a.act);
       else
-        stream_kernel<DT, BITS, MP, MT, WK, NU, TN, false, true><<<grid, block, lds, a.stream>>>(
+        stream_kernel<DT, BITS, MP, MT, WK, NU, TN, false, true, SWI><<<grid, block, lds, a.stream>>>(
             x, codes, bias, scale, a.out, a.M, a.K, a.N, a.gshift, a.out_f32, pre, a.act);
       return;
     }
   }
   if (a.gshift >= 0)
-    stream_kernel<DT, BITS, MP, MT, WK, NU, TN, true, false><<<grid, block, lds, a.stream>>>(
+    stream_kernel<DT, BITS, MP, MT, WK, NU, TN, true, false, SWI><<<grid, block, lds, a.stream>>>(
         x, codes, bias, scale, a.out, a.M, a.K, a.N, a.gshift, a.out_f32, nullptr, a.act);
   else
-    stream_kernel<DT, BITS, MP, MT, WK, NU, TN, false, false><<<grid, block, lds, a.stream>>>(
+    stream_kernel<DT, BITS, MP, MT, WK, NU, TN, false, false, SWI><<<grid, block, lds, a.stream>>>(
         x, codes, bias, scale, a.out, a.M, a.K, a.N, a.gshift, a.out_f32, nullptr, a.act);
 }
 
@@ -568,6 +608,37 @@ void launch_wk(const Args& a, int wk, int nu) {
     else if (wk >= 2) launch_one<DT, BITS, MP, MT, 2, 0>(a);
     else launch_one<DT, BITS, MP, MT, 1, 0>(a);
   }
+}
+
+// The gate|up form: `total` wavefronts per workgroup, half of them per strip.
+template <int DT, int BITS, int MP>
+void launch_wk_swi(const Args& a, int total, int nu) {
+  if constexpr (MP == 4 || MP == 8) {
+    if (nu == 2) { launch_tn<DT, BITS, MP, 1, 16, 2, 1, true>(a); return; }
+    if (nu == 4) { launch_tn<DT, BITS, MP, 1, 16, 4, 1, true>(a); return; }
+  }
+  if (nu == 1) {
+    if (total >= 16) launch_tn<DT, BITS, MP, 1, 16, 1, 1, true>(a);
+    else if (total >= 8) launch_tn<DT, BITS, MP, 1, 8, 1, 1, true>(a);
+    else if (total >= 4) launch_tn<DT, BITS, MP, 1, 4, 1, 1, true>(a);
+    else launch_tn<DT, BITS, MP, 1, 2, 1, 1, true>(a);
+  } else {
+    if constexpr ((MP >= 2 && MP <= 8) || (MP == 1 && BITS == 4)) {
+      if (total >= 16) { launch_tn<DT, BITS, MP, 1, 16, 0, 1, true>(a); return; }
+    }
+    if (total >= 8) launch_tn<DT, BITS, MP, 1, 8, 0, 1, true>(a);
+    else if (total >= 4) launch_tn<DT, BITS, MP, 1, 4, 0, 1, true>(a);
+    else launch_tn<DT, BITS, MP, 1, 2, 0, 1, true>(a);
+  }
+}
+
+template <int DT, int BITS>
+void launch_m_swi(const Args& a, int total, int nu) {
+  if (a.M <= 1) launch_wk_swi<DT, BITS, 1>(a, total, nu);
+  else if (a.M <= 2) launch_wk_swi<DT, BITS, 2>(a, total, nu);
+  else if (a.M <= 4) launch_wk_swi<DT, BITS, 4>(a, total, nu);
+  else if (a.M <= 8) launch_wk_swi<DT, BITS, 8>(a, total, nu);
+  else launch_wk_swi<DT, BITS, 16>(a, total, nu);
 }
 
 template <int DT, int BITS>
@@ -637,16 +708,41 @@ void describe_linear_stream(int64_t M, int64_t K, int64_t N, int bits, int group
   (void)group_size;
 }
 
+// Up to 16 rows of a gate|up projection (N a multiple of 32) leave the kernel as
+// silu(gate) * up.
+bool linear_stream_fuses_swiglu(int64_t M, int64_t N) { return M >= 1 && M <= 16 && N % 32 == 0; }
+
 // f.pre_scale is honoured for one row only (the caller scales the activations
-// itself otherwise); f.act may be none or gelu.
+// itself otherwise); f.act may be none, gelu or -- where
+// linear_stream_fuses_swiglu says so -- swiglu (out is then [M, N/2]).
 int launch_linear_stream(const void* x, const void* codes, const void* bias, const void* scale,
                          int dtype, int64_t M, int64_t K, int64_t N, int bits, int group_size,
                          void* out, bool out_f32, hipStream_t stream, const Fuse& f) {
   const int gshift = group_size == 64 ? 6 : (group_size == 128 ? 7 : -1);
   int wk = 1, nu = 0, tn = 1;
   pick_split(M, K, N, bits, &wk, &nu, &tn);
+  const bool swi = f.act == WOL_ACT_SWIGLU;
+  if (swi && !linear_stream_fuses_swiglu(M, N)) return WOL_ERR_BAD_SHAPE;
   const Args a{x, codes, bias, scale, out, static_cast<int>(M), static_cast<int>(K),
-               static_cast<int>(N), gshift, out_f32 ? 1 : 0, tn, stream, M == 1 ? f.pre_scale : nullptr, f.act};
+               static_cast<int>(N), gshift, out_f32 ? 1 : 0, tn, stream, M == 1 ? f.pre_scale : nullptr,
+               swi ? WOL_ACT_NONE : f.act};
+  if (swi) {
+    // the split of one strip, twice in a workgroup; where that is more
+    // wavefronts than a workgroup holds, the halves walk their units instead
+    int mp = 1;
+    while (mp < 16 && mp < M) mp *= 2;
+    const int walk_max = (mp >= 2 && mp <= 8) || (mp == 1 && bits == 4) ? 16 : 8;
+    int total = 2 * wk;
+    if (nu == 1 && total > 16) nu = 0;
+    if (nu == 2 || nu == 4) total = 16;
+    if (nu == 0 && total > walk_max) total = walk_max;
+    if (dtype == WOL_DTYPE_BF16) {
+      if (bits == 8) launch_m_swi<WOL_DTYPE_BF16, 8>(a, total, nu); else launch_m_swi<WOL_DTYPE_BF16, 4>(a, total, nu);
+    } else {
+      if (bits == 8) launch_m_swi<WOL_DTYPE_F16, 8>(a, total, nu); else launch_m_swi<WOL_DTYPE_F16, 4>(a, total, nu);
+    }
+    return check_launch();
+  }
   if (dtype == WOL_DTYPE_BF16) {
     if (bits == 8) launch_m<WOL_DTYPE_BF16, 8>(a, wk, nu); else launch_m<WOL_DTYPE_BF16, 4>(a, wk, nu);
   } else {

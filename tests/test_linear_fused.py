@@ -179,6 +179,93 @@ def test_swiglu_in_the_gemm_epilogue(device, oracle, dt, bits):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dt", [H.F16, H.BF16])
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("g", [-1, 128])
+def test_swiglu_in_the_streaming_kernel(device, oracle, dt, bits, g):
+    # up to 16 rows the streaming kernel gives half of a workgroup's wavefronts
+    # the gate strip and the other half the up strip and writes [M, N/2] itself.
+    # Shapes: every operand height (1, 2, 4, 8, 16 rows), K whose units go one,
+    # two or four to a wavefront at once, K that a wavefront walks (8192, and
+    # 11008 / 1088 with their partial last unit and int4 half tile), one pair
+    # of strips and many; K = 512 ... 1088 keep the batched kernel out at
+    # several rows
+    import ctypes
+
+    from paddle_amd import _lib
+
+    rng = np.random.default_rng(3)
+    for M, K, N in ((1, 512, 32), (1, 4096, 1024), (1, 8192, 256), (1, 11008, 64), (2, 1024, 96), (3, 512, 256),
+                    (4, 1088, 64), (5, 1024, 160), (8, 512, 64), (9, 1024, 96), (16, 1088, 128)):
+        lws = _lib.lib.wol_linear_workspace(M, K, N, bits, g)
+        plan = ctypes.create_string_buffer(256)
+        _lib.check(_lib.lib.wol_linear_plan(M, K, N, bits, g, lws, plan, 256))
+        if b"stream_kernel" in plan.value:  # (16 rows of int8 at K = 1088 go to the batched kernel and the pass)
+            assert _lib.lib.wol_linear_fused_workspace(M, K, N, bits, g, 0, 2) == lws
+        wb = H.make_weight(K, N, dt, seed=K + N + M)
+        xb = H.make_act(M, K, dt, seed=M)
+        bb = H.make_bias(N, dt, seed=6)
+        pre = H.f32_to_bits((0.5 + rng.random(K, dtype=np.float32)).astype(np.float32), dt)
+        oc, osc = oracle.weight_quantize(wb, dt, bits, g)
+        packed = H.gfx950_from_q(H.q_from_canonical(oc, bits), bits)
+        for bias, use_pre in ((None, False), (bb, False), (bb, M == 1)):
+            print("case", dt, bits, g, M, K, N, bias is not None, use_pre, flush=True)
+            _, wantT = oracle.linear_fused(xb, pre if use_pre else None, oc, osc, bias, dt, bits, g, 2)
+            got = _fused(xb, pre if use_pre else None, packed, bias, osc, dt, N, bits, g, 2)
+            assert got.shape == (M, N // 2)
+            err = H.rel_l2(H.bits_to_f32(got, dt), H.bits_to_f32(wantT, dt))
+            assert err <= TOL, (err, dt, bits, g, M, K, N, bias is not None, use_pre)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("g", [-1, 64, 128])
+def test_swiglu_in_the_batched_kernel(device, oracle, dt, bits, g):
+    # 2 to 16 rows at K = 2048, 4096 (and 8192 for int4) on weights wide enough
+    # for the batched kernel (2.5 strips per CU and more): a workgroup owns a
+    # range of strip pairs (gate strip, up strip) and combines them at the end
+    # of every run of three pairs.  Workgroups with one or two pairs, with three
+    # or four (a second run of one pair), with a remainder.  The weights are made
+    # and quantised on the device; the oracle checks column slices
+    import ctypes
+
+    import torch
+    from paddle_amd import _lib
+    from paddle_amd.nn import quant as Q
+
+    shapes = [(2, 2048, 28704), (7, 4096, 10272), (16, 4096, 28704)]
+    if bits == 4 and g != 64:
+        shapes.append((9, 8192, 12320))
+    for M, K, N in shapes:
+        lws = _lib.lib.wol_linear_workspace(M, K, N, bits, g)
+        plan = ctypes.create_string_buffer(256)
+        _lib.check(_lib.lib.wol_linear_plan(M, K, N, bits, g, lws, plan, 256))
+        assert b"batch_kernel" in plan.value and b"reduce" not in plan.value, plan.value
+        assert _lib.lib.wol_linear_fused_workspace(M, K, N, bits, g, 0, 2) == lws
+        xb = H.make_act(M, K, dt, seed=M)
+        bb = H.make_bias(N, dt, seed=6)
+        gen = torch.Generator(device="cuda").manual_seed(K + N)
+        w = (torch.randn(K, N, device="cuda", generator=gen) * 0.02).to(H.torch_dtype(dt))
+        codes, scale = Q.weight_quantize(w, algo="weight_only_int8" if bits == 8 else "weight_only_int4", group_size=g)
+        x_d, b_d = (H.bits_to_torch(v, dt, "cuda:0") for v in (xb, bb))
+        for bias in (None, bb):
+            print("case", dt, bits, g, M, K, N, bias is not None, flush=True)
+            got = _fused_dev(x_d, None, codes, None if bias is None else b_d, scale, dt, N, bits, g, 2)
+            assert got.shape == (M, N // 2) and bool(torch.isfinite(got.float()).all())
+            # the first workgroup's pairs (the fourth is a run of its own where it has four), pairs in the
+            # middle and at the end of the range
+            for c0 in (0, 16, 3 * 16, 4 * 16, (N // 4) // 16 * 16, N // 2 - 48, N // 2 - 16):
+                cols = np.r_[c0:c0 + 16, N // 2 + c0:N // 2 + c0 + 16]
+                oc, osc = oracle.weight_quantize(H.torch_to_bits(w[:, cols].contiguous()), dt, bits, g)
+                assert np.array_equal(osc, H.torch_to_bits(scale[..., cols].contiguous()))
+                _, wantT = oracle.linear_fused(xb, None, oc, osc, None if bias is None else bias[cols], dt, bits, g, 2)
+                part = got[:, c0:c0 + 16].contiguous()
+                err = H.rel_l2(H.bits_to_f32(H.torch_to_bits(part), dt), H.bits_to_f32(wantT, dt))
+                assert err <= TOL, (err, dt, bits, g, M, K, N, c0, bias is not None)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
 def test_fused_pre_scale_equals_the_two_ops(device, oracle, dt):
     # folding apply_per_channel_scale into the linear must not change a bit:
     # the same products, rounded the same way, enter the same kernel
@@ -206,17 +293,21 @@ def test_fused_pre_scale_equals_the_two_ops(device, oracle, dt):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("act,use_pre", [(1, False), (2, True)])
+@pytest.mark.parametrize("act,use_pre", [(1, False), (2, False), (2, True)])
 def test_fused_on_the_batched_kernel_with_k_runs(device, oracle, act, use_pre):
     # 24 rows on a 25 MB int8 weight: wol_linear takes the batched kernel with K
-    # runs, so gelu and bias are applied by the kernel that adds the runs, swiglu
-    # by its pass over the fp32 sums, the pre-scale by a pass in front
+    # runs, so bias, gelu and swiglu are applied by the kernel that adds the
+    # runs; with activation scales the call takes another kernel (here the
+    # GEMM, whose group-wise form leaves the swiglu to a pass over fp32 sums)
+    # and the pre-scale is a pass in front
     from paddle_amd import _lib
     import ctypes
 
     dt, bits, g, M, K, N = H.BF16, 8, 64, 24, 2048, 12288
     buf = ctypes.create_string_buffer(512)
     assert _lib.lib.wol_linear_plan(M, K, N, bits, g, 1 << 30, buf, 512) == 0 and b"K runs" in buf.value
+    if not use_pre:  # nothing but the linear's own scratch: no extra pass
+        assert _lib.lib.wol_linear_fused_workspace(M, K, N, bits, g, 0, act) == _lib.lib.wol_linear_workspace(M, K, N, bits, g)
     rng = np.random.default_rng(13)
     wb = H.make_weight(K, N, dt, seed=3)
     xb = H.make_act(M, K, dt, seed=4)
