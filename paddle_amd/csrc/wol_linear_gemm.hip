@@ -462,7 +462,19 @@ struct MoeTile {
 // accumulators and only [M, N/2] leaves the kernel.  SWI = 1 applies it to the
 // fp32 sums (wol_linear_fused); SWI = 2 first rounds both sums to T, as a
 // separate fc1 output would have been (the mixture-of-experts FFN).
-template <int DT, int BITS, int G, int OFFS, int WM, int WN, int TM, int TN, int STAGES, int SWI = 0>
+//
+// RESC (group-wise scales): one set of accumulators instead of two.  The
+// running sums are kept in units of the current group's scale: where a group
+// starts they are multiplied by (previous unit / new unit) and the group's
+// MFMAs then accumulate straight into them; the epilogue multiplies by the last
+// unit.  Every rescaling rounds the sums once (2^-24 relative, a few dozen
+// times per output element), code * scale is still never rounded to T, and
+// the registers of the second accumulator set are free for the largest tile.
+// The unit of a column follows its group scale but never falls more than 2^64
+// below the largest scale the column has had so far (a group that small
+// weighs nothing next to the others in fp32), so the sums cannot overflow
+// however the scales of a column differ.
+template <int DT, int BITS, int G, int OFFS, int WM, int WN, int TM, int TN, int STAGES, int SWI = 0, bool RESC = false>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   constexpr int NW = WM * WN;
@@ -495,6 +507,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
                 "the slice that holds the barrier neither starts nor ends a group");
   static_assert(SWI == 0 || (TN == 2 && G == 0), "the swiglu epilogue pairs the two blocks of a wavefront");
   static_assert(OFFS != 2 || G == 0, "row sums by dot products are taken out once, in the epilogue");
+  static_assert(!RESC || (G != 0 && OFFS == 0), "rescaled sums are for group-wise scales and the exact dequantisers");
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
   const uint16_t* __restrict__ x = p.x;
@@ -630,7 +643,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   };
 
   f32x16 tot[TM][TN];
-  f32x16 part[G != 0 ? TM : 1][G != 0 ? TN : 1];
+  f32x16 part[G != 0 && !RESC ? TM : 1][G != 0 && !RESC ? TN : 1];
+  float unit[TN], mrun[TN];  // RESC: what one unit of this lane's sums of block c is worth; the largest scale so far
+#pragma unroll
+  for (int c = 0; c < TN; ++c) unit[c] = mrun[c] = 0.0f;
   f32x16 canc[OFFS == 1 ? TM : 1];
   float rsum[OFFS == 2 ? TM : 1];  // this lane's share of the sum of the activations of row r32 of block a
 #pragma unroll
@@ -652,6 +668,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   const int a_row_off = (wm * TM * 32 + r32) * (TK * 2);
   const int b_off = kABytes + (wn * TN * 2 + sp) * 1024 + (j + 16 * b) * 16;
   constexpr int kValuPerMfma = ((OFFS == 2 ? 4 * TN + 4 * TM : (BITS == 8 ? 16 : 12) * TN) + TM * TN - 1) / (TM * TN) + 2;
+  constexpr int kValuRescale = RESC ? 16 : 0;  // more per MFMA in the slice that starts a group
   constexpr int kHalf = (TM * TN + 1) / 2;  // MFMAs of a slice issued before the barrier
 
   // The wavefront's pipeline registers: raw codes of the current and the next
@@ -686,11 +703,28 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
     }
   };
   // MFMAs lo .. hi-1 (numbered a * TN + c) of slice q
-  auto mfmas = [&](const u32x4 (&a4)[TM], const u32x4 (&b4)[TN], int q, int lo, int hi) {
-    const bool first = q % kFold == 0;
+  // gstart: the tile starts a group (a group of 128 spans two int8 tiles: the second one of a pair does not)
+  auto mfmas = [&](const u32x4 (&a4)[TM], const u32x4 (&b4)[TN], int q, int lo, int hi, bool gstart = true) {
+    const bool first = q % kFold == 0 && (!RESC || gstart);
     f32x16 zero;
 #pragma unroll
     for (int r = 0; r < 16; ++r) zero[r] = 0.0f;
+    float rho[TN];
+    if (RESC && first) {
+#pragma unroll
+      for (int c = 0; c < TN; ++c) {
+        const float s = to_f32<DT>(sraw[q / kFold][c]);
+        mrun[c] = fmaxf(mrun[c], s);
+        const float u0 = fmaxf(s, mrun[c] * 0x1p-64f);
+        // a scale of zero before any other (or one in the denormal range, which the reciprocal below
+        // does not take): the unit stays what it is
+        const float u = u0 < 0x1p-126f ? unit[c] : u0;
+        // what was summed under a unit of zero (groups whose scale is zero may hold any codes) counts
+        // for nothing; inside a group, and from a group to one of the same scale, nothing changes
+        rho[c] = unit[c] == 0.0f ? 0.0f : (u == unit[c] ? 1.0f : unit[c] * __builtin_amdgcn_rcpf(u));
+        unit[c] = u;
+      }
+    }
 #pragma unroll
     for (int a = 0; a < TM; ++a)
 #pragma unroll
@@ -707,7 +741,12 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
                               Dequant<DT, BITS>::kCancel, Dequant<DT, BITS>::kCancel};
             canc[a] = mfma32<DT>(a4[a], cb, (G != 0 && first) ? zero : canc[a]);
           }
-          if (G == 0) {
+          if (RESC && first) {
+            f32x16 t = tot[a][c];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) t[r] *= rho[c];
+            tot[a][c] = mfma32<DT>(a4[a], b4[c], t);
+          } else if (G == 0 || RESC) {
             tot[a][c] = mfma32<DT>(a4[a], b4[c], tot[a][c]);
           } else if (first) {
             part[a][c] = mfma32<DT>(a4[a], b4[c], zero);
@@ -718,7 +757,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   };
   // after the last slice of a group: tot += part * scale
   auto fold = [&](const uint16_t (&sr)[kGT > 0 ? kGT : 1][TN], int q) {
-    if (G != 0 && q % kFold == kFold - 1) {
+    if (G != 0 && !RESC && q % kFold == kFold - 1) {
 #pragma unroll
       for (int c = 0; c < TN; ++c) {
         const float sc = to_f32<DT>(sr[q / kFold][c]);
@@ -746,7 +785,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   // tile it+3 sits in the middle of the last but one slice, once the
   // wavefront has fetched its last operands of the tile; the raw codes of tile
   // it+1 are read right behind it and have a whole slice to arrive.
-  auto tile = [&](int it, u32x4 (&raw)[TN][2], u32x4 (&raw_next)[TN][2]) {
+  auto tile = [&](auto odd_tile, int it, u32x4 (&raw)[TN][2], u32x4 (&raw_next)[TN][2]) {
+    // RESC with groups of two tiles: the run starts on a group (launch_dma sees to it), so odd tiles continue one
+    constexpr bool gstart = !(RESC && G > TK && decltype(odd_tile)::value);
     const unsigned char* stage = smem + (it % kStages) * kStage;
     const unsigned char* next = smem + ((it + 1) % kStages) * kStage;
     read_scales(stage, sraw);  // before the stage is handed over
@@ -759,7 +800,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
         if (kSpread) issue_range(last ? it + kStages : it + kStages - 1, seg_lo(seg), seg_lo(seg + 1));
         read_a(last ? next : stage, af[(q + 1) & 1], last ? 0 : q + 1);
         dequant(bf[(q + 1) & 1], last ? raw_next : raw, last ? 0 : q + 1);
-        mfmas(af[q & 1], bf[q & 1], q, 0, TM * TN);
+        mfmas(af[q & 1], bf[q & 1], q, 0, TM * TN, gstart);
 #pragma unroll
         for (int i = 0; i < TM * TN; ++i) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                   // one MFMA
@@ -768,7 +809,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
             __builtin_amdgcn_sched_group_barrier(0x004, 2, 0);                 // its LDS address into m0
             __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                 // one tile load
           }
-          __builtin_amdgcn_sched_group_barrier(0x002, kValuPerMfma, 0);        // VALU
+          if (RESC && gstart && q % kFold == 0) __builtin_amdgcn_sched_group_barrier(0x002, kValuPerMfma + kValuRescale, 0);
+          else __builtin_amdgcn_sched_group_barrier(0x002, kValuPerMfma, 0);  // VALU
         }
         __builtin_amdgcn_sched_barrier(0);
         fold(sraw, q);
@@ -806,8 +848,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
     }
   };
   for (int it = 0; it < niter; it += 2) {
-    tile(it, braw[0], braw[1]);
-    if (it + 1 < niter) tile(it + 1, braw[1], braw[0]);
+    tile(std::false_type(), it, braw[0], braw[1]);
+    if (it + 1 < niter) tile(std::true_type(), it + 1, braw[1], braw[0]);
   }
   wait_vmcnt<0>();
   __builtin_amdgcn_s_barrier();  // the spare loads are done and every wavefront has stopped reading
@@ -817,7 +859,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   float sc[TN], bv[TN];
 #pragma unroll
   for (int c = 0; c < TN; ++c) {
-    sc[c] = G == 0 ? to_f32<DT>(scale[ncol[c]]) : 1.0f;
+    sc[c] = RESC ? unit[c] : (G == 0 ? to_f32<DT>(scale[ncol[c]]) : 1.0f);
     bv[c] = (bias != nullptr && p.nsplit == 1) ? to_f32<DT>(bias[ncol[c]]) : 0.0f;
   }
   if (OFFS == 1 && G == 0) {
@@ -1087,13 +1129,13 @@ constexpr size_t dma_lds_bytes() {
 // Launches the fast kernel on the columns of strips [strip_lo, strip_hi), K
 // cut into nsplit runs (nsplit > 1 needs a.ws: nsplit x M x columns floats).
 // SWI != 0 (swiglu epilogue): the strips are those of the gate half, [0, N / 32), a.out is [M, N / 2].
-template <int DT, int BITS, int G, int OFFS, int WM, int WN, int TM, int TN, int STAGES = 3, int SWI = 0>
+template <int DT, int BITS, int G, int OFFS, int WM, int WN, int TM, int TN, int STAGES = 3, int SWI = 0, bool RESC = false>
 void launch_dma(const Args& a, int strip_lo, int strip_hi, int nsplit) {
   constexpr int BM = WM * TM * 32, BN = (SWI ? 1 : TN) * WN * 32, TK = BITS == 8 ? 64 : 128;
   if (strip_hi <= strip_lo) return;
   if (SWI) nsplit = 1;
   constexpr size_t lds = dma_lds_bytes<BITS, G, WM, WN, TM, TN, STAGES>();
-  auto kern = gemm_dma_kernel<DT, BITS, G, OFFS, WM, WN, TM, TN, STAGES, SWI>;
+  auto kern = gemm_dma_kernel<DT, BITS, G, OFFS, WM, WN, TM, TN, STAGES, SWI, RESC>;
   static std::atomic<uint32_t> configured{0};  // per instantiation
   allow_lds(reinterpret_cast<const void*>(kern), lds, configured);
   const int ncols = (strip_hi - strip_lo) * kStripCols;
@@ -1113,6 +1155,7 @@ void launch_dma(const Args& a, int strip_lo, int strip_hi, int nsplit) {
   p.nby = (a.M + BM - 1) / BM;
   const int tiles = a.K / TK;
   p.tiles_per_split = (tiles + nsplit - 1) / nsplit;
+  if (RESC && G > TK) p.tiles_per_split = (p.tiles_per_split + 1) & ~1;  // every run starts on a group of two tiles
   p.nsplit = (tiles + p.tiles_per_split - 1) / p.tiles_per_split;
   p.xcd_rows = plan_xcd_rows(p.nbx, p.nby, BM * 2, WN * TN * 32 * BITS / 8);
   p.act = a.act;
@@ -1220,16 +1263,18 @@ inline SkinnyPlan plan_skinny(int M, int K, int N, int bits, int group, size_t w
 // 256 x 256 tiles (above 64 rows), and the first strip of those columns.
 inline void half_tile_config(int M, int N, int bits, int group, int* bm, int* bn, int* strip_lo) {
   *strip_lo = 0;
-  if (group == 0) {  // per-channel scales: 256 x 256 tiles on whole rounds of the CUs
+  // 256 x 256 tiles on whole rounds of the CUs (int4 with group-wise scales has none:
+  // two stages of its 128-deep tiles and their scales do not fit the LDS)
+  if (group == 0 || bits == 8) {
     const int c = plan_big_columns(M, N, bits == 8) * 16, nstrips = N / kStripCols;
     *strip_lo = c < nstrips ? c : nstrips;
   }
-  if (bits == 8) {
+  if (bits == 8 || group != 0) {
     *bm = tall_half_tile(M) ? 256 : 128;
     *bn = tall_half_tile(M) ? 128 : 256;
   } else {
     *bm = 128;
-    *bn = group == 64 ? 128 : 256;
+    *bn = 256;
   }
 }
 
@@ -1299,26 +1344,27 @@ void launch_fast(const Args& a) {
     if (bm == 256) WOL_HALF(false, 2, 4, 4, 1);
     else WOL_HALF(false, 2, 4, 2, 2);
   } else if constexpr (BITS == 8) {
-    // group-wise scales need a second set of accumulators: half-size tiles
-    if (bm == 256) WOL_HALF(false, 2, 4, 4, 1);
-    else WOL_HALF(false, 2, 4, 2, 2);
-  } else if constexpr (G == 64) {
-    // int4 tiles are 128 k deep; two groups per k tile: two scale sets on top
-    // of two accumulator sets do not fit 256 registers at 128 x 256 (the
-    // spills, being memory loads, also break the in-order accounting of the
-    // tile loads): 128 x 128
-    WOL_HALF(false, 2, 4, 2, 1);
-  } else if constexpr (G == 0 && DT == WOL_DTYPE_BF16) {
+    // group-wise scales: the sums are kept in units of the current group's
+    // scale (RESC), so one set of accumulators serves and the tiles are those
+    // of the per-channel weights
+    launch_dma<DT, BITS, G, 0, 2, 4, 4, 2, 3, 0, true>(a, 0, lo, 1);
+    if (bm == 256) WOL_HALF(0, 2, 4, 4, 1, 3, 0, true);
+    else WOL_HALF(0, 2, 4, 2, 2, 3, 0, true);
+  } else if constexpr (G != 0) {
+    // int4 with group-wise scales: the same, on 256 x 128 tiles where the rows
+    // fill them (four A blocks share every dequantised B block, and the exact
+    // int4 dequantiser is the expensive part), 128 x 256 otherwise
+    if (bm == 256) WOL_HALF(0, 2, 4, 4, 1, 2, 0, true);
+    else WOL_HALF(0, 2, 4, 2, 2, 2, 0, true);
+  } else if constexpr (DT == WOL_DTYPE_BF16) {
     // the exact int4 -> bf16 dequantiser costs 32 VALU instructions per 8
     // codes; the offset form is faster: with row sums by dot products on the
     // 256 x 256 tile (two stages of 64 + 16 KiB fill the LDS), with one
     // cancelling MFMA per A block on the 128 x 256 tiles of the remainder
     launch_dma<DT, BITS, G, 2, 2, 4, 4, 2, 2>(a, 0, lo, 1);
     WOL_HALF(true, 2, 4, 2, 2);
-  } else if constexpr (G == 0) {
-    launch_dma<DT, BITS, G, 0, 2, 4, 4, 2, 2>(a, 0, lo, 1);
-    WOL_HALF(false, 2, 4, 2, 2);
   } else {
+    launch_dma<DT, BITS, G, 0, 2, 4, 4, 2, 2>(a, 0, lo, 1);
     WOL_HALF(false, 2, 4, 2, 2);
   }
 #undef WOL_HALF

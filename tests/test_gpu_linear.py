@@ -622,7 +622,16 @@ def test_weight_larger_than_2_gib(device):
         for i, k in enumerate(ks):
             onehot[i, k] = 1.0
         rows = QL.weight_only_linear_fp32(onehot, codes, None, scale, "int8", 128)
-        assert torch.equal(rows[: len(ks)].to(torch.bfloat16), wdq[ks])
+        if M == 4:
+            assert torch.equal(rows[: len(ks)].to(torch.bfloat16), wdq[ks])
+        else:
+            # the GEMM keeps its sums in units of the current group's scale and
+            # rescales them from group to group (a rounding of 2^-24 each time),
+            # so a row comes back to within a few fp32 ulps of code * scale: half
+            # a bf16 ulp (2^-8 relative at most) from the rounded value, and a little
+            want = wdq[ks].float()
+            assert bool(((rows[: len(ks)] - want).abs() <= want.abs() * (2.0 ** -8 + 1e-5)).all())
+            assert bool((rows[: len(ks)] != 0).eq(want != 0).all())
         assert not rows[len(ks):].any()
 
 
@@ -719,7 +728,7 @@ def test_stream_kernel_every_k_tail(G, oracle, bits):
                   seed=K + M, kernel=KERNEL_STREAM)
 
 
-@pytest.mark.parametrize("dt,bits,g,M,K,N", [(H.BF16, 8, 64, 300, 2048, 22016), (H.F16, 4, 128, 300, 4096, 22016)])
+@pytest.mark.parametrize("dt,bits,g,M,K,N", [(H.BF16, 8, 64, 700, 2048, 22016), (H.F16, 4, 128, 300, 4096, 22016)])
 def test_gemm_partial_last_round_split(G, oracle, dt, bits, g, M, K, N):
     # above 64 rows the tiles of a partial last round are launched with K cut
     # into runs: their columns go through fp32 partial sums and a reduce over
@@ -746,6 +755,53 @@ def test_gemm_partial_last_round_split(G, oracle, dt, bits, g, M, K, N):
     rows = np.r_[0:3, M - 3:M]
     r32, _ = oracle.linear(xb[rows], oc, osc, bb, dt, bits, g)
     assert H.rel_l2(split32[rows], r32) < 2e-5
+
+
+@pytest.mark.parametrize("dt,bits,g,M,K,N,spread", [
+    (H.BF16, 8, 64, 700, 2048, 22016, (-12, 4)),    # 256 x 256 tiles + a 256 x 128 remainder with K in runs
+    (H.F16, 8, 128, 300, 2112, 4096, (-8, 3)),      # groups of two k tiles, an odd number of tiles, K in runs of whole groups
+    (H.BF16, 8, 128, 300, 2048, 8192, (-100, 20)),  # scales of a column further apart than fp32 sums can span
+    (H.BF16, 4, 64, 300, 4096, 4096, (-12, 4)),     # int4: 128 x 256 tiles, two groups per k tile
+    (H.F16, 4, 128, 130, 2048, 4096, (-8, 3)),      # int4: 256 x 128 tiles
+])
+def test_group_wise_gemm_keeps_its_sums_in_units_of_the_group_scale(G, oracle, dt, bits, g, M, K, N, spread):
+    # above 64 rows the GEMM has one set of accumulators for group-wise scales: the
+    # sums are multiplied by (previous unit / new unit) where a group starts and by
+    # the last unit at the end.  Weights whose groups differ by many powers of two
+    # inside a column, with all-zero groups (scale 0) at the start, in the middle
+    # and at the end of K: every column must still match the oracle's fp32 sums,
+    # column by column (a whole-matrix norm would hide the small columns).
+    rng = np.random.default_rng(K + N + M)
+    ng = (K + g - 1) // g
+    lo, hi = spread
+    e = rng.integers(lo, hi + 1, size=(ng, N)).astype(np.float32)
+    if lo < -64:  # mostly ordinary groups, a few absurdly small or large ones
+        e = np.where(rng.random((ng, N)) < 0.8, rng.integers(-4, 3, size=(ng, N)), e).astype(np.float32)
+    mag = np.exp2(e)
+    mag[rng.random((ng, N)) < 0.1] = 0.0
+    mag[0, : N // 3] = 0.0       # columns that start with a zero group
+    mag[-1, N // 4 : N // 2] = 0.0  # ... and end with one
+    mag[:, 5] = 0.0              # an all-zero column
+    w = rng.standard_normal((K, N), dtype=np.float32) * 0.02 * np.repeat(mag, g, axis=0)[:K]
+    wb = H.f32_to_bits(w, dt)
+    xb = H.make_act(M, K, dt, seed=M)
+    oc, osc = oracle.weight_quantize(wb, dt, bits, g)
+    packed = H.gfx950_from_q(H.q_from_canonical(oc, bits), bits)
+    got = G.linear(xb, packed, None, osc, dt, N, bits, g, f32=True)
+    assert np.isfinite(got).all()
+    rows = np.r_[0:4, M // 2:M // 2 + 2, M - 3:M]
+    want, _ = oracle.linear(xb[rows], oc, osc, None, dt, bits, g)
+    err = np.linalg.norm(got[rows] - want, axis=0)
+    ref = np.linalg.norm(want, axis=0)
+    assert (got[:, 5] == 0).all() and (err[ref == 0] == 0).all()
+    worst = (err[ref > 0] / ref[ref > 0]).max()
+    assert worst < 2e-5, worst
+    # the same through T outputs and with K in runs where the plan has them (the scratch decides)
+    gotT = G.linear(xb, packed, None, osc, dt, N, bits, g)
+    assert np.array_equal(gotT, H.f32_to_bits(got, dt))
+    plain = G.linear(xb, packed, None, osc, dt, N, bits, g, f32=True, no_workspace=True)
+    errp = np.linalg.norm(plain[rows] - want, axis=0)
+    assert (errp[ref > 0] / ref[ref > 0]).max() < 2e-5
 
 
 def test_call_log_names_the_kernel(device):
