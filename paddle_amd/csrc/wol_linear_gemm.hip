@@ -505,7 +505,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   constexpr int kPerStage = kALoads + kBLoads + (G == 0 ? 0 : 1);
   static_assert(Q >= 2 && (Q - 2) % kFold != 0 && (Q - 2) % kFold != kFold - 1,
                 "the slice that holds the barrier neither starts nor ends a group");
-  static_assert(SWI == 0 || (TN == 2 && G == 0), "the swiglu epilogue pairs the two blocks of a wavefront");
+  static_assert(SWI == 0 || ((TN == 2 || (TN == 1 && WN % 2 == 0)) && (G == 0 || RESC)),
+                "the swiglu epilogue pairs the two blocks of a wavefront, or two neighbouring wavefronts");
+  // SWI with one block per wavefront: wavefront columns 2i and 2i+1 hold the gate and the up block of
+  // the same 32 output columns, and the up wavefront hands its sums over through LDS in the epilogue
+  constexpr bool kPair = SWI != 0 && TN == 1;
   static_assert(OFFS != 2 || G == 0, "row sums by dot products are taken out once, in the epilogue");
   static_assert(!RESC || (G != 0 && OFFS == 0), "rescaled sums are for group-wise scales and the exact dequantisers");
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -585,7 +589,15 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   const int sval = 2 * (wave * 64 + lane) < kGT * BN ? 2 * (wave * 64 + lane) : 0;
   const int sfold = sval / BN;
   int scol = strip_blk * kStripCols + sval % BN;
-  scol = scol < n_hi ? scol : n_hi - 2;  // past the last column: valid data, never used
+  if (SWI) {
+    // position p of the tile's columns is column p % 32 of block (p / 32) % 2 of wavefront column p / 64:
+    // the gate columns of that wavefront column, or the up columns N / 2 further on
+    const int pcol = sval % BN;
+    scol = (strip_blk + (pcol / 64) * 2) * kStripCols + pcol % 32;
+    scol = scol < n_hi ? scol : n_hi - 2;
+    scol += ((pcol / 32) % 2) * (N / 2);
+  }
+  scol = scol < (SWI ? N : n_hi) ? scol : n_hi - 2;  // past the last column: valid data, never used
   // Loads lo .. hi-1 of tile `it` into its stage; a stage's loads are numbered
   // [scales,] A loads, B loads.
   auto issue_range = [&](int it, int lo, int hi) {
@@ -622,7 +634,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   auto seg_n = [&](int s) { return seg_lo(s + 1) - seg_lo(s); };
 
   // columns of this lane's accumulators: block c of the wavefront, column r32
-  const int col0 = (strip_blk + wn * (SWI ? 1 : TN) * 2) * 16;
+  const int col0 = (strip_blk + (kPair ? wn / 2 : wn) * (SWI ? 1 : TN) * 2) * 16;
   int ncol[TN];
 #pragma unroll
   for (int c = 0; c < TN; ++c) {
@@ -630,6 +642,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
     ncol[c] = n < n_hi ? n : n_hi - 1;
     if (SWI && c == 1) ncol[c] = ncol[0] + N / 2;
   }
+  if (kPair && wn % 2 == 1) ncol[0] += N / 2;
   // this lane's scales of the tile in `stage`, out of LDS
   auto read_scales = [&](const unsigned char* stage, uint16_t (&dst)[kGT > 0 ? kGT : 1][TN]) {
     if (G != 0) {
@@ -925,12 +938,48 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   uint16_t* slab = reinterpret_cast<uint16_t*>(smem) + wave * 32 * kSlabRow;
   constexpr int kPieces = 32 * (kOutBlocks * 32 / 8);
   const int ld_out = SWI ? N / 2 : N;             // row length of the output
+  if constexpr (kPair) {
+    // behind the slabs: one block of fp32 sums per pair of wavefronts
+    constexpr int kXOff = (NW * 32 * kSlabRow * 2 + 255) / 256 * 256;
+    static_assert(kXOff + NW / 2 * 4096 <= kStages * kStage, "slabs and handed-over sums must fit in the stage buffers");
+    float* xbuf = reinterpret_cast<float*>(smem + kXOff) + (wave / 2) * 1024;
+#pragma unroll
+    for (int a = 0; a < TM; ++a) {
+      if (wn % 2 == 1) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) xbuf[r * 64 + lane] = tot[a][0][r] * sc[0] + bv[0];
+      }
+      __syncthreads();
+      if (wn % 2 == 0) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          float g = tot[a][0][r] * sc[0] + bv[0], u = xbuf[r * 64 + lane];
+          if (SWI == 2) {
+            g = to_f32<DT>(cast_out<DT>(g));
+            u = to_f32<DT>(cast_out<DT>(u));
+          }
+          slab[(8 * (r / 4) + 4 * b + r % 4) * kSlabRow + r32] = cast_out<DT>(act_swiglu(g, u));
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int q = lane; q < kPieces; q += 64) {
+          const int r = q / 4, cc = q % 4;
+          const int m = m0 + (wm * TM + a) * 32 + r;
+          const int n = col0 + cc * 8;
+          const u32x4 v = *reinterpret_cast<const u32x4*>(&slab[r * kSlabRow + cc * 8]);
+          if (m < M && n < n_hi) *reinterpret_cast<u32x4*>(out + static_cast<int64_t>(m) * ld_out + n) = v;
+        }
+      }
+      __syncthreads();  // the handed-over sums have been read
+    }
+    return;
+  }
 #pragma unroll
   for (int a = 0; a < TM; ++a) {
     if (SWI) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        float g = tot[a][0][r] * sc[0] + bv[0], u = tot[a][1][r] * sc[1] + bv[1];
+        float g = tot[a][0][r] * sc[0] + bv[0], u = tot[a][TN - 1][r] * sc[TN - 1] + bv[TN - 1];
         if (SWI == 2) {  // as if fc1 had been written out in T and read back
           g = to_f32<DT>(cast_out<DT>(g));
           u = to_f32<DT>(cast_out<DT>(u));
@@ -1131,7 +1180,7 @@ constexpr size_t dma_lds_bytes() {
 // SWI != 0 (swiglu epilogue): the strips are those of the gate half, [0, N / 32), a.out is [M, N / 2].
 template <int DT, int BITS, int G, int OFFS, int WM, int WN, int TM, int TN, int STAGES = 3, int SWI = 0, bool RESC = false>
 void launch_dma(const Args& a, int strip_lo, int strip_hi, int nsplit) {
-  constexpr int BM = WM * TM * 32, BN = (SWI ? 1 : TN) * WN * 32, TK = BITS == 8 ? 64 : 128;
+  constexpr int BM = WM * TM * 32, BN = (SWI ? TN * WN * 16 : TN * WN * 32), TK = BITS == 8 ? 64 : 128;  // BN: output columns
   if (strip_hi <= strip_lo) return;
   if (SWI) nsplit = 1;
   constexpr size_t lds = dma_lds_bytes<BITS, G, WM, WN, TM, TN, STAGES>();
@@ -1624,24 +1673,41 @@ void describe_linear_gemm(int64_t M, int64_t K, int64_t N, int bits, int group_s
 }
 
 // swiglu of a gate | up projection inside the GEMM's epilogue: the tiles with two
-// blocks per wavefront, per-channel scales, above the small-M configurations.
+// blocks per wavefront, above the small-M configurations.
 bool linear_gemm_fuses_swiglu(int64_t M, int64_t K, int64_t N, int bits, int group_size) {
   const int tk = bits == 8 ? 64 : 128;
-  return M > kSkinnyMaxM && group_size == -1 && K % tk == 0 && K / tk >= 2 && N % 32 == 0;
+  (void)group_size;
+  return M > kSkinnyMaxM && K % tk == 0 && K / tk >= 2 && N % 32 == 0;
 }
 
 namespace {
 // out [M, N / 2] = T(swiglu(x . W + bias)) in one launch
-template <int DT, int BITS>
+template <int DT, int BITS, int G>
 void launch_swiglu_gemm(const Args& a) {
   const int gate_strips = a.N / 2 / kStripCols;
-  if constexpr (BITS == 8) {
+  if constexpr (G != 0) {
+    // group-wise scales: the tiles with two blocks per wavefront and rescaled sums
+    if constexpr (BITS == 8) {
+      if (a.M >= 192) launch_dma<DT, 8, G, 0, 2, 4, 4, 2, 3, 1, true>(a, 0, gate_strips, 1);
+      else launch_dma<DT, 8, G, 0, 2, 4, 2, 2, 3, 1, true>(a, 0, gate_strips, 1);
+    } else {
+      // (256 x 128 tiles: gate and up blocks in neighbouring wavefronts)
+      if (tall_half_tile(a.M)) launch_dma<DT, 4, G, 0, 2, 4, 4, 1, 2, 1, true>(a, 0, gate_strips, 1);
+      else launch_dma<DT, 4, G, 0, 2, 4, 2, 2, 2, 1, true>(a, 0, gate_strips, 1);
+    }
+  } else if constexpr (BITS == 8) {
     if (a.M >= 192) launch_dma<DT, 8, 0, false, 2, 4, 4, 2, 3, 1>(a, 0, gate_strips, 1);
     else launch_dma<DT, 8, 0, false, 2, 4, 2, 2, 3, 1>(a, 0, gate_strips, 1);
   } else {
     if (a.M >= 192) launch_dma<DT, 4, 0, DT == WOL_DTYPE_BF16 ? 2 : 0, 2, 4, 4, 2, 2, 1>(a, 0, gate_strips, 1);
     else launch_dma<DT, 4, 0, DT == WOL_DTYPE_BF16 ? 1 : 0, 2, 4, 2, 2, 3, 1>(a, 0, gate_strips, 1);
   }
+}
+template <int DT, int BITS>
+void launch_swiglu_gemm_g(const Args& a) {
+  if (a.gshift < 0) launch_swiglu_gemm<DT, BITS, 0>(a);
+  else if (a.gshift == 6) launch_swiglu_gemm<DT, BITS, 64>(a);
+  else launch_swiglu_gemm<DT, BITS, 128>(a);
 }
 }  // namespace
 
@@ -1656,9 +1722,9 @@ int launch_linear_gemm(const void* x, const void* codes, const void* bias, const
   if (f.act == WOL_ACT_SWIGLU) {
     if (out_f32 || !linear_gemm_fuses_swiglu(M, K, N, bits, group_size)) return WOL_ERR_BAD_SHAPE;
     if (dtype == WOL_DTYPE_BF16) {
-      if (bits == 8) launch_swiglu_gemm<WOL_DTYPE_BF16, 8>(a); else launch_swiglu_gemm<WOL_DTYPE_BF16, 4>(a);
+      if (bits == 8) launch_swiglu_gemm_g<WOL_DTYPE_BF16, 8>(a); else launch_swiglu_gemm_g<WOL_DTYPE_BF16, 4>(a);
     } else {
-      if (bits == 8) launch_swiglu_gemm<WOL_DTYPE_F16, 8>(a); else launch_swiglu_gemm<WOL_DTYPE_F16, 4>(a);
+      if (bits == 8) launch_swiglu_gemm_g<WOL_DTYPE_F16, 8>(a); else launch_swiglu_gemm_g<WOL_DTYPE_F16, 4>(a);
     }
     return check_launch();
   }

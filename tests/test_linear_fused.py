@@ -154,27 +154,29 @@ def test_fused_against_oracle(device, oracle, dt, bits, g):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dt", [H.F16, H.BF16])
 @pytest.mark.parametrize("bits", [8, 4])
-def test_swiglu_in_the_gemm_epilogue(device, oracle, dt, bits):
-    # above 64 rows with per-channel scales the GEMM pairs gate and up columns in
-    # one wavefront and writes [M, N/2] itself: no fp32 sums, no extra pass.
+@pytest.mark.parametrize("g", [-1, 64, 128])
+def test_swiglu_in_the_gemm_epilogue(device, oracle, dt, bits, g):
+    # above 64 rows the GEMM pairs gate and up columns in one wavefront and
+    # writes [M, N/2] itself: no fp32 sums, no extra pass (group-wise scales: the
+    # tiles whose sums are kept in units of the group scale; their scales are
+    # gathered from the gate and the up columns like the codes).
     # 128-row and 256-row tiles, rows off the tile height, a gate half that ends
     # inside a column tile (N/2 = 1168), with and without bias
     from paddle_amd import _lib
 
-    for M, K, N in ((100, 512, 1024), (200, 512, 512), (300, 1024, 2336), (513, 256, 768)):
-        assert _lib.lib.wol_linear_fused_workspace(M, K, N, bits, -1, 0, 2) == _lib.lib.wol_linear_workspace(M, K, N, bits, -1)
-        assert _lib.lib.wol_linear_fused_workspace(M, K, N, bits, 128, 0, 2) >= M * N * 4  # group-wise: the pass
+    for M, K, N in ((100, 512, 1024), (200, 512, 512), (300, 1024, 2336), (513, 256, 768), (1000, 256, 2336)):
+        assert _lib.lib.wol_linear_fused_workspace(M, K, N, bits, g, 0, 2) == _lib.lib.wol_linear_workspace(M, K, N, bits, g)
         wb = H.make_weight(K, N, dt, seed=K + N + M)
         xb = H.make_act(M, K, dt, seed=M)
         bb = H.make_bias(N, dt, seed=6)
-        oc, osc = oracle.weight_quantize(wb, dt, bits, -1)
+        oc, osc = oracle.weight_quantize(wb, dt, bits, g)
         packed = H.gfx950_from_q(H.q_from_canonical(oc, bits), bits)
         for bias in (None, bb):
-            _, wantT = oracle.linear_fused(xb, None, oc, osc, bias, dt, bits, -1, 2)
-            got = _fused(xb, None, packed, bias, osc, dt, N, bits, -1, 2)
+            _, wantT = oracle.linear_fused(xb, None, oc, osc, bias, dt, bits, g, 2)
+            got = _fused(xb, None, packed, bias, osc, dt, N, bits, g, 2)
             assert got.shape == (M, N // 2)
             err = H.rel_l2(H.bits_to_f32(got, dt), H.bits_to_f32(wantT, dt))
-            assert err <= TOL, (err, dt, bits, M, K, N, bias is not None)
+            assert err <= TOL, (err, dt, bits, g, M, K, N, bias is not None)
 
 
 @pytest.mark.gpu
