@@ -296,6 +296,38 @@ def bench_linear_grad(torch, np, Q, _lib, H, dev, quick, failures):
             "rows": rows, "rel_l2_vs_oracle": err, "parity_sample": "first 4 rows of the M=2048 result"}
 
 
+def bench_fused_swiglu(torch, Q, dev, quick):
+    """weight_only_linear_fused(act="swiglu") on a gate|up projection of Llama-2-7B's
+    size (K = 4096, N = 2 x 11008) beside the plain linear on the same weight:
+    the swiglu is formed inside the decode kernels and the GEMM epilogue, so the
+    fused call should cost what the linear costs and save the separate
+    [M, N] -> [M, N/2] pass and its round trip through memory."""
+    K, N = 4096, 22016
+    bf16 = torch.bfloat16
+    w = _device_weight(torch, K, N, bf16, 700, dev)
+    rows = []
+    for bits, g in ((4, 128),) if quick else ((4, 128), (8, -1), (8, 64)):
+        codes, scale = _quantize(Q, w, bits, g)
+        ncp = max(2, -(-640 * 1024 * 1024 // codes.numel()))
+        cps = [codes.clone() for _ in range(ncp)]
+        wd = "int8" if bits == 8 else "int4"
+        for M in (1, 16, 2048):
+            gen = torch.Generator(device=dev)
+            gen.manual_seed(M)
+            x = torch.randn((M, K), generator=gen, device=dev, dtype=torch.float32).to(bf16)
+            n = 4 if M > 64 else 100
+            plain, _ = time_graph(torch, lambda i: Q.weight_only_linear(x, cps[i % ncp], None, scale, wd, None, g), n,
+                                  warm_launches=2 * n, warm_ms=20.0, replays=5)
+            fused, _ = time_graph(torch, lambda i: Q.weight_only_linear_fused(x, cps[i % ncp], None, scale, wd, g,
+                                                                             act="swiglu"), n,
+                                  warm_launches=2 * n, warm_ms=20.0, replays=5)
+            rows.append({"weights": "int%d g%d" % (bits, g), "M": M, "linear_us": round(plain / n * 1e6, 2),
+                         "fused_swiglu_us": round(fused / n * 1e6, 2), "fused_over_linear": round(fused / plain, 4)})
+        del cps
+    return {"workload": "gate|up projection K=4096 N=22016, bf16: weight_only_linear against "
+                        "weight_only_linear_fused(act=swiglu, out [M, 11008])", "rows": rows}
+
+
 def bench_moe_ffn(torch, np, Q, H, dev, quick, failures):
     """moe_ffn on weight-only int8 experts of Mixtral-8x7B's size (8 experts,
     hidden 4096, fc1 width 2 x 14336 for swiglu, bf16): a prefill-like call
@@ -643,7 +675,7 @@ def main():
         }
 
     # ---------------- every BASELINE configuration ----------------
-    configs = stack = grad = moe = None
+    configs = stack = grad = moe = fused = None
     if not args.no_configs:
         del copies, scales
         torch.cuda.empty_cache()
@@ -652,6 +684,8 @@ def main():
         grad = bench_linear_grad(torch, np, Q, _lib, H, dev, args.quick, failures)
         torch.cuda.empty_cache()
         moe = bench_moe_ffn(torch, np, Q, H, dev, args.quick, failures)
+        torch.cuda.empty_cache()
+        fused = bench_fused_swiglu(torch, Q, dev, args.quick)
 
     # ---------------- parity of what was measured, against the oracle ----------------
     O = H.O
@@ -782,6 +816,7 @@ def main():
         "decoder_stack": stack,
         "linear_grad": grad,
         "moe_ffn": moe,
+        "fused_swiglu": fused,
         "llm_int8": llm,
         "cpu_baseline": cpu,
         "parity": parity,
@@ -800,6 +835,9 @@ def main():
     if moe:
         for r in moe["rows"]:
             flat["moe_ffn_rows%d_frac" % r["rows"]] = r["frac"]
+    if fused:
+        for r in fused["rows"]:
+            flat["fused_swiglu_%s_M%d_over_linear" % (r["weights"].replace(" ", "_"), r["M"])] = r["fused_over_linear"]
     if llm:
         flat["llm_int8_frac"] = llm["roofline"]["frac"]
     for nm, tf in (ladder or {}).items():

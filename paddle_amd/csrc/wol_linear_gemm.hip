@@ -1214,6 +1214,13 @@ void launch_dma(const Args& a, int strip_lo, int strip_hi, int nsplit) {
   kern<<<dim3(static_cast<unsigned>(p.nbx * p.nby * p.nsplit)), dim3(64 * WM * WN), lds, a.stream>>>(p);
   if (nsplit > 1) {
     const int64_t total = static_cast<int64_t>(a.M) * ncols;
+    if (!SWI && a.act == WOL_ACT_SWIGLU) {
+      // a gate|up projection whose runs cover all of N (the small-M configurations): the kernel
+      // that adds the runs forms silu(gate) * up, out is [M, N / 2]
+      reduce_partials_swiglu_kernel<DT><<<dim3(static_cast<unsigned>((total / 8 + 255) / 256)), dim3(256), 0, a.stream>>>(
+          static_cast<const float*>(a.ws), p.nsplit, p.bias, a.out, a.out_f32, total / 2, a.N);
+      return;
+    }
     reduce_partials_kernel<DT><<<dim3(static_cast<unsigned>((total / 4 + 255) / 256)), dim3(256), 0, a.stream>>>(
         static_cast<const float*>(a.ws), p.nsplit, p.bias, a.out, a.out_f32, total, a.N,
         strip_lo * kStripCols, ncols, a.act);
@@ -1674,10 +1681,13 @@ void describe_linear_gemm(int64_t M, int64_t K, int64_t N, int bits, int group_s
 
 // swiglu of a gate | up projection inside the GEMM's epilogue: the tiles with two
 // blocks per wavefront, above the small-M configurations.
+// Up to 64 rows: where K is cut into runs, in the kernel that adds them.
 bool linear_gemm_fuses_swiglu(int64_t M, int64_t K, int64_t N, int bits, int group_size) {
   const int tk = bits == 8 ? 64 : 128;
-  (void)group_size;
-  return M > kSkinnyMaxM && K % tk == 0 && K / tk >= 2 && N % 32 == 0;
+  if (K % tk != 0 || K / tk < 2 || N % 32 != 0) return false;
+  if (M > kSkinnyMaxM) return true;
+  return plan_skinny(static_cast<int>(M), static_cast<int>(K), static_cast<int>(N), bits,
+                     group_size > 0 ? group_size : 0, SIZE_MAX).ns > 1;
 }
 
 namespace {
@@ -1719,7 +1729,11 @@ int launch_linear_gemm(const void* x, const void* codes, const void* bias, const
   const int gshift = group_size == 64 ? 6 : (group_size == 128 ? 7 : -1);
   const Args a{x, codes, bias, scale, out, static_cast<int>(M), static_cast<int>(K),
                static_cast<int>(N), gshift, out_f32 ? 1 : 0, workspace, workspace_bytes, stream, f.act};
-  if (f.act == WOL_ACT_SWIGLU) {
+  if (f.act == WOL_ACT_SWIGLU && M <= kSkinnyMaxM) {
+    // the runs of K must be the ones the plan was made with: all of the scratch is required
+    if (out_f32 || !linear_gemm_fuses_swiglu(M, K, N, bits, group_size)) return WOL_ERR_BAD_SHAPE;
+    if (workspace == nullptr || workspace_bytes < linear_gemm_workspace(M, K, N, bits, group_size)) return WOL_ERR_WORKSPACE;
+  } else if (f.act == WOL_ACT_SWIGLU) {
     if (out_f32 || !linear_gemm_fuses_swiglu(M, K, N, bits, group_size)) return WOL_ERR_BAD_SHAPE;
     if (dtype == WOL_DTYPE_BF16) {
       if (bits == 8) launch_swiglu_gemm_g<WOL_DTYPE_BF16, 8>(a); else launch_swiglu_gemm_g<WOL_DTYPE_BF16, 4>(a);

@@ -267,6 +267,48 @@ def test_swiglu_in_the_batched_kernel(device, oracle, dt, bits, g):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dt,bits,g,M,K,N", [(H.BF16, 8, -1, 48, 4096, 12288), (H.F16, 4, 128, 17, 8192, 22016),
+                                             (H.BF16, 4, 64, 40, 4096, 22016), (H.F16, 8, 64, 64, 8192, 28672)])
+def test_swiglu_where_the_small_m_gemm_adds_its_runs(device, oracle, dt, bits, g, M, K, N):
+    # 17 to 64 rows on a large weight: the GEMM cuts K into runs and the kernel
+    # that adds them forms the swiglu, so the fused call needs the linear's own
+    # scratch and nothing more.  Device-made weight, oracle on column slices.
+    import ctypes
+
+    import torch
+    from paddle_amd import _lib
+    from paddle_amd.nn import quant as Q
+
+    lws = _lib.lib.wol_linear_workspace(M, K, N, bits, g)
+    plan = ctypes.create_string_buffer(256)
+    _lib.check(_lib.lib.wol_linear_plan(M, K, N, bits, g, lws, plan, 256))
+    assert b"gemm_dma_kernel" in plan.value and b"reduce_partials" in plan.value, plan.value
+    assert _lib.lib.wol_linear_fused_workspace(M, K, N, bits, g, 0, 2) == lws > 0
+    xb = H.make_act(M, K, dt, seed=M)
+    bb = H.make_bias(N, dt, seed=6)
+    gen = torch.Generator(device="cuda").manual_seed(K + N)
+    w = (torch.randn(K, N, device="cuda", generator=gen) * 0.02).to(H.torch_dtype(dt))
+    codes, scale = Q.weight_quantize(w, algo="weight_only_int8" if bits == 8 else "weight_only_int4", group_size=g)
+    x_d, b_d = (H.bits_to_torch(v, dt, "cuda:0") for v in (xb, bb))
+    for bias in (None, bb):
+        got = _fused_dev(x_d, None, codes, None if bias is None else b_d, scale, dt, N, bits, g, 2)
+        assert got.shape == (M, N // 2) and bool(torch.isfinite(got.float()).all())
+        for c0 in (0, 256 - 16, (N // 4) // 16 * 16, N // 2 - 32):
+            cols = np.r_[c0:c0 + 32, N // 2 + c0:N // 2 + c0 + 32]
+            oc, osc = oracle.weight_quantize(H.torch_to_bits(w[:, cols].contiguous()), dt, bits, g)
+            assert np.array_equal(osc, H.torch_to_bits(scale[..., cols].contiguous()))
+            _, wantT = oracle.linear_fused(xb, None, oc, osc, None if bias is None else bias[cols], dt, bits, g, 2)
+            part = got[:, c0:c0 + 32].contiguous()
+            err = H.rel_l2(H.bits_to_f32(H.torch_to_bits(part), dt), H.bits_to_f32(wantT, dt))
+            assert err <= TOL, (err, dt, bits, g, M, K, N, c0, bias is not None)
+    # without the scratch the call is refused, not run on another plan
+    out = torch.empty((M, N // 2), dtype=x_d.dtype, device="cuda")
+    rc = _lib.lib.wol_linear_fused(x_d.data_ptr(), None, codes.data_ptr(), None, scale.data_ptr(), dt, M, K, N, bits, g, 2,
+                                   out.data_ptr(), None, 0, None)
+    assert rc == 8  # WOL_ERR_WORKSPACE
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dt", [H.F16, H.BF16])
 def test_fused_pre_scale_equals_the_two_ops(device, oracle, dt):
     # folding apply_per_channel_scale into the linear must not change a bit:
