@@ -28,7 +28,21 @@
 #include "wol_common.h"
 #include "wol_dequant.h"
 
+// The instantiations are split over two translation units by activation
+// type, so that they compile side by side: this file is the bf16 half and
+// holds the host-side planning; wol_linear_stream_f16.hip includes it with
+// WOL_STREAM_F16_TU defined and yields the fp16 half only.
 namespace wol {
+
+// What a launch needs, whichever half runs it.
+struct StreamArgs {
+  const void* x; const void* codes; const void* bias; const void* scale; void* out;
+  int M, K, N, gshift, out_f32, tn; hipStream_t stream;
+  const void* pre; int act;  // act: none or gelu; the gate|up form is chosen by the caller of the half
+};
+// The fp16 half (wol_linear_stream_f16.hip): swi = the gate|up form, wk = wavefronts of the workgroup.
+void launch_linear_stream_f16(const StreamArgs& a, int bits, bool swi, int wk, int nu);
+
 namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -534,11 +548,7 @@ __global__ __launch_bounds__(WK * 64) void stream_kernel(
   k.run(codes, bias, out, out_f32, red);
 }
 
-struct Args {
-  const void* x; const void* codes; const void* bias; const void* scale; void* out;
-  int M, K, N, gshift, out_f32, tn; hipStream_t stream;
-  const void* pre; int act;  // act: none or gelu; the gate|up form is a template argument
-};
+using Args = StreamArgs;
 
 template <int DT, int BITS, int MP, int MT, int WK, int NU, int TN, bool SWI = false>
 void launch_tn(const Args& a) {
@@ -655,6 +665,15 @@ void launch_m(const Args& a, int wk, int nu) {
 
 }  // namespace
 
+#if defined(WOL_STREAM_F16_TU)
+void launch_linear_stream_f16(const StreamArgs& a, int bits, bool swi, int wk, int nu) {
+  if (swi) {
+    if (bits == 8) launch_m_swi<WOL_DTYPE_F16, 8>(a, wk, nu); else launch_m_swi<WOL_DTYPE_F16, 4>(a, wk, nu);
+  } else {
+    if (bits == 8) launch_m<WOL_DTYPE_F16, 8>(a, wk, nu); else launch_m<WOL_DTYPE_F16, 4>(a, wk, nu);
+  }
+}
+#else
 // Work split.  A unit is kU k steps of one strip.  When the problem is small
 // enough that one unit per wavefront keeps every wavefront resident at once
 // (at most ~6 per SIMD on 1024 SIMDs) and the unit count per strip is a power
@@ -739,16 +758,17 @@ int launch_linear_stream(const void* x, const void* codes, const void* bias, con
     if (dtype == WOL_DTYPE_BF16) {
       if (bits == 8) launch_m_swi<WOL_DTYPE_BF16, 8>(a, total, nu); else launch_m_swi<WOL_DTYPE_BF16, 4>(a, total, nu);
     } else {
-      if (bits == 8) launch_m_swi<WOL_DTYPE_F16, 8>(a, total, nu); else launch_m_swi<WOL_DTYPE_F16, 4>(a, total, nu);
+      launch_linear_stream_f16(a, bits, true, total, nu);
     }
     return check_launch();
   }
   if (dtype == WOL_DTYPE_BF16) {
     if (bits == 8) launch_m<WOL_DTYPE_BF16, 8>(a, wk, nu); else launch_m<WOL_DTYPE_BF16, 4>(a, wk, nu);
   } else {
-    if (bits == 8) launch_m<WOL_DTYPE_F16, 8>(a, wk, nu); else launch_m<WOL_DTYPE_F16, 4>(a, wk, nu);
+    launch_linear_stream_f16(a, bits, false, wk, nu);
   }
   return check_launch();
 }
+#endif  // WOL_STREAM_F16_TU
 
 }  // namespace wol

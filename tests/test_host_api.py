@@ -67,8 +67,13 @@ def test_workspace_queries(lib):
     assert L.wol_linear_workspace(1, 4096, 11008, 4, 128) == 0       # streaming kernel
     assert L.wol_linear_workspace(2048, 4096, 12288, 8, -1) == 0     # one workgroup per tile covers all of K
     assert L.wol_linear_workspace(1024, 4096, 4096, 8, 64) == 2 * 1024 * 4096 * 4  # 128 tiles: two K runs
-    # 384 tiles: the 256 of the whole round run as they are, the other 128 (4096 columns) in two K runs
-    assert L.wol_linear_workspace(1024, 4096, 12288, 8, 64) == 2 * 1024 * 4096 * 4
+    # group-wise int8 takes 256 x 256 tiles like per-channel int8: 192 of them, one round, no K runs
+    assert L.wol_linear_workspace(1024, 4096, 12288, 8, 64) == 0
+    # group-wise int4, 256 x 128 tiles, 384 of them: the 256 of the whole round run as they are, the other 128
+    # (4096 columns) in two K runs
+    assert L.wol_linear_workspace(1024, 4096, 12288, 4, 128) == 2 * 1024 * 4096 * 4
+    # 256 x 256 tiles on the columns of whole rounds, one 256 x 128 column tile left over: four K runs of it
+    assert L.wol_linear_workspace(700, 2048, 22016, 8, 64) == 4 * 700 * 256 * 4
     # small M on the GEMM: whole fp32 [M, N] partial buffers, at most 16 of them
     for M, K, N, bits, g in [(64, 8192, 28672, 4, 128), (48, 4096, 11008, 4, -1), (24, 8192, 28672, 4, 128)]:
         need = L.wol_linear_workspace(M, K, N, bits, g)
