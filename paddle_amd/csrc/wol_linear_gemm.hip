@@ -137,6 +137,11 @@ __device__ inline void tile_of_block(int id, int nbx, int nby, int* bx, int* by)
 // and each owns nby/rg row blocks x nbx/(8/rg) column blocks, the shape that
 // makes the sum of the A rows and B columns an L2 has to fetch smallest
 // (plan_xcd_rows on the host).  rg == 0: plain order.
+// rg < 0 (the grouped GEMM over experts; nby a multiple of 8 * -rg): runs of
+// -rg consecutive row tiles -- one expert's, when the experts have about that
+// many -- go to one XCD with all their column tiles, column tile by column
+// tile, so that the row tiles of an expert meet its weights in one L2 while
+// they are there, and no other XCD fetches them.
 __device__ inline void tile_of_block_2d(int id, int nbx, int nby, int rg, int* bx, int* by) {
   if (rg == 0) {
     *by = id % nby;
@@ -144,6 +149,13 @@ __device__ inline void tile_of_block_2d(int id, int nbx, int nby, int rg, int* b
     return;
   }
   constexpr int kXcd = 8;
+  if (rg < 0) {
+    const int tpe = -rg, x = id % kXcd, i = id / kXcd;
+    const int per = tpe * nbx, gi = i / per, w = i % per;
+    *by = (gi * kXcd + x) * tpe + w % tpe;
+    *bx = w / tpe;
+    return;
+  }
   const int x = id % kXcd, i = id / kXcd;
   const int r = nby / rg, c = nbx / (kXcd / rg);
   *by = (x % rg) * r + i % r;
@@ -1493,6 +1505,7 @@ struct MoeLaunch {
   int64_t rows;
   float* partial;
   const int64_t* valid_rows;
+  int tiles_per_expert = 0;  // > 0: row tiles an expert has on average; its tiles then share an XCD (max_tiles a multiple of 8 x this)
 };
 
 // One grouped GEMM: every expert's rows against that expert's weights, tiles
@@ -1522,10 +1535,11 @@ void launch_moe_gemm_cfg(const void* x, const MoeLaunch& ml, const void* codes, 
   p.strip_lo = 0; p.strip_hi = static_cast<int>(out_cols / kStripCols);
   p.nbx = static_cast<int>((out_cols + BN - 1) / BN);
   p.nby = max_tiles;
+  p.xcd_rows = 0;
+  if (ml.tiles_per_expert > 0 && max_tiles % (8 * ml.tiles_per_expert) == 0) p.xcd_rows = -ml.tiles_per_expert;
   p.tiles_per_split = (tiles + ns - 1) / ns;
   p.nsplit = (tiles + p.tiles_per_split - 1) / p.tiles_per_split;
   p.out = p.nsplit > 1 ? static_cast<void*>(ml.partial) : out;
-  p.xcd_rows = 0;
   p.act = WOL_ACT_NONE;
   p.moe_table = table;
   p.moe_codes_stride = K * N * BITS / 8;
@@ -1775,15 +1789,24 @@ int launch_moe_ffn(const void* x, const int64_t* rows_before_expert, const void*
                    int num_experts, int bits, void* out, void* workspace, hipStream_t stream) {
   unsigned char* ws = static_cast<unsigned char*>(workspace);
   const int bm = moe_tile_rows(rows, num_experts, bits);
-  const int max_tiles = moe_max_tiles(rows, num_experts, bm);
+  int max_tiles = moe_max_tiles(rows, num_experts, bm);
+  // large tiles (one workgroup per CU): an expert's row tiles and all their column tiles on one XCD.  The
+  // table (sized for 32-row tiles) has room for the padding of its length to a multiple of 8 experts' tiles.
+  int tpe = 0;
+  if (bm >= 128) {
+    tpe = static_cast<int>((rows / (num_experts > 0 ? num_experts : 1) + bm - 1) / bm);
+    tpe = tpe < 1 ? 1 : tpe;
+    const int padded = (max_tiles + 8 * tpe - 1) / (8 * tpe) * (8 * tpe);
+    if (padded <= moe_max_tiles(rows, num_experts, 32)) max_tiles = padded; else tpe = 0;
+  }
   MoeTile* table = reinterpret_cast<MoeTile*>(ws);
   unsigned char* fc1 = ws + moe_up(static_cast<size_t>(moe_max_tiles(rows, num_experts, 32)) * sizeof(MoeTile));
   unsigned char* act = fc1 + moe_up(static_cast<size_t>(rows) * inter * 2);
   float* partial = reinterpret_cast<float*>(act + moe_up(static_cast<size_t>(rows) * (inter / 2) * 2));
   // the second GEMM has hidden / 256 column tiles only: K (= inter / 2) in runs when the tiles are small
-  const MoeLaunch l1{reinterpret_cast<const int*>(table), max_tiles, bm, 1, rows, nullptr, nullptr};
+  const MoeLaunch l1{reinterpret_cast<const int*>(table), max_tiles, bm, 1, rows, nullptr, nullptr, tpe};
   const MoeLaunch l2{reinterpret_cast<const int*>(table), max_tiles, bm, moe_runs(inter / 2, hidden, bits, bm, max_tiles),
-                     rows, bm < 128 ? partial : nullptr, rows_before_expert + (num_experts - 1)};
+                     rows, bm < 128 ? partial : nullptr, rows_before_expert + (num_experts - 1), tpe};
   moe_plan_kernel<<<dim3(1), dim3(256), 0, stream>>>(rows_before_expert, num_experts, bm, max_tiles, rows, table);
 #define WOL_MOE(DT, B)                                                                                        \
   do {                                                                                                        \
