@@ -183,6 +183,14 @@ size_t wol_linear_workspace(int64_t M, int64_t K, int64_t N, int bits,
  * allows and it is measured faster (10 to 32 rows on some shapes), the
  * batched kernel with K cut into runs across workgroups runs instead.  The
  * reference's split is M <= 3 (gpu/weight_only_linear_kernel.cu:60-61).
+ * code * scale is never rounded to T in any kernel (the reference's GEMM
+ * rounds the scaled weight to T, cutlass_extensions/gemm/warp/
+ * mma_tensorop_dequantizer.h:155-195): per-channel scales multiply the fp32
+ * sums; group-wise scales multiply each group's fp32 sum up to 64 rows, and
+ * above 64 rows the running sums are kept in units of the current group's
+ * scale and rescaled from group to group (one fp32 rounding of the sums per
+ * group; a column's unit never falls more than 2^64 below its largest scale,
+ * so no ratio of scales overflows).
  * x, codes, scale, out and (when given) bias must be 16-byte aligned: the
  * kernels read and write 16 bytes at a time, the output rows included
  * (WOL_ERR_ALIGNMENT otherwise).
