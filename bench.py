@@ -417,7 +417,7 @@ def cpu_decode_baseline(np, torch, H, w_bits, x_bits, cfg, budget_s=10.0):
     x32 = torch.from_numpy(H.bits_to_f32(x_bits, dt))
     cores = torch.get_num_threads()
     t_start = time.perf_counter()
-    while reps < 3 or (time.perf_counter() - t_start < budget_s and reps < 50):
+    while reps < 3 or (time.perf_counter() - t_start < budget_s and reps < 400):
         t0 = time.perf_counter()
         w32, _ = O.dequantize(codes, scale, dt, bits, g)
         t1 = time.perf_counter()
