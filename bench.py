@@ -328,6 +328,63 @@ def bench_fused_swiglu(torch, Q, dev, quick):
                         "weight_only_linear_fused(act=swiglu, out [M, 11008])", "rows": rows}
 
 
+def bench_prefill_phases(torch, np, Q, _lib, dev):
+    """wol_prefill_phases: the prefill GEMM's 256 x 256 launch on an instantiation
+    that reads the cycle counter around its waits.  Per k tile and wavefront,
+    averaged over all wavefronts of the launch: cycles between the barriers
+    (MFMAs and what is issued among them), waiting for the wavefront's own tile
+    loads, waiting at the barrier; and the prologue and epilogue of a tile."""
+    K = 4096
+    bf16 = torch.bfloat16
+    rows = []
+    for M, N in ((2048, 8192), (8192, 8192)):
+        w = _device_weight(torch, K, N, bf16, 900, dev)
+        codes, scale = _quantize(Q, w, 8, -1)
+        del w
+        gen = torch.Generator(device=dev)
+        gen.manual_seed(M)
+        x = torch.randn((M, K), generator=gen, device=dev, dtype=torch.float32).to(bf16)
+        out = torch.empty((M, N), dtype=bf16, device=dev)
+        wgs = (M // 256) * (N // 256)
+        ph = torch.zeros(wgs * 64, dtype=torch.int64, device=dev)
+
+        def stamped(_i):
+            _lib.check(_lib.lib.wol_prefill_phases(x.data_ptr(), codes.data_ptr(), scale.data_ptr(), M, K, N,
+                                                   out.data_ptr(), ph.data_ptr(), ph.numel() * 8, torch.cuda.current_stream().cuda_stream))
+
+        t_st, _ = time_graph(torch, stamped, 4, warm_launches=8, warm_ms=30.0, replays=5)
+        t_pl, _ = time_graph(torch, lambda i: Q.weight_only_linear(x, codes, None, scale, "int8"), 4, warm_launches=8,
+                             warm_ms=30.0, replays=5)
+        torch.cuda.synchronize()
+        c = ph.cpu().numpy().reshape(wgs * 8, 8).astype(np.float64)
+        tiles = float(c[0, 7])
+        mean = c.mean(axis=0)
+        tiles_per_cu = max(1.0, wgs / 256.0)
+        rows.append({
+            "M": M, "K": K, "N": N, "workgroups": wgs, "k_tiles": int(tiles),
+            "stamped_us": round(t_st / 4 * 1e6, 1), "product_us": round(t_pl / 4 * 1e6, 1),
+            "counter_ghz": round(mean[6] * tiles_per_cu / (t_st / 4) / 1e9, 3),
+            "cycles_per_k_tile": {"between_barriers": round(mean[1] / tiles, 1), "wait_own_loads": round(mean[2] / tiles, 1),
+                                  "wait_barrier": round(mean[3] / tiles, 1),
+                                  "mfma_issue_at_full_rate": 2048},
+            "cycles_per_tile": {"prologue": round(mean[0], 0), "last_tile_tail": round(mean[4], 0),
+                                "epilogue": round(mean[5], 0), "total": round(mean[6], 0)},
+            "share_of_total": {"between_barriers": round(mean[1] / mean[6], 4), "wait_own_loads": round(mean[2] / mean[6], 4),
+                               "wait_barrier": round(mean[3] / mean[6], 4), "prologue": round(mean[0] / mean[6], 4),
+                               "epilogue": round((mean[4] + mean[5]) / mean[6], 4)},
+            "slowest_wavefront_wait_barrier_share": round(float((c[:, 3] / c[:, 6]).min()), 4),
+            # wavefronts 0-3 of a workgroup are the first on their SIMDs, 4-7 the second
+            "by_wavefront_of_simd": {
+                name: {"between_barriers": round(float(g[:, 1].mean()) / tiles, 1),
+                       "wait_barrier": round(float(g[:, 3].mean()) / tiles, 1)}
+                for name, g in (("first", c.reshape(wgs, 8, 8)[:, :4].reshape(-1, 8)),
+                                ("second", c.reshape(wgs, 8, 8)[:, 4:].reshape(-1, 8)))},
+        })
+    return {"what": "wol_prefill_phases: per-wavefront cycle stamps in the 256 x 256 tile of the prefill GEMM "
+                    "(int8 per-channel, bf16); 2048 cycles per k tile is what two wavefronts per SIMD need to issue "
+                    "their 2 x 32 MFMAs of 32 cycles back to back", "rows": rows}
+
+
 def bench_moe_ffn(torch, np, Q, H, dev, quick, failures):
     """moe_ffn on weight-only int8 experts of Mixtral-8x7B's size (8 experts,
     hidden 4096, fc1 width 2 x 14336 for swiglu, bf16): a prefill-like call
@@ -675,7 +732,7 @@ def main():
         }
 
     # ---------------- every BASELINE configuration ----------------
-    configs = stack = grad = moe = fused = None
+    configs = stack = grad = moe = fused = phases = None
     if not args.no_configs:
         del copies, scales
         torch.cuda.empty_cache()
@@ -686,6 +743,8 @@ def main():
         moe = bench_moe_ffn(torch, np, Q, H, dev, args.quick, failures)
         torch.cuda.empty_cache()
         fused = bench_fused_swiglu(torch, Q, dev, args.quick)
+        torch.cuda.empty_cache()
+        phases = bench_prefill_phases(torch, np, Q, _lib, dev)
 
     # ---------------- parity of what was measured, against the oracle ----------------
     O = H.O
@@ -817,6 +876,7 @@ def main():
         "linear_grad": grad,
         "moe_ffn": moe,
         "fused_swiglu": fused,
+        "prefill_phases": phases,
         "llm_int8": llm,
         "cpu_baseline": cpu,
         "parity": parity,
@@ -838,6 +898,10 @@ def main():
     if fused:
         for r in fused["rows"]:
             flat["fused_swiglu_%s_M%d_over_linear" % (r["weights"].replace(" ", "_"), r["M"])] = r["fused_over_linear"]
+    if phases:
+        for r in phases["rows"]:
+            for k, v in r["share_of_total"].items():
+                flat["prefill_phase_M%d_%s_share" % (r["M"], k)] = v
     if llm:
         flat["llm_int8_frac"] = llm["roofline"]["frac"]
     for nm, tf in (ladder or {}).items():

@@ -72,6 +72,33 @@ int wol_mfma_probe(int variant, const void* operands, size_t operand_bytes,
                    int workgroups, int iters, float* out, void* stream);
 
 /*
+ * Where the wavefronts of the prefill GEMM spend their cycles: runs the
+ * 256 x 256 launch of wol_linear (bf16 activations, int8 codes with
+ * per-channel scales, GFX950 layout; M and N multiples of 256, K a multiple
+ * of 64 and at least 192; no bias) on an instantiation of the same kernel that
+ * reads the shader's cycle counter at kernel entry, around the two waits of
+ * every k tile and around the epilogue.  out: [M, N] bf16, bit for bit what
+ * wol_linear writes.  phases: for workgroup w (of (M / 256) * (N / 256)) and
+ * wavefront v (of 8), eight 64-bit counts at phases[(w * 8 + v) * 8 ...]:
+ *   0  kernel entry to the first k tile's barrier (addresses, first loads)
+ *   1  between the barriers of the k loop: MFMAs and whatever is issued among
+ *      them (fragment reads, dequantisation, tile loads) and stalls on it
+ *   2  waiting for this wavefront's own direct-to-LDS loads of the next tile
+ *   3  waiting at the workgroup barrier for the other wavefronts
+ *   4  the last tile's tail and the closing barrier
+ *   5  epilogue (scale, cast, store)
+ *   6  entry to end
+ *   7  k tiles (K / 64)
+ * Every stamp costs a scalar memory round trip (three per k tile), so the
+ * stamped kernel runs a few per cent longer than the product's.
+ */
+#define WOL_PREFILL_PHASES_PER_WORKGROUP 64 /* counts: 8 wavefronts x 8 */
+int wol_prefill_phases(const void* x, const void* codes, const void* scale,
+                       int64_t M, int64_t K, int64_t N, void* out,
+                       unsigned long long* phases, size_t phases_bytes,
+                       void* stream);
+
+/*
  * Writes into buf (NUL-terminated, at most buf_bytes) one line naming the
  * kernel and launch shape wol_linear takes for a problem when it is handed
  * workspace_bytes of scratch.  No device work.  For benchmarks and dispatch

@@ -312,6 +312,9 @@ int launch_linear_grad(const void* out_grad, const void* codes, const void* scal
 int launch_read_floor(const void* codes, int64_t K, int64_t N, int bits, void* out,
                       hipStream_t stream);
 int launch_mfma_probe(int variant, const void* ops, int workgroups, int iters, float* out, hipStream_t stream);
+// The prefill GEMM's 256 x 256 launch (int8 per-channel, bf16) with cycle stamps per wavefront (wol_prefill_phases).
+int launch_prefill_phases(const void* x, const void* codes, const void* scale, int64_t M, int64_t K, int64_t N,
+                          void* out, unsigned long long* stamps, hipStream_t stream);
 int launch_mfma_ceiling(const void* operands, int workgroups, int iters, float* out,
                         hipStream_t stream);
 int launch_prescale(const void* x, const void* scales, int dtype, int64_t rows, int64_t cols,

@@ -421,6 +421,8 @@ struct DmaParams {
   const int* moe_table;
   int64_t moe_codes_stride;     // bytes between two experts' packed weights
   int moe_rows;                 // rows of the whole grouped problem (the partial sums' row count)
+  // STAMP instantiation only: six cycle counts per wavefront, [workgroup][wavefront][8] (see wol_prefill_phases)
+  unsigned long long* stamps;
 };
 
 // One entry of the row-tile table of a grouped launch.
@@ -486,7 +488,14 @@ struct MoeTile {
 // below the largest scale the column has had so far (a group that small
 // weighs nothing next to the others in fp32), so the sums cannot overflow
 // however the scales of a column differ.
-template <int DT, int BITS, int G, int OFFS, int WM, int WN, int TM, int TN, int STAGES, int SWI = 0, bool RESC = false>
+//
+// STAMP (a diagnostic instantiation, never on a product path): every wavefront
+// reads the cycle counter at kernel entry, around the two waits of every k
+// tile (for its own tile loads, then for the workgroup) and around the
+// epilogue, and leaves the sums in p.stamps.  The reads sit where the
+// wavefront has just waited for all its LDS traffic anyway.
+template <int DT, int BITS, int G, int OFFS, int WM, int WN, int TM, int TN, int STAGES, int SWI = 0, bool RESC = false,
+          bool STAMP = false>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   constexpr int NW = WM * WN;
@@ -525,6 +534,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   static_assert(OFFS != 2 || G == 0, "row sums by dot products are taken out once, in the epilogue");
   static_assert(!RESC || (G != 0 && OFFS == 0), "rescaled sums are for group-wise scales and the exact dequantisers");
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  unsigned long long st_entry = 0, st_prev = 0, st_work = 0, st_loads = 0, st_bar = 0, st_loop0 = 0;
+  if (STAMP) st_entry = __builtin_readcyclecounter();
 
   const uint16_t* __restrict__ x = p.x;
   const uint16_t* __restrict__ scale = p.scale;
@@ -695,6 +706,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   constexpr int kValuPerMfma = ((OFFS == 2 ? 4 * TN + 4 * TM : (BITS == 8 ? 16 : 12) * TN) + TM * TN - 1) / (TM * TN) + 2;
   constexpr int kValuRescale = RESC ? 16 : 0;  // more per MFMA in the slice that starts a group
   constexpr int kHalf = (TM * TN + 1) / 2;  // MFMAs of a slice issued before the barrier
+  // The largest tile (one workgroup per CU, wavefronts w and w + 4 on one SIMD): left alone the older
+  // wavefront of a SIMD wins every arbitration, finishes a k tile in two thirds of the tile's time and
+  // waits out the rest at the barrier (cycle stamps: 1864 against 2634 cycles of work per tile, 888
+  // against 114 at the barrier).  Taking turns evens that out; it is worth 1.5 to 2 %.
+  constexpr bool kTakeTurns = NW == 8 && TM * TN == 8;
 
   // The wavefront's pipeline registers: raw codes of the current and the next
   // tile, and two sets of operands -- the one the MFMAs of slice q use and the
@@ -800,6 +816,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   if (kStages == 3) issue_range(2, 0, seg_lo(2));  // the rest of tile 2 goes out during tile 0
   wait_vmcnt<(kStages - 2) * kPerStage + (kStages == 3 ? (2 * kPerStage + Q - 1) / Q : kPerStage)>();  // tile 0 has landed
   __builtin_amdgcn_s_barrier();
+  if (STAMP) st_loop0 = st_prev = __builtin_readcyclecounter();
   read_b(smem, braw[0]);
   read_a(smem, af[0], 0);
   dequant(bf[0], braw[0], 0);
@@ -818,6 +835,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
     read_scales(stage, sraw);  // before the stage is handed over
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
+      if (kTakeTurns) {
+        // slice by slice the two wavefronts of a SIMD take turns at the higher priority
+        if ((wave >> 2) == (q & 1)) __builtin_amdgcn_s_setprio(1);
+        else __builtin_amdgcn_s_setprio(0);
+      }
       if (q != Q - 2) {
         const bool last = q == Q - 1;
         // this slice's share of the tile loads (segment 1 of tile it+3, or segment q+2 of tile it+2)
@@ -852,8 +874,18 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
         // wavefront is there, tile it+1 (landed by now) may be read and the
         // stage refilled with tile it+3
         __builtin_amdgcn_s_waitcnt(0x0070 | (0xF << 0) | (3 << 14));  // lgkmcnt(0)
+        unsigned long long st_a = 0, st_b = 0;
+        if (STAMP) st_a = __builtin_readcyclecounter();
         wait_vmcnt<(kStages - 2) * kPerStage>();
+        if (STAMP) st_b = __builtin_readcyclecounter();
         __builtin_amdgcn_s_barrier();
+        if (STAMP) {
+          const unsigned long long st_c = __builtin_readcyclecounter();
+          st_work += st_a - st_prev;
+          st_loads += st_b - st_a;
+          st_bar += st_c - st_b;
+          st_prev = st_c;
+        }
         issue_range(it + kStages, 0, seg_lo(1));
         read_b(next, raw_next);
         dequant(bf[(q + 1) & 1], raw, q + 1);
@@ -878,6 +910,23 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   }
   wait_vmcnt<0>();
   __builtin_amdgcn_s_barrier();  // the spare loads are done and every wavefront has stopped reading
+  unsigned long long st_loop1 = 0;
+  if (STAMP) st_loop1 = __builtin_readcyclecounter();
+  // the stamps leave at the end of the epilogue (lane 0 of every wavefront)
+  auto leave_stamps = [&]() {
+    if (STAMP && lane == 0 && p.stamps != nullptr) {
+      unsigned long long* o = p.stamps + (static_cast<size_t>(blockIdx.x) * NW + wave) * 8;
+      const unsigned long long st_end = __builtin_readcyclecounter();
+      o[0] = st_loop0 - st_entry;   // entry to the first tile's barrier
+      o[1] = st_work;               // between the barriers: MFMAs and everything issued among them
+      o[2] = st_loads;              // waiting for this wavefront's own tile loads
+      o[3] = st_bar;                // waiting for the other wavefronts
+      o[4] = st_loop1 - st_prev;    // the last tile's tail and the closing barrier
+      o[5] = st_end - st_loop1;     // epilogue
+      o[6] = st_end - st_entry;     // all of it
+      o[7] = static_cast<unsigned long long>(niter);
+    }
+  };
 
   // ---- epilogue: scale, bias, cast; 32-row slabs leave through LDS as 16-byte stores ----
   // accumulator element r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its block
@@ -1017,6 +1066,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
     }
     __builtin_amdgcn_wave_barrier();
   }
+  leave_stamps();
 #endif
 }
 
@@ -1223,6 +1273,7 @@ void launch_dma(const Args& a, int strip_lo, int strip_hi, int nsplit) {
   p.moe_table = nullptr;
   p.moe_codes_stride = 0;
   p.moe_rows = 0;
+  p.stamps = nullptr;
   kern<<<dim3(static_cast<unsigned>(p.nbx * p.nby * p.nsplit)), dim3(64 * WM * WN), lds, a.stream>>>(p);
   if (nsplit > 1) {
     const int64_t total = static_cast<int64_t>(a.M) * ncols;
@@ -1544,6 +1595,7 @@ void launch_moe_gemm_cfg(const void* x, const MoeLaunch& ml, const void* codes, 
   p.moe_table = table;
   p.moe_codes_stride = K * N * BITS / 8;
   p.moe_rows = static_cast<int>(ml.rows);
+  p.stamps = nullptr;
   kern<<<dim3(static_cast<unsigned>(p.nbx * p.nby * p.nsplit)), dim3(64 * WM * WN), lds, stream>>>(p);
   if (p.nsplit > 1) {
     const int64_t total = ml.rows * N;
@@ -1994,6 +2046,39 @@ void launch_probe(const void* ops, int wgs, int iters, float* out, hipStream_t s
 }
 
 }  // namespace
+
+// The prefill GEMM's 256 x 256 int8 per-channel bf16 launch with cycle stamps
+// (M and N multiples of 256, K a multiple of 64 and at least 192): out [M, N]
+// bf16, stamps [(M / 256) * (N / 256)][8 wavefronts][8] counts.
+int launch_prefill_phases(const void* x, const void* codes, const void* scale, int64_t M, int64_t K, int64_t N,
+                          void* out, unsigned long long* stamps, hipStream_t stream) {
+  constexpr int WM = 2, WN = 4, TM = 4, TN = 2, STAGES = 3;
+  constexpr size_t lds = dma_lds_bytes<8, 0, WM, WN, TM, TN, STAGES>();
+  auto kern = gemm_dma_kernel<WOL_DTYPE_BF16, 8, 0, 0, WM, WN, TM, TN, STAGES, 0, false, true>;
+  static std::atomic<uint32_t> configured{0};
+  allow_lds(reinterpret_cast<const void*>(kern), lds, configured);
+  DmaParams p;
+  p.x = static_cast<const uint16_t*>(x);
+  p.codes = static_cast<const uint8_t*>(codes);
+  p.bias = nullptr;
+  p.scale = static_cast<const uint16_t*>(scale);
+  p.out = out;
+  p.M = static_cast<int>(M); p.K = static_cast<int>(K); p.N = static_cast<int>(N);
+  p.out_f32 = 0;
+  p.strip_lo = 0; p.strip_hi = static_cast<int>(N / kStripCols);
+  p.nbx = static_cast<int>(N / 256);
+  p.nby = static_cast<int>(M / 256);
+  p.tiles_per_split = static_cast<int>(K / 64);
+  p.nsplit = 1;
+  p.xcd_rows = plan_xcd_rows(p.nbx, p.nby, 256 * 2, 256);
+  p.act = WOL_ACT_NONE;
+  p.moe_table = nullptr;
+  p.moe_codes_stride = 0;
+  p.moe_rows = 0;
+  p.stamps = stamps;
+  kern<<<dim3(static_cast<unsigned>(p.nbx * p.nby)), dim3(64 * WM * WN), lds, stream>>>(p);
+  return check_launch();
+}
 
 int launch_mfma_probe(int variant, const void* ops, int workgroups, int iters, float* out, hipStream_t stream) {
   switch (variant) {

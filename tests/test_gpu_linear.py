@@ -694,6 +694,38 @@ def test_mfma_probe_variants_run(device):
         assert bool(torch.isfinite(out).all()), v
 
 
+def test_prefill_phases_counts_and_output(device):
+    # the cycle-stamped instantiation of the prefill GEMM: its output is the
+    # product's bit for bit, and every wavefront's counts add up (the phases
+    # between entry and end sum to the total, the k-tile count is K / 64)
+    import torch
+    from paddle_amd import _lib
+    from paddle_amd.nn import quant as Q
+
+    import ctypes
+
+    M, K, N = 2048, 256, 8192  # 256 tiles of 256 x 256: what wol_linear launches for this shape, in one piece
+    plan = ctypes.create_string_buffer(256)
+    _lib.check(_lib.lib.wol_linear_plan(M, K, N, 8, -1, 0, plan, 256))
+    assert plan.value.endswith(b"256x256 tiles on columns [0,8192)"), plan.value
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    w = (torch.randn(K, N, device="cuda", generator=gen) * 0.02).to(torch.bfloat16)
+    x = torch.randn(M, K, device="cuda", generator=gen).to(torch.bfloat16)
+    codes, scale = Q.weight_quantize(w, algo="weight_only_int8")
+    want = Q.weight_only_linear(x, codes, None, scale, "int8")
+    out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    wgs = (M // 256) * (N // 256)
+    ph = torch.zeros(wgs * 64, dtype=torch.int64, device="cuda")
+    _lib.check(_lib.lib.wol_prefill_phases(x.data_ptr(), codes.data_ptr(), scale.data_ptr(), M, K, N, out.data_ptr(),
+                                           ph.data_ptr(), ph.numel() * 8, None))
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
+    c = ph.cpu().numpy().reshape(wgs * 8, 8)
+    assert (c[:, 7] == K // 64).all()
+    assert (c[:, :7] > 0).all() and (c[:, 6] < 10 ** 9).all()
+    assert (c[:, 0:6].sum(axis=1) == c[:, 6]).all()
+
+
 def test_read_floor_reads_every_byte_once(device):
     # the measurement aid behind bench.py's read_floor: each wavefront XORs the
     # dwords of its eighth of a strip

@@ -250,6 +250,21 @@ def test_mfma_probe_argument_errors(lib):
     assert L.wol_mfma_probe(5, p, need - 1, 1, 1, p, None) == 8  # too few operand bytes for the variants that load
 
 
+def test_prefill_phases_argument_errors(lib):
+    L = lib.lib
+    p = ctypes.c_void_p(0x1000)
+    big = 1 << 30
+    assert L.wol_prefill_phases(p, p, p, 256, 4096, 256, p, p, big, None) not in (1, 5, 8, 9)  # valid: fails only for want of a device
+    assert L.wol_prefill_phases(p, p, p, 255, 4096, 256, p, p, big, None) == 5
+    assert L.wol_prefill_phases(p, p, p, 256, 4096, 128, p, p, big, None) == 5
+    assert L.wol_prefill_phases(p, p, p, 256, 128, 256, p, p, big, None) == 5   # fewer k tiles than stages
+    assert L.wol_prefill_phases(p, p, p, 256, 4100, 256, p, p, big, None) == 5
+    assert L.wol_prefill_phases(p, None, p, 256, 4096, 256, p, p, big, None) == 1
+    assert L.wol_prefill_phases(p, p, p, 256, 4096, 256, p, None, big, None) == 1
+    assert L.wol_prefill_phases(ctypes.c_void_p(0x1004), p, p, 256, 4096, 256, p, p, big, None) == 9
+    assert L.wol_prefill_phases(p, p, p, 512, 4096, 512, p, p, 4 * 64 * 8 - 1, None) == 8
+
+
 def test_linear_plan_names_the_kernel_per_shape(lib):
     # wol_linear's choice between its three kernels, as the library reports it
     # (no device work): one row streams a workgroup per strip; 2 and 5..16 rows
