@@ -706,11 +706,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
   constexpr int kValuPerMfma = ((OFFS == 2 ? 4 * TN + 4 * TM : (BITS == 8 ? 16 : 12) * TN) + TM * TN - 1) / (TM * TN) + 2;
   constexpr int kValuRescale = RESC ? 16 : 0;  // more per MFMA in the slice that starts a group
   constexpr int kHalf = (TM * TN + 1) / 2;  // MFMAs of a slice issued before the barrier
-  // The largest tile (one workgroup per CU, wavefronts w and w + 4 on one SIMD): left alone the older
-  // wavefront of a SIMD wins every arbitration, finishes a k tile in two thirds of the tile's time and
-  // waits out the rest at the barrier (cycle stamps: 1864 against 2634 cycles of work per tile, 888
-  // against 114 at the barrier).  Taking turns evens that out; it is worth 1.5 to 2 %.
-  constexpr bool kTakeTurns = NW == 8 && TM * TN == 8;
+  // (With one workgroup per CU, wavefronts w and w + 4 share a SIMD and the older one wins every
+  // arbitration: it finishes a k tile in two thirds of the tile's time and waits out the rest at the
+  // barrier.  Handing the priority back and forth with s_setprio evens their arrival out and makes the
+  // kernel 3 % slower: the tile's period follows the sum of their work, and the switches add to it.)
 
   // The wavefront's pipeline registers: raw codes of the current and the next
   // tile, and two sets of operands -- the one the MFMAs of slice q use and the
@@ -835,11 +834,6 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_dma_kernel(const DmaParams 
     read_scales(stage, sraw);  // before the stage is handed over
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
-      if (kTakeTurns) {
-        // slice by slice the two wavefronts of a SIMD take turns at the higher priority
-        if ((wave >> 2) == (q & 1)) __builtin_amdgcn_s_setprio(1);
-        else __builtin_amdgcn_s_setprio(0);
-      }
       if (q != Q - 2) {
         const bool last = q == Q - 1;
         // this slice's share of the tile loads (segment 1 of tile it+3, or segment q+2 of tile it+2)
