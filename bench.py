@@ -385,6 +385,67 @@ def bench_prefill_phases(torch, np, Q, _lib, dev):
                     "their 2 x 32 MFMAs of 32 cycles back to back", "rows": rows}
 
 
+def bench_decode_phases(torch, np, Q, _lib, dev, c, x, copies, scales, steps):
+    """wol_decode_phases: the headline decode kernel on an instantiation that reads
+    the clocks as it goes, launched as the headline figure launches the product
+    kernel (`steps` launches in one graph, each on the next copy of the weights,
+    the copies together several times the Infinity Cache).  Four consecutive
+    launches in the middle of the graph stamp into phases of their own, so that
+    the device's constant-rate clock (100 MHz) places every wavefront of theirs
+    on one time line: how long after a launch's first wavefront its last one
+    enters, how long after it the last one ends (the span in which the weights
+    are read), and how long the device then takes until the next launch's first
+    wavefront starts.  The shader-cycle stamps split a wavefront's life into
+    its phases."""
+    K, N, g = c["K"], c["N"], c["group_size"]
+    out = torch.empty((1, N), dtype=torch.bfloat16, device=dev)
+    wgs, L = N // 16, 4
+    first = max(0, steps // 2 - L // 2)
+    ph = [torch.zeros(wgs * 64, dtype=torch.int64, device=dev) for _ in range(L + 1)]  # the last one takes all other launches'
+
+    def stamped(i):
+        j = i % len(copies)
+        p_ = ph[i - first] if first <= i < first + L else ph[L]
+        _lib.check(_lib.lib.wol_decode_phases(x.data_ptr(), copies[j].data_ptr(), scales[j].data_ptr(), K, N, g, out.data_ptr(),
+                                              p_.data_ptr(), p_.numel() * 8, torch.cuda.current_stream().cuda_stream))
+
+    t_st, _ = time_graph(torch, stamped, steps, warm_launches=400)
+    torch.cuda.synchronize()
+    cs = [p_.cpu().numpy().reshape(wgs * 8, 8).astype(np.float64) for p_ in ph[:L]]
+    tick_us = 0.01
+    enter = [float((c_[:, 0].max() - c_[:, 0].min()) * tick_us) for c_ in cs]
+    span = [float((c_[:, 1].max() - c_[:, 0].min()) * tick_us) for c_ in cs]
+    gap = [float((cs[i + 1][:, 0].min() - cs[i][:, 1].max()) * tick_us) for i in range(L - 1)]
+    period = [float((cs[i + 1][:, 0].min() - cs[i][:, 0].min()) * tick_us) for i in range(L - 1)]
+    allc = np.concatenate(cs)
+    mean = allc.mean(axis=0)
+    bytes_read = K * N // 2  # the codes alone, as the headline figure counts
+    span_us = statistics.median(span)
+    names = ("arguments", "issue_loads", "wait_loads", "compute", "wait_barrier", "epilogue")
+    life = allc[:, 2:8].sum(axis=1)
+    ghz = float(life.mean() / ((allc[:, 1] - allc[:, 0]) * tick_us).mean() / 1e3)
+    # when a wavefront's last load has landed, on the launch's own time line
+    landed = [(c_[:, 0] - c_[:, 0].min()) * tick_us + c_[:, 2:5].sum(axis=1) / (ghz * 1e3) for c_ in cs]
+    return {
+        "what": "wol_decode_phases: clock stamps per wavefront of the headline decode kernel (bf16, int4 group %d, "
+                "M=1, K=%d, N=%d); %d launches in one graph on %d weight copies, %d consecutive ones stamped into phases "
+                "of their own" % (g, K, N, steps, len(copies), L),
+        "workgroups": wgs, "stamped_us": round(t_st / steps * 1e6, 3),
+        "last_wavefront_enters_after_us": round(statistics.median(enter), 2),
+        "first_entry_to_last_end_us": round(span_us, 2),
+        "last_end_to_next_launch_first_entry_us": round(statistics.median(gap), 2),
+        "first_entry_to_next_first_entry_us": round(statistics.median(period), 2),
+        "hbm_frac_within_span": round(bytes_read / (span_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+        "wavefront_life_us": round(float(((allc[:, 1] - allc[:, 0]) * tick_us).mean()), 2),
+        "shader_clock_ghz": round(ghz, 3),
+        "loads_landed_after_us": {"first_wavefront": round(statistics.median(float(l.min()) for l in landed), 2),
+                                  "median_wavefront": round(statistics.median(float(np.median(l)) for l in landed), 2),
+                                  "last_wavefront": round(statistics.median(float(l.max()) for l in landed), 2)},
+        "cycles": {n: round(float(mean[2 + i]), 0) for i, n in enumerate(names)},
+        "share_of_life": {n: round(float(mean[2 + i] / life.mean()), 4) for i, n in enumerate(names)},
+    }
+
+
 def bench_moe_ffn(torch, np, Q, H, dev, quick, failures):
     """moe_ffn on weight-only int8 experts of Mixtral-8x7B's size (8 experts,
     hidden 4096, fc1 width 2 x 14336 for swiglu, bf16): a prefill-like call
@@ -732,8 +793,10 @@ def main():
         }
 
     # ---------------- every BASELINE configuration ----------------
-    configs = stack = grad = moe = fused = phases = None
+    configs = stack = grad = moe = fused = phases = dphases = None
     if not args.no_configs:
+        if c["K"] == 4096 and c["bits"] == 4 and c["group_size"] in (64, 128) and not args.eager:
+            dphases = bench_decode_phases(torch, np, Q, _lib, dev, c, x, copies, scales, args.steps)
         del copies, scales
         torch.cuda.empty_cache()
         configs = bench_configs(torch, Q, _lib, dev, args.quick)
@@ -877,6 +940,7 @@ def main():
         "moe_ffn": moe,
         "fused_swiglu": fused,
         "prefill_phases": phases,
+        "decode_phases": dphases,
         "llm_int8": llm,
         "cpu_baseline": cpu,
         "parity": parity,
@@ -902,6 +966,9 @@ def main():
         for r in phases["rows"]:
             for k, v in r["share_of_total"].items():
                 flat["prefill_phase_M%d_%s_share" % (r["M"], k)] = v
+    if dphases:
+        for k in ("first_entry_to_last_end_us", "last_end_to_next_launch_first_entry_us", "hbm_frac_within_span"):
+            flat["decode_phase_" + k] = dphases[k]
     if llm:
         flat["llm_int8_frac"] = llm["roofline"]["frac"]
     for nm, tf in (ladder or {}).items():

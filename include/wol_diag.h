@@ -72,6 +72,31 @@ int wol_mfma_probe(int variant, const void* operands, size_t operand_bytes,
                    int workgroups, int iters, float* out, void* stream);
 
 /*
+ * Where the wavefronts of the decode GEMV spend their time: runs the kernel
+ * wol_linear takes for one row of bf16 activations on int4 codes with
+ * group-wise scales at K = 4096 (the benchmark's headline shape: a workgroup
+ * of 8 wavefronts per 16-column strip, every load of a wavefront issued at
+ * once) on an instantiation that reads the clocks as it goes.  out: [1, N]
+ * bf16, bit for bit what wol_linear writes.  phases: for workgroup w (of
+ * N / 16) and wavefront v (of 8), eight 64-bit values at
+ * phases[(w * 8 + v) * 8 ...]:
+ *   0  entry, 1  end: the constant-rate clock (100 MHz, common to the device)
+ *   2  entry until the kernel's arguments are in registers, shader cycles
+ *   3  addresses, every load issued
+ *   4  waiting until every load has landed (an explicit wait the product
+ *      kernel does not have: it starts on the first tile as it arrives)
+ *   5  dequantisation, MFMAs, folding, partial sums into LDS
+ *   6  waiting at the workgroup barrier
+ *   7  adding the wavefronts' sums, scale, store
+ * Values 2 to 7 add up to the wavefront's life in shader cycles.
+ */
+#define WOL_DECODE_PHASES_PER_WORKGROUP 64 /* values: 8 wavefronts x 8 */
+int wol_decode_phases(const void* x, const void* codes, const void* scale,
+                      int64_t K, int64_t N, int group_size, void* out,
+                      unsigned long long* phases, size_t phases_bytes,
+                      void* stream);
+
+/*
  * Where the wavefronts of the prefill GEMM spend their cycles: runs the
  * 256 x 256 launch of wol_linear (bf16 activations, int8 codes with
  * per-channel scales, GFX950 layout; M and N multiples of 256, K a multiple

@@ -42,6 +42,7 @@ SYMBOLS = (
     "wol_mfma_ceiling",
     "wol_mfma_probe",
     "wol_prefill_phases",
+    "wol_decode_phases",
     "wol_linear_plan",
     "wol_linear_grad_plan",
     "wol_llm_int8_linear_workspace",
@@ -116,6 +117,8 @@ def _load():
     lib.wol_mfma_probe.restype = ci
     lib.wol_prefill_phases.argtypes = [vp, vp, vp, i64, i64, i64, vp, vp, sz, vp]
     lib.wol_prefill_phases.restype = ci
+    lib.wol_decode_phases.argtypes = [vp, vp, vp, i64, i64, ci, vp, vp, sz, vp]
+    lib.wol_decode_phases.restype = ci
     lib.wol_linear_plan.argtypes = [i64, i64, i64, ci, ci, sz, ctypes.c_char_p, sz]
     lib.wol_linear_plan.restype = ci
     lib.wol_linear_grad_plan.argtypes = [i64, i64, i64, ctypes.c_char_p, sz]

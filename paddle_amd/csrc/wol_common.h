@@ -312,6 +312,10 @@ int launch_linear_grad(const void* out_grad, const void* codes, const void* scal
 int launch_read_floor(const void* codes, int64_t K, int64_t N, int bits, void* out,
                       hipStream_t stream);
 int launch_mfma_probe(int variant, const void* ops, int workgroups, int iters, float* out, hipStream_t stream);
+// The headline decode kernel (bf16, int4 with group-wise scales, one row, K = 4096) with clock stamps per wavefront
+// (wol_decode_phases).
+int launch_decode_phases(const void* x, const void* codes, const void* scale, int64_t K, int64_t N, int group_size,
+                         void* out, unsigned long long* stamps, hipStream_t stream);
 // The prefill GEMM's 256 x 256 launch (int8 per-channel, bf16) with cycle stamps per wavefront (wol_prefill_phases).
 int launch_prefill_phases(const void* x, const void* codes, const void* scale, int64_t M, int64_t K, int64_t N,
                           void* out, unsigned long long* stamps, hipStream_t stream);

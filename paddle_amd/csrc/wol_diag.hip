@@ -113,6 +113,18 @@ int wol_mfma_ceiling(const void* operands, int workgroups, int iters, float* out
   return wol::launch_mfma_ceiling(operands, workgroups, iters, out, static_cast<hipStream_t>(stream));
 }
 
+int wol_decode_phases(const void* x, const void* codes, const void* scale, int64_t K, int64_t N, int group_size,
+                      void* out, unsigned long long* phases, size_t phases_bytes, void* stream) {
+  if (K != 4096 || N <= 0 || N % 16 != 0 || N > (1 << 24) || (group_size != 64 && group_size != 128))
+    return WOL_ERR_BAD_SHAPE;
+  if (x == nullptr || codes == nullptr || scale == nullptr || out == nullptr || phases == nullptr) return WOL_ERR_NULL_POINTER;
+  if (((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(codes) | reinterpret_cast<uintptr_t>(scale) |
+        reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(phases)) & 15u) != 0)
+    return WOL_ERR_ALIGNMENT;
+  if (phases_bytes < static_cast<size_t>(N / 16) * WOL_DECODE_PHASES_PER_WORKGROUP * 8) return WOL_ERR_WORKSPACE;
+  return wol::launch_decode_phases(x, codes, scale, K, N, group_size, out, phases, static_cast<hipStream_t>(stream));
+}
+
 int wol_prefill_phases(const void* x, const void* codes, const void* scale, int64_t M, int64_t K, int64_t N,
                        void* out, unsigned long long* phases, size_t phases_bytes, void* stream) {
   if (M <= 0 || N <= 0 || M % 256 != 0 || N % 256 != 0 || K % 64 != 0 || K < 192 || M > (1 << 20) || N > (1 << 20) ||

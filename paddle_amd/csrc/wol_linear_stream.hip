@@ -72,6 +72,20 @@ __device__ inline float sum_lane_groups(float v, bool x16, bool x32) {
   return v;
 }
 
+// Which block of strips a workgroup takes.  Workgroups are dealt to the 8 XCDs
+// round-robin by their linear id, and every XCD has an L2 of its own.  Four
+// neighbouring strips share each 128-byte line of the scales, the bias and the
+// output (16 columns of 2 bytes per strip): in linear order the four would sit
+// on four XCDs and each L2 would fetch the line for itself, four times the
+// scales' bytes from HBM.  Every round of 32 workgroups therefore takes 32
+// consecutive blocks with four neighbours per XCD; what is left over after the
+// last whole round keeps the linear order.
+__device__ inline int block_of_workgroup(int b, int nblocks) {
+  if (b >= (nblocks & ~31)) return b;
+  const int r = b & 31;
+  return (b & ~31) + (r & 7) * 4 + (r >> 3);
+}
+
 // NU > 0: every wavefront owns exactly NU units and issues all their loads at
 // once (the whole problem is in flight from the first cycle; used when K is
 // small enough).  NU == 0: a wavefront walks its share of the units with the
@@ -92,7 +106,13 @@ __device__ inline float sum_lane_groups(float v, bool x16, bool x32) {
 // works on gate strip b, the second half on up strip b + N/32, each half
 // splitting K as a whole workgroup does otherwise; the two sums of an output
 // element meet in the epilogue, which is the only place that differs.
-template <int DT, int BITS, int MP, int MT, int WK, int NU, int TN, bool GROUPED, bool PRE, bool SWI>
+//
+// STAMP (a diagnostic instantiation, never on a product path; NU > 0 only):
+// every wavefront reads the clocks at entry, once its loads are issued, once
+// they have all landed (an explicit wait the product kernel does not have),
+// after its arithmetic, after the workgroup's barrier and at the end, and
+// leaves them in `stamps` (wol_decode_phases).
+template <int DT, int BITS, int MP, int MT, int WK, int NU, int TN, bool GROUPED, bool PRE, bool SWI, bool STAMP = false>
 struct StreamKernel {
   static_assert(MT == 1 || MP == 16, "several M tiles only with full 16-row operands");
   static_assert(!SWI || (TN == 1 && MT == 1 && WK >= 2), "the gate|up form pairs two single strips");
@@ -124,6 +144,7 @@ struct StreamKernel {
   const uint16_t* x;
   const uint16_t* scale;
   const uint16_t* pre;  // [K] per-channel scales of the activations (PRE)
+  unsigned long long* stamps = nullptr;  // STAMP: [workgroup][wavefront][8]
   int act;              // WOL_ACT_NONE or WOL_ACT_GELU
   int M, K, N;
   int gshift;  // log2(group_size) when GROUPED
@@ -316,16 +337,22 @@ struct StreamKernel {
 
   __device__ inline void run(const uint8_t* codes, const uint16_t* bias, void* out, int out_f32,
                              float* red) {
+    unsigned long long st_rt0 = 0, st_c0 = 0, st_ca = 0, st_c1 = 0, st_c2 = 0, st_c3 = 0, st_c4 = 0;
+    if (STAMP) {
+      st_rt0 = __builtin_amdgcn_s_memrealtime();
+      st_c0 = __builtin_readcyclecounter();
+    }
     lane = threadIdx.x & 63;
     const int wave_all = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wave = SWI ? wave_all % kWS : wave_all;  // its place among the wavefronts of its strip
     j = lane & 15;
     kb = lane >> 4;
     const int nstrips = N / kStripCols;
+    const int bid = block_of_workgroup(static_cast<int>(blockIdx.x), static_cast<int>(gridDim.x));
     const uint8_t* strip[TN];
 #pragma unroll
     for (int t = 0; t < TN; ++t) {
-      int tn = blockIdx.x * TN + t;
+      int tn = bid * TN + t;
       if (SWI) tn += (wave_all / kWS) * (nstrips / 2);  // the up strip of the same output columns
       tn = tn < nstrips ? tn : nstrips - 1;  // a strip past the end repeats the last one and is not stored
       n[t] = tn * kStripCols + j;
@@ -333,6 +360,10 @@ struct StreamKernel {
     }
     magic = Dequant<DT, BITS>::kMagic;
     asm volatile("" : "+v"(magic));  // keep the constant in a VGPR
+    if (STAMP) {
+      asm volatile("" ::"s"(strip[0]), "s"(scale), "s"(x));  // the kernel's arguments have arrived
+      st_ca = __builtin_readcyclecounter();
+    }
     const int nsteps = K / 32;
     vsteps = BITS == 4 ? (K / 128) * 4 : nsteps;
     const int nunits = (NU > 0 ? nsteps : vsteps) / kU;  // whole units
@@ -352,9 +383,14 @@ struct StreamKernel {
     const u32x4* tp[TN];
 #pragma unroll
     for (int t = 0; t < kEp; ++t) {
-      const int col = SWI ? static_cast<int>(blockIdx.x) * kStripCols + j + t * (N / 2) : n[t];
-      ep_sraw[t] = scale[col];
-      ep_braw[t] = (bias != nullptr ? bias : scale)[col];  // one unconditional load
+      const int col = SWI ? bid * kStripCols + j + t * (N / 2) : n[t];
+      // group-wise scales have been applied step by step; and most linears
+      // of a decoder carry no bias: neither load is issued then (a load of two
+      // bytes per lane occupies the CU's memory pipeline like any other)
+      ep_sraw[t] = 0;
+      ep_braw[t] = 0;
+      if (!GROUPED) ep_sraw[t] = scale[col];
+      if (bias != nullptr) ep_braw[t] = bias[col];
     }
 #pragma unroll
     for (int t = 0; t < TN; ++t) tp[t] = reinterpret_cast<const u32x4*>(strip[t]) + lane;
@@ -363,6 +399,12 @@ struct StreamKernel {
 #pragma unroll
       for (int i = 0; i < NU; ++i) load_unit(d[i], tp, wave * NU + i);
       __builtin_amdgcn_sched_barrier(0);  // every load is in flight before the first wait
+      if (STAMP) {
+        st_c1 = __builtin_readcyclecounter();
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): every load has landed
+        st_c2 = __builtin_readcyclecounter();
+        __builtin_amdgcn_sched_barrier(0);
+      }
 #pragma unroll
       for (int i = 0; i < NU; ++i) compute_unit(d[i]);
     } else {
@@ -479,7 +521,23 @@ struct StreamKernel {
         for (int r = 0; r < kLive; ++r)
           red[(((t * WK + wave_all) * MT + mt) * 4 + r) * 64 + lane] = tot[mt][r];
     }
+    if (STAMP) st_c3 = __builtin_readcyclecounter();
     __syncthreads();
+    if (STAMP) st_c4 = __builtin_readcyclecounter();
+    auto leave_stamps = [&]() {
+      if (STAMP && lane == 0 && stamps != nullptr) {
+        unsigned long long* o = stamps + (static_cast<size_t>(blockIdx.x) * WK + wave_all) * 8;
+        const unsigned long long c5 = __builtin_readcyclecounter();
+        o[0] = st_rt0;                             // entry, constant-rate clock (100 MHz)
+        o[1] = __builtin_amdgcn_s_memrealtime();   // end, the same clock
+        o[2] = st_ca - st_c0;                      // entry until the kernel's arguments are in registers
+        o[3] = st_c1 - st_ca;                      // addresses, every load issued
+        o[4] = st_c2 - st_c1;                      // waiting for the loads
+        o[5] = st_c3 - st_c2;                      // dequantisation, MFMAs, folding, sums into LDS
+        o[6] = st_c4 - st_c3;                      // waiting for the workgroup's other wavefronts
+        o[7] = c5 - st_c4;                         // adding the wavefronts' sums, scale, store
+      }
+    };
     const int rows = M < 16 * MT ? M : 16 * MT;
     if (SWI) {
       float ep_scale[2], ep_bias[2];
@@ -499,7 +557,7 @@ struct StreamKernel {
           v[h] = s * ep_scale[h] + ep_bias[h];
         }
         const float s = act_swiglu(v[0], v[1]);
-        const int64_t o = static_cast<int64_t>(m) * (N / 2) + static_cast<int>(blockIdx.x) * kStripCols + nl;
+        const int64_t o = static_cast<int64_t>(m) * (N / 2) + bid * kStripCols + nl;
         if (out_f32)
           static_cast<float*>(out)[o] = s;
         else
@@ -509,7 +567,7 @@ struct StreamKernel {
     }
 #pragma unroll
     for (int t = 0; t < TN; ++t) {
-      if (static_cast<int>(blockIdx.x) * TN + t >= nstrips) break;  // the repeated last strip
+      if (bid * TN + t >= nstrips) break;  // the repeated last strip
       const float ep_scale = GROUPED ? 1.0f : to_f32<DT>(ep_sraw[t]);
       const float ep_bias = bias != nullptr ? to_f32<DT>(ep_braw[t]) : 0.0f;
       for (int idx = threadIdx.x; idx < rows * 16; idx += WK * 64) {
@@ -527,6 +585,7 @@ struct StreamKernel {
           static_cast<uint16_t*>(out)[o] = cast_out<DT>(s);
       }
     }
+    leave_stamps();
   }
 };
 
@@ -549,6 +608,25 @@ __global__ __launch_bounds__(WK * 64) void stream_kernel(
 }
 
 using Args = StreamArgs;
+
+// The headline decode kernel (one row, int4, group-wise scales, 8 wavefronts, one unit each) with stamps.
+template <int DT>
+__global__ __launch_bounds__(512) void stream_phases_kernel(
+    const uint16_t* __restrict__ x, const uint8_t* __restrict__ codes, const uint16_t* __restrict__ scale,
+    void* __restrict__ out, int K, int N, int gshift, unsigned long long* __restrict__ stamps) {
+  extern __shared__ float red[];
+  StreamKernel<DT, 4, 1, 1, 8, 1, 1, true, false, false, true> k;
+  k.x = x;
+  k.scale = scale;
+  k.pre = nullptr;
+  k.stamps = stamps;
+  k.act = WOL_ACT_NONE;
+  k.M = 1;
+  k.K = K;
+  k.N = N;
+  k.gshift = gshift;
+  k.run(codes, nullptr, out, 0, red);
+}
 
 template <int DT, int BITS, int MP, int MT, int WK, int NU, int TN, bool SWI = false>
 void launch_tn(const Args& a) {
@@ -664,6 +742,21 @@ void launch_m(const Args& a, int wk, int nu) {
 }
 
 }  // namespace
+
+#if !defined(WOL_STREAM_F16_TU)
+// bf16 activations, int4 codes with group-wise scales, K = 4096 (eight wavefronts with one unit of 512 k
+// each, every load issued at once: the kernel wol_linear takes for the benchmark's headline shape).
+int launch_decode_phases(const void* x, const void* codes, const void* scale, int64_t K, int64_t N, int group_size,
+                         void* out, unsigned long long* stamps, hipStream_t stream) {
+  if (K != 4096 || (group_size != 64 && group_size != 128) || N % kStripCols != 0) return WOL_ERR_BAD_SHAPE;
+  const dim3 grid(static_cast<unsigned>(N / kStripCols)), block(512);
+  const size_t lds = static_cast<size_t>(8) * 256 * sizeof(float);
+  stream_phases_kernel<WOL_DTYPE_BF16><<<grid, block, lds, stream>>>(
+      static_cast<const uint16_t*>(x), static_cast<const uint8_t*>(codes), static_cast<const uint16_t*>(scale), out,
+      static_cast<int>(K), static_cast<int>(N), group_size == 64 ? 6 : 7, stamps);
+  return check_launch();
+}
+#endif
 
 #if defined(WOL_STREAM_F16_TU)
 void launch_linear_stream_f16(const StreamArgs& a, int bits, bool swi, int wk, int nu) {

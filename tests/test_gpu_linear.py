@@ -694,6 +694,36 @@ def test_mfma_probe_variants_run(device):
         assert bool(torch.isfinite(out).all()), v
 
 
+def test_decode_phases_counts_and_output(device):
+    # the clock-stamped instantiation of the headline decode kernel: its output
+    # is the product's bit for bit and every wavefront's phases add up
+    import torch
+    from paddle_amd import _lib
+    from paddle_amd.nn import quant as Q
+
+    K, N = 4096, 1024
+    gen = torch.Generator(device="cuda").manual_seed(6)
+    w = (torch.randn(K, N, device="cuda", generator=gen) * 0.02).to(torch.bfloat16)
+    x = torch.randn(1, K, device="cuda", generator=gen).to(torch.bfloat16)
+    for g in (64, 128):
+        codes, scale = Q.weight_quantize(w, algo="weight_only_int4", group_size=g)
+        want = Q.weight_only_linear(x, codes, None, scale, "int4", None, g)
+        out = torch.full((1, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+        ph = torch.zeros(N // 16 * 64, dtype=torch.int64, device="cuda")
+        _lib.check(_lib.lib.wol_decode_phases(x.data_ptr(), codes.data_ptr(), scale.data_ptr(), K, N, g, out.data_ptr(),
+                                              ph.data_ptr(), ph.numel() * 8, None))
+        torch.cuda.synchronize()
+        assert torch.equal(out, want)
+        c = ph.cpu().numpy().reshape(-1, 8)
+        assert (c[:, 1] >= c[:, 0]).all() and (c[:, 2:8] > 0).all() and (c[:, 2:8].sum(axis=1) < 10 ** 8).all()
+        # the device's 100 MHz clock and the shader cycles tell the same story: 0.5 to 3 GHz
+        life_us = (c[:, 1] - c[:, 0]) * 0.01
+        long_ = life_us > 1.0
+        if long_.any():
+            ghz = c[long_, 2:8].sum(axis=1) / life_us[long_] / 1e3
+            assert 0.5 < ghz.mean() < 3.0
+
+
 def test_prefill_phases_counts_and_output(device):
     # the cycle-stamped instantiation of the prefill GEMM: its output is the
     # product's bit for bit, and every wavefront's counts add up (the phases

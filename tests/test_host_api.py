@@ -250,6 +250,19 @@ def test_mfma_probe_argument_errors(lib):
     assert L.wol_mfma_probe(5, p, need - 1, 1, 1, p, None) == 8  # too few operand bytes for the variants that load
 
 
+def test_decode_phases_argument_errors(lib):
+    L = lib.lib
+    p = ctypes.c_void_p(0x1000)
+    big = 1 << 30
+    assert L.wol_decode_phases(p, p, p, 4096, 11008, 128, p, p, big, None) not in (1, 5, 8, 9)  # valid: fails only for want of a device
+    assert L.wol_decode_phases(p, p, p, 8192, 11008, 128, p, p, big, None) == 5   # built for K = 4096
+    assert L.wol_decode_phases(p, p, p, 4096, 11000, 128, p, p, big, None) == 5
+    assert L.wol_decode_phases(p, p, p, 4096, 11008, -1, p, p, big, None) == 5    # group-wise scales only
+    assert L.wol_decode_phases(p, p, None, 4096, 11008, 128, p, p, big, None) == 1
+    assert L.wol_decode_phases(p, p, p, 4096, 11008, 128, ctypes.c_void_p(0x1002), p, big, None) == 9
+    assert L.wol_decode_phases(p, p, p, 4096, 11008, 128, p, p, 688 * 64 * 8 - 1, None) == 8
+
+
 def test_prefill_phases_argument_errors(lib):
     L = lib.lib
     p = ctypes.c_void_p(0x1000)
