@@ -441,9 +441,46 @@ def bench_decode_phases(torch, np, Q, _lib, dev, c, x, copies, scales, steps):
         "loads_landed_after_us": {"first_wavefront": round(statistics.median(float(l.min()) for l in landed), 2),
                                   "median_wavefront": round(statistics.median(float(np.median(l)) for l in landed), 2),
                                   "last_wavefront": round(statistics.median(float(l.max()) for l in landed), 2)},
+        # workgroups in the order they were dealt out, 256 (one per CU) to a round: when a round's workgroups have their data
+        "last_load_landed_by_round_of_256_us": [
+            round(statistics.median(float(l.reshape(wgs, 8).max(axis=1)[r0:r0 + 256].mean()) for l in landed), 2)
+            for r0 in range(0, wgs, 256)],
         "cycles": {n: round(float(mean[2 + i]), 0) for i, n in enumerate(names)},
         "share_of_life": {n: round(float(mean[2 + i] / life.mean()), 4) for i, n in enumerate(names)},
     }
+
+
+def bench_decode_rounds(torch, Q, _lib, dev, c, steps):
+    """The headline decode call and the pure read of the same bytes over the number
+    of strips (K, bits and group size of the headline; N from one workgroup per CU
+    to five): a launch costs a fixed part plus a part per round of 256 workgroups."""
+    K, g, bits = c["K"], c["group_size"], c["bits"]
+    wd = "int8" if bits == 8 else "int4"
+    rows = []
+    for N in (4096, 8192, 10240, 11008, 12288, 14336, 16384, 20480):
+        codes, scale = _quantize(Q, _device_weight(torch, K, N, torch.bfloat16, 950, dev), bits, g)
+        wbytes = K * N * bits // 8
+        ncopies = max(2, -(-768 * 1024 * 1024 // wbytes))
+        copies = [codes.clone() for _ in range(ncopies)]
+        scales = [scale.clone() for _ in range(ncopies)]
+        x = torch.randn((1, K), device=dev, dtype=torch.float32).to(torch.bfloat16)
+        floor_out = torch.empty(N // 16 * 8, dtype=torch.int32, device=dev)
+
+        def call(i):
+            return Q.weight_only_linear(x, copies[i % ncopies], None, scales[i % ncopies], wd, None, g)
+
+        def floor(i):
+            _lib.check(_lib.lib.wol_read_floor(copies[i % ncopies].data_ptr(), K, N, bits, floor_out.data_ptr(),
+                                               torch.cuda.current_stream().cuda_stream))
+
+        t_c, _ = time_graph(torch, call, steps, warm_launches=400)
+        t_f, _ = time_graph(torch, floor, steps, warm_launches=400)
+        rows.append({"N": N, "strips": N // 16, "rounds_of_256": round(N / 16 / 256, 2),
+                     "linear_us": round(t_c / steps * 1e6, 3), "read_floor_us": round(t_f / steps * 1e6, 3)})
+        del copies, scales
+        torch.cuda.empty_cache()
+    return {"what": "wol_linear (M=1, int%d g%d, K=%d, bf16) and wol_read_floor over N: one workgroup per 16-column strip, "
+                    "256 CUs" % (bits, g, K), "rows": rows}
 
 
 def bench_moe_ffn(torch, np, Q, H, dev, quick, failures):
@@ -793,9 +830,9 @@ def main():
         }
 
     # ---------------- every BASELINE configuration ----------------
-    configs = stack = grad = moe = fused = phases = dphases = None
+    configs = stack = grad = moe = fused = phases = dphases = drounds = None
     if not args.no_configs:
-        if c["K"] == 4096 and c["bits"] == 4 and c["group_size"] in (64, 128) and not args.eager:
+        if c["K"] == 4096 and c["bits"] == 4 and c["group_size"] in (64, 128) and not args.eager and args.steps >= 8:
             dphases = bench_decode_phases(torch, np, Q, _lib, dev, c, x, copies, scales, args.steps)
         del copies, scales
         torch.cuda.empty_cache()
@@ -808,6 +845,9 @@ def main():
         fused = bench_fused_swiglu(torch, Q, dev, args.quick)
         torch.cuda.empty_cache()
         phases = bench_prefill_phases(torch, np, Q, _lib, dev)
+        torch.cuda.empty_cache()
+        if not args.quick and not args.eager:
+            drounds = bench_decode_rounds(torch, Q, _lib, dev, c, max(args.steps, 100))
 
     # ---------------- parity of what was measured, against the oracle ----------------
     O = H.O
@@ -941,6 +981,7 @@ def main():
         "fused_swiglu": fused,
         "prefill_phases": phases,
         "decode_phases": dphases,
+        "decode_rounds": drounds,
         "llm_int8": llm,
         "cpu_baseline": cpu,
         "parity": parity,
@@ -969,6 +1010,10 @@ def main():
     if dphases:
         for k in ("first_entry_to_last_end_us", "last_end_to_next_launch_first_entry_us", "hbm_frac_within_span"):
             flat["decode_phase_" + k] = dphases[k]
+    if drounds:
+        for r_ in drounds["rows"]:
+            flat["decode_rounds_strips%d_linear_us" % r_["strips"]] = r_["linear_us"]
+            flat["decode_rounds_strips%d_read_floor_us" % r_["strips"]] = r_["read_floor_us"]
     if llm:
         flat["llm_int8_frac"] = llm["roofline"]["frac"]
     for nm, tf in (ladder or {}).items():

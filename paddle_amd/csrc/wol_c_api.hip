@@ -116,6 +116,11 @@ bool use_stream(int64_t M, int64_t K, int64_t N, int bits, bool have_ws) {
 bool use_batch(int64_t M, int64_t K, int64_t N, int bits, int group_size) {
   if (M < 2 || M > 16 || !wol::linear_batch_supports(M, K, bits, group_size)) return false;
   const double per_cu = static_cast<double>(N / wol::kStripCols) / wol::linear_batch_cus();
+  // 2 to 4 rows where the streaming kernel issues all loads of a wavefront at
+  // once (K = 2048 and 4096, 2 to 7 strips per CU): it is 3 to 20 % faster
+  // than this kernel except on int4 at K >= 4096 from 5 strips per CU on
+  // (4 to 9 % slower there)
+  if (M <= 4 && wol::linear_stream_loads_at_once(M, K, N, bits)) return bits == 4 && K >= 4096 && per_cu >= 5.0;
   if (M == 3 || M == 4) return per_cu >= 3.5;
   if (M == 2) return per_cu >= (bits == 4 ? 2.5 : 5.0);
   return per_cu >= 2.5;

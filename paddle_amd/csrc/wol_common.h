@@ -297,6 +297,9 @@ int launch_reduce_partials(const float* part, int nsplit, const void* bias, int 
                            bool out_f32, int64_t M, int64_t N, int act, hipStream_t stream);
 // One-line descriptions of what the launchers would run for a problem.
 void describe_linear_stream(int64_t M, int64_t K, int64_t N, int bits, int group_size, char* buf, size_t n);
+// Whether the streaming kernel runs the problem with every load of a wavefront issued at once (K divides into a
+// power of two of units per strip that a workgroup's wavefronts take whole) rather than walking its units.
+bool linear_stream_loads_at_once(int64_t M, int64_t K, int64_t N, int bits);
 void describe_linear_gemm(int64_t M, int64_t K, int64_t N, int bits, int group_size, size_t ws_bytes,
                           char* buf, size_t n);
 int launch_linear_gemm(const void* x, const void* codes, const void* bias, const void* scale,

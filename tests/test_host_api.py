@@ -280,9 +280,10 @@ def test_prefill_phases_argument_errors(lib):
 
 def test_linear_plan_names_the_kernel_per_shape(lib):
     # wol_linear's choice between its three kernels, as the library reports it
-    # (no device work): one row streams a workgroup per strip; 2 and 5..16 rows
-    # go to the batched decode kernel from two strips per CU on, 3 and 4 rows
-    # from five on, and only for the K it is built for; above 64 rows the GEMM
+    # (no device work): one row streams a workgroup per strip; 5..16 rows go to
+    # the batched decode kernel from 2.5 strips per CU on, 2 to 4 rows only where
+    # the streaming kernel has to walk its units or, on int4 at K >= 4096, from
+    # five strips per CU on, and only for the K it is built for; above 64 rows the GEMM
     def plan(M, K, N, bits, g):
         buf = ctypes.create_string_buffer(256)
         ws = lib.lib.wol_linear_workspace(M, K, N, bits, g)
@@ -291,8 +292,13 @@ def test_linear_plan_names_the_kernel_per_shape(lib):
 
     assert "stream_kernel" in plan(1, 4096, 11008, 4, 128)
     assert "batch_kernel" in plan(16, 4096, 11008, 4, -1)
-    assert "batch_kernel" in plan(2, 4096, 11008, 4, -1)
+    assert "stream_kernel" in plan(2, 4096, 11008, 4, -1)
+    assert "issued at once" in plan(2, 4096, 28672, 8, -1)   # whatever the number of strips
+    assert "batch_kernel" in plan(2, 4096, 28672, 4, -1)
+    assert "batch_kernel" in plan(2, 8192, 11008, 4, -1)     # 32 units of two rows per strip: the streaming kernel would walk
     assert "stream_kernel" in plan(4, 4096, 11008, 4, -1)
+    assert "stream_kernel" in plan(4, 4096, 16384, 8, -1)
+    assert "issued at once" in plan(1, 8192, 28672, 4, 128)
     assert "batch_kernel" in plan(4, 8192, 28672, 4, 128)
     assert "batch_kernel" in plan(8, 4096, 12288, 8, 64)
     assert "stream_kernel" in plan(8, 4096, 4096, 8, 64)    # one strip per CU

@@ -238,9 +238,9 @@ def test_swiglu_in_the_batched_kernel(device, oracle, dt, bits, g):
     from paddle_amd import _lib
     from paddle_amd.nn import quant as Q
 
-    shapes = [(2, 2048, 28704), (7, 4096, 10272), (16, 4096, 28704)]
+    shapes = [(5, 2048, 28704), (7, 4096, 10272), (16, 4096, 28704)]
     if bits == 4 and g != 64:
-        shapes.append((9, 8192, 12320))
+        shapes += [(9, 8192, 12320), (2, 8192, 12320)]
     for M, K, N in shapes:
         lws = _lib.lib.wol_linear_workspace(M, K, N, bits, g)
         plan = ctypes.create_string_buffer(256)
