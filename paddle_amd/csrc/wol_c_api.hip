@@ -121,6 +121,8 @@ bool use_batch(int64_t M, int64_t K, int64_t N, int bits, int group_size) {
   // than this kernel except on int4 at K >= 4096 from 5 strips per CU on
   // (4 to 9 % slower there)
   if (M <= 4 && wol::linear_stream_loads_at_once(M, K, N, bits)) return bits == 4 && K >= 4096 && per_cu >= 5.0;
+  // the same for 5 to 8 rows on int8 (K = 2048: 3 to 12 % at every width; K = 4096: 1 to 11 % below 5 strips per CU)
+  if (M <= 8 && bits == 8 && wol::linear_stream_loads_at_once(M, K, N, bits)) return K >= 4096 && per_cu >= 5.0;
   if (M == 3 || M == 4) return per_cu >= 3.5;
   if (M == 2) return per_cu >= (bits == 4 ? 2.5 : 5.0);
   return per_cu >= 2.5;

@@ -677,6 +677,7 @@ void launch_wk(const Args& a, int wk, int nu) {
   if constexpr ((MP == 4 || MP == 8) && MT == 1) {
     // several units per wavefront, still all in flight at once (8 wavefronts)
     if (nu == 2) { launch_one<DT, BITS, MP, MT, 8, 2>(a); return; }
+    if (nu == 4 && wk >= 16) { launch_one<DT, BITS, MP, MT, 16, 4>(a); return; }
     if (nu == 4) { launch_one<DT, BITS, MP, MT, 8, 4>(a); return; }
   }
   if (nu == 1) {
@@ -776,7 +777,8 @@ void launch_linear_stream_f16(const StreamArgs& a, int bits, bool swi, int wk, i
 // resident at once (~6 per SIMD on 1024 SIMDs).  With 3 to 8 rows and 16 or 32
 // units per strip eight wavefronts take two or four units each, all loads
 // again issued at once, at any number of strips (7 to 17 % faster than the
-// walk from 1 024 strips on).  Otherwise wavefronts walk their units with up
+// walk from 1 024 strips on; with 64 units sixteen wavefronts take four each,
+// up to 1 536 strips).  Otherwise wavefronts walk their units with up
 // to three more in flight, and WK follows a budget of resident wavefronts that
 // shrinks with the row count.
 static void pick_split(int64_t M, int64_t K, int64_t N, int bits, int* wk, int* nu, int* tn) {
@@ -799,6 +801,14 @@ static void pick_split(int64_t M, int64_t K, int64_t N, int bits, int* wk, int* 
   if (mp >= 4 && mp <= 8 && nunits * ku == nsteps && (nunits == 16 || nunits == 32)) {
     *wk = 8;
     *nu = static_cast<int>(nunits / 8);
+    return;
+  }
+  // 64 units per strip (K = 8192, and K = 4096 on int8 at 5 to 8 rows): sixteen
+  // wavefronts with four units each, 5 to 11 % faster than the walk up to
+  // 1 376 strips; at 1 792 the walk is faster
+  if (mp >= 4 && mp <= 8 && nunits * ku == nsteps && nunits == 64 && strips <= 1536) {
+    *wk = 16;
+    *nu = 4;
     return;
   }
   // measured: one or two rows want up to ~8 wavefronts per SIMD, full 16-row
@@ -857,6 +867,7 @@ int launch_linear_stream(const void* x, const void* codes, const void* bias, con
     const int walk_max = (mp >= 2 && mp <= 8) || (mp == 1 && bits == 4) ? 16 : 8;
     int total = 2 * wk;
     if (nu == 1 && total > 16) nu = 0;
+    if (nu == 4 && wk == 16) nu = 0;  // 64 units per strip: twice sixteen wavefronts
     if (nu == 2 || nu == 4) total = 16;
     if (nu == 0 && total > walk_max) total = walk_max;
     if (dtype == WOL_DTYPE_BF16) {

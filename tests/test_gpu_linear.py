@@ -878,7 +878,7 @@ def test_call_log_names_the_kernel(device):
         "from paddle_amd.nn import quant as Q\n"
         "w = (torch.randn(2048, 12288, device='cuda') * 0.02).to(torch.bfloat16)\n"
         "c, s = Q.weight_quantize(w, algo='weight_only_int8')\n"
-        "for M in (1, 8, 300):\n"
+        "for M in (1, 12, 300):\n"
         "    Q.weight_only_linear(torch.randn(M, 2048, device='cuda').to(torch.bfloat16), c, None, s, 'int8')\n"
         "torch.cuda.synchronize()\n"
     )

@@ -300,7 +300,9 @@ def test_linear_plan_names_the_kernel_per_shape(lib):
     assert "stream_kernel" in plan(4, 4096, 16384, 8, -1)
     assert "issued at once" in plan(1, 8192, 28672, 4, 128)
     assert "batch_kernel" in plan(4, 8192, 28672, 4, 128)
-    assert "batch_kernel" in plan(8, 4096, 12288, 8, 64)
+    assert "stream_kernel" in plan(8, 4096, 12288, 8, 64)   # 64 units per strip, sixteen wavefronts with four each
+    assert "batch_kernel" in plan(8, 4096, 22016, 8, 64)    # from five strips per CU on
+    assert "batch_kernel" in plan(8, 4096, 12288, 4, 128)
     assert "stream_kernel" in plan(8, 4096, 4096, 8, 64)    # one strip per CU
     assert "stream_kernel" in plan(8, 11008, 4096, 8, 64)   # a K the batched kernel is not built for
     assert "stream_kernel" in plan(8, 8192, 28672, 8, -1)   # int8 at K = 8192 does not fit its registers
