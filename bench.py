@@ -637,6 +637,8 @@ def main():
     ap.add_argument("--no-llm-int8", action="store_true", help="skip the llm_int8_linear timing")
     ap.add_argument("--no-configs", action="store_true", help="skip the per-configuration table")
     ap.add_argument("--no-ladder", action="store_true", help="skip the wol_mfma_probe ladder")
+    ap.add_argument("--no-decode-rounds", action="store_true",
+                    help="skip the decode call over the number of strips (it launches the headline kernel on other grids)")
     ap.add_argument("--quick", action="store_true", help="shorter per-configuration runs, 8 decoder layers")
     ap.add_argument("--eager", action="store_true", help="time eager launches instead of a graph")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -846,7 +848,7 @@ def main():
         torch.cuda.empty_cache()
         phases = bench_prefill_phases(torch, np, Q, _lib, dev)
         torch.cuda.empty_cache()
-        if not args.quick and not args.eager:
+        if not args.quick and not args.eager and not args.no_decode_rounds:
             drounds = bench_decode_rounds(torch, Q, _lib, dev, c, max(args.steps, 100))
 
     # ---------------- parity of what was measured, against the oracle ----------------
