@@ -86,6 +86,28 @@ __device__ inline int block_of_workgroup(int b, int nblocks) {
   return (b & ~31) + (r & 7) * 4 + (r >> 3);
 }
 
+// The same for the kernels whose workgroups are all resident at once (every
+// load issued at once, 257 to 1024 workgroups on 256 CUs): there workgroups b, b + 256, b + 512, b + 768 run on one CU (read back
+// from HW_REG_HW_ID: always so), and giving them neighbouring strips lets the
+// CU's L1 fetch a line of scales once for all of them as well -- the gathers
+// of the later workgroups meet the first one's outstanding miss.  CU slot
+// c = b % 256 sits on XCD c % 8; slots are numbered XCD by XCD so that the
+// strips of neighbouring slots still meet in one L2, and the slots the last,
+// partial round reaches (c < nblocks % 256) own one strip more.  Written
+// without a branch: both numberings are a few scalar instructions, and a
+// branch here cost the launches that keep the other numbering 1 %.
+__device__ inline int block_of_resident_workgroup(int b, int nblocks) {
+  const int r5 = b & 31;
+  const int by_xcd = b >= (nblocks & ~31) ? b : (b & ~31) + (r5 & 7) * 4 + (r5 >> 3);
+  const int q = nblocks >> 8, rem = nblocks & 255;
+  const int c = b & 255, r = b >> 8;
+  const int x = c & 7, i = c >> 3;
+  const int a = rem >> 3, t = rem & 7;
+  const int more = a + (x < t ? 1 : 0);  // slots of this XCD with one strip more
+  const int by_cu = (x * 32 + i) * q + a * x + (x < t ? x : t) + (i < more ? i : more) + r;
+  return nblocks > 256 && nblocks <= 1024 ? by_cu : by_xcd;
+}
+
 // NU > 0: every wavefront owns exactly NU units and issues all their loads at
 // once (the whole problem is in flight from the first cycle; used when K is
 // small enough).  NU == 0: a wavefront walks its share of the units with the
@@ -348,7 +370,8 @@ struct StreamKernel {
     j = lane & 15;
     kb = lane >> 4;
     const int nstrips = N / kStripCols;
-    const int bid = block_of_workgroup(static_cast<int>(blockIdx.x), static_cast<int>(gridDim.x));
+    const int bid = NU > 0 ? block_of_resident_workgroup(static_cast<int>(blockIdx.x), static_cast<int>(gridDim.x))
+                           : block_of_workgroup(static_cast<int>(blockIdx.x), static_cast<int>(gridDim.x));
     const uint8_t* strip[TN];
 #pragma unroll
     for (int t = 0; t < TN; ++t) {
