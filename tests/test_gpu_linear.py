@@ -663,6 +663,45 @@ def test_config_5_full_size_properties(device, shape):
     _full_size_properties(H.BF16, 8, 64, *shape)
 
 
+@pytest.mark.parametrize("bits,g", [(4, 128), (8, -1), (4, 64)])
+def test_strip_numbering_around_whole_rounds_of_workgroups(device, oracle, bits, g):
+    # The streaming kernel hands its strips to workgroups in an order that
+    # follows the CUs (257 to 1024 workgroups) or the XCDs (otherwise): strip
+    # counts on both sides of every switch and of whole rounds of 256, at row
+    # counts that take every all-at-once split.  Device-made weights, the oracle
+    # on the strips where a wrong numbering would show (first, last, around the
+    # multiples of 256 and of 32) and on a few others.
+    import torch
+    import gpu_calls as G
+    from paddle_amd.nn import quant as Q
+
+    dt, K = H.BF16, 2048
+    rng = np.random.default_rng(bits * 100 + (g if g > 0 else 0))
+    for strips in (255, 256, 257, 300, 511, 512, 513, 688, 1023, 1024, 1025, 1100):
+        N = strips * 16
+        gen = torch.Generator(device="cuda").manual_seed(strips)
+        w = (torch.randn(K, N, device="cuda", generator=gen) * 0.02).to(H.torch_dtype(dt))
+        codes, scale = Q.weight_quantize(w, algo="weight_only_int8" if bits == 8 else "weight_only_int4", group_size=g)
+        picks = sorted(set([0, 1, 2, 3, 31, 32, 33, 255, 256, 257, 258, 511, 512, 513, 767, 768, 769, strips - 34, strips - 33,
+                            strips - 2, strips - 1] + [int(v) for v in rng.integers(0, strips, 8)]))
+        picks = [s_ for s_ in picks if 0 <= s_ < strips]
+        cols = np.concatenate([np.arange(s_ * 16, s_ * 16 + 16) for s_ in picks])
+        oc, osc = oracle.weight_quantize(H.torch_to_bits(w[:, cols].contiguous()), dt, bits, g)
+        assert np.array_equal(osc, H.torch_to_bits(scale[..., cols].contiguous()))
+        for M in (1, 2, 5):
+            xb = H.make_act(M, K, dt, seed=strips + M)
+            bb = H.make_bias(N, dt, seed=strips)
+            out = G.linear_dev(H.bits_to_torch(xb, dt, "cuda:0"), codes, H.bits_to_torch(bb, dt, "cuda:0"), scale, dt, N,
+                               bits, g, kernel=KERNEL_STREAM)
+            got = H.torch_to_bits(out)
+            # every strip is written: none keeps the NaN the output was filled with (a strip computed
+            # in another's place fails the slices below)
+            assert np.isfinite(H.bits_to_f32(got, dt)).all()
+            _, wantT = oracle.linear(xb, oc, osc, bb[cols], dt, bits, g)
+            err = H.rel_l2(H.bits_to_f32(got[:, cols], dt), H.bits_to_f32(wantT, dt))
+            assert err <= 1e-3, (err, strips, M, bits, g)
+
+
 def test_empty_batch_and_leading_dims(device):
     import torch
 
